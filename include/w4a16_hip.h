@@ -1,0 +1,159 @@
+/*
+ * w4a16_hip.h — C ABI of the MI355X (gfx950) W4A16 linear-op library, libw4a16hip.so.
+ *
+ * The library replaces, for the W4A16 linear path only, the reference's CUDA driver layer and the operators built
+ * on it.  Each entry point names the reference interface it stands in for (paths relative to the reference
+ * checkout).  Plain C types only: a Rust `extern "C"` block, cgo or ctypes can bind this file 1:1.
+ *
+ * Conventions
+ *   - Every function returning int returns 0 on success.  Non-zero is either a hipError_t value or one of the
+ *     W4A16_ERR_* codes below; w4a16_last_error() then returns a NUL-terminated message (thread-local, valid until
+ *     the next failing call on the same thread).  The reference returns Result<_, String> with text
+ *     "rawcuda: <api>: <err>" (crates/backend-gpu/src/rawcuda/ctx/mod.rs:294-309); messages here read
+ *     "w4a16hip: <api>: <err>".
+ *   - Device pointers are uint64_t, as CUdeviceptr is in the reference (ffi.rs).  The context owns device memory it
+ *     allocated and frees what is left at destroy (ctx/mem.rs:4-44); the caller owns host buffers.
+ *   - A context is used by one thread at a time (the reference context is Send, not Sync: w4a16_dec/mod.rs:626).
+ *   - Operands: x  u16 [t][k] f16;  q  u32 [n][k/8], element i of a row = nibble (q[i>>3] >> 4*(i&7)) & 0xF,
+ *     weight = nibble - 8;  s  u16 [n][k/group] f16 (or bf16);  y [t][n] f32 or f16
+ *     (crates/core/src/quant/lane.rs:62-63).
+ */
+#ifndef W4A16_HIP_H
+#define W4A16_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct w4a16_ctx w4a16_ctx;
+typedef struct w4a16_event w4a16_event;
+
+enum {
+    W4A16_OK = 0,
+    W4A16_ERR_SHAPE = 10001,       /* shape contract violated (gptq4.rs:31-58, upload.rs:26-32)            */
+    W4A16_ERR_SYMBOL = 10002,      /* kernel symbol not loaded (ctx/mod.rs:262-267)                         */
+    W4A16_ERR_UNSUPPORTED = 10003, /* group / scale dtype combination has no kernel (gptq4.rs:60-70)        */
+    W4A16_ERR_NOT_FOUND = 10004,   /* linear name not registered (w4a16_dec/kernels/gemv.rs:10-13)          */
+    W4A16_ERR_ARG = 10005,         /* null pointer, zero size, bad enum                                     */
+    W4A16_ERR_ASSET = 10006        /* code object file missing or unreadable (assets.rs:336-346)            */
+};
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* w4a16_last_error(void);
+
+/* ------------------------------------------------------------------------------------------------------------
+ * Driver layer — stands in for CudaCtx over the dlopen'ed libcuda table
+ * (crates/backend-gpu/src/rawcuda/ffi.rs:237-292, ctx/mod.rs:62-77, 100-419, ctx/mem.rs, ctx/prof.rs).
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* CudaCtx::new_dev (ctx/mod.rs:100-152): initialise HIP, select the device, create the launch stream and a second
+ * stream (both non-blocking, default priority), and load every code object of the built-in manifest from
+ * `asset_dir` (NULL = the directory "assets" beside the shared library; a single asset can be redirected with the
+ * environment variable LLM170_HIP_<NAME>_HSACO_PATH, as LLM170_CUDA_<NAME>_FATBIN_PATH does in assets.rs:336-339). */
+int w4a16_ctx_create(int device_ordinal, const char* asset_dir, w4a16_ctx** out);
+/* Drop of CudaCtx: frees every tracked allocation (ctx/mem.rs:32-44), modules, streams. */
+void w4a16_ctx_destroy(w4a16_ctx* ctx);
+
+/* CudaCtx::load_fatbin (ctx/mod.rs:196-228): hipModuleLoadData on a gfx950 code object image, then resolve every
+ * listed symbol eagerly; a missing symbol fails the load and names it. */
+int w4a16_module_load(w4a16_ctx* ctx, const char* key, const void* image, size_t len, const char* const* symbols,
+                      size_t nsym);
+/* CudaCtx::function (ctx/mod.rs:262-267): 0 if `symbol` is resolved, W4A16_ERR_SYMBOL otherwise. */
+int w4a16_has_symbol(w4a16_ctx* ctx, const char* symbol);
+/* CudaCtx::launch / launch_shared (ctx/mod.rs:270-363): hipModuleLaunchKernel(f, gx,gy,1, block,1,1, shmem,
+ * launch stream, params, NULL); params is an array of pointers to the argument values (args.rs:4-31). */
+int w4a16_launch(w4a16_ctx* ctx, const char* symbol, unsigned gx, unsigned gy, unsigned block, unsigned shmem,
+                 void** params);
+
+/* CudaCtx::alloc / free / h2d / d2h / d2d / memset (ctx/mem.rs:4-44, 164-336).  Copies and the fill are ordered on
+ * the launch stream; h2d and d2h return after the data has moved. */
+int w4a16_alloc(w4a16_ctx* ctx, size_t bytes, uint64_t* dptr);
+int w4a16_free(w4a16_ctx* ctx, uint64_t dptr);
+int w4a16_h2d(w4a16_ctx* ctx, uint64_t dst, const void* src, size_t bytes);
+int w4a16_d2h(w4a16_ctx* ctx, void* dst, uint64_t src, size_t bytes);
+int w4a16_d2d(w4a16_ctx* ctx, uint64_t dst, uint64_t src, size_t bytes);
+int w4a16_memset0(w4a16_ctx* ctx, uint64_t dst, size_t bytes);
+/* CudaCtx::sync (ctx/mod.rs:407-412): wait for the launch stream. */
+int w4a16_sync(w4a16_ctx* ctx);
+/* Bytes currently allocated through this context (CudaCtx::allocs bookkeeping, ctx/mem.rs:4-30). */
+size_t w4a16_allocated_bytes(w4a16_ctx* ctx);
+
+/* Event timing on the launch stream (ctx/prof.rs:4-54: event create / record / elapsed). */
+int w4a16_event_create(w4a16_ctx* ctx, w4a16_event** out);
+int w4a16_event_record(w4a16_ctx* ctx, w4a16_event* ev);
+int w4a16_event_elapsed_ms(w4a16_ctx* ctx, w4a16_event* start, w4a16_event* stop, float* ms); /* waits for stop */
+void w4a16_event_destroy(w4a16_ctx* ctx, w4a16_event* ev);
+
+/* Names in the built-in asset manifest (assets.rs:276-334): returns the number of assets; when `asset` is in range
+ * stores its name and NULL-terminated symbol list. */
+size_t w4a16_manifest(size_t asset, const char** name, const char* const** symbols);
+
+/* ------------------------------------------------------------------------------------------------------------
+ * Operator layer
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* check_shapes (gptq4.rs:31-58): group in {128,32}, k % group == 0, t >= 1, qlen == n*(k/8) words,
+ * slen == n*(k/group) halves, xlen == t*k halves.  (The reference's extra t==1 limit k <= 256*group exists only
+ * for its shared-memory scale cache; the kernels here have no such limit and the rule is not carried over.) */
+int w4a16_check_shapes(size_t t, size_t qlen, size_t slen, size_t xlen, size_t n, size_t k, size_t group);
+
+/* kernel_sym (gptq4.rs:60-70): name of the bit-exact kernel serving (group, scale dtype); NULL + W4A16_ERR_UNSUPPORTED
+ * for other combinations.  Served here: (128,f16) (32,bf16) as in the reference, plus (32,f16) and (128,bf16). */
+const char* w4a16_kernel_sym(int group, int scale_bf16);
+
+/* Gptq4::gemm / Gptq4::gemv (gptq4.rs:85-190): upload x, q, s; run the kernel that reproduces
+ * dot_row_w4a16_lane_group bit for bit (64 strided f32 lanes, un-fused multiply and add, f64 tree;
+ * crates/core/src/quant/lane.rs:2-70); download out f32 [t][n]; free.  A test operator, not the fast path. */
+int w4a16_gemm_host(w4a16_ctx* ctx, const uint16_t* x_f16, size_t t, const uint32_t* q, const uint16_t* s, size_t n,
+                    size_t k, size_t group, int scale_bf16, float* out_f32);
+
+/* W4a16Dec::upload_lin_g (w4a16_dec/upload.rs:15-65): register a linear by name.  q: n*k/2 bytes, s: n*(k/group)*2
+ * bytes in the operand format above; lengths are enforced.  Keeps the operands resident as given and, when
+ * n % 16 == 0 and k % 128 == 0, also in the tiled layout the streaming and MFMA kernels read (the reference likewise
+ * keeps a repacked copy next to the original, upload.rs:99-179).  Re-registering a name frees the old buffers. */
+int w4a16_upload_lin(w4a16_ctx* ctx, const char* name, const void* q, size_t qlen_bytes, const void* s,
+                     size_t slen_bytes, size_t n, size_t k, size_t group, int scale_bf16);
+/* consolidate_marlin_dense (upload.rs:67-97): free the as-given copy of one linear once the tiled one exists
+ * (bit-exact path and raw dump then report W4A16_ERR_NOT_FOUND for it). */
+int w4a16_lin_drop_raw(w4a16_ctx* ctx, const char* name);
+/* lin_spec (w4a16_dec/mod.rs:1193-1206): shape of a registered linear. */
+int w4a16_lin_info(w4a16_ctx* ctx, const char* name, size_t* n, size_t* k, size_t* group, int* scale_bf16,
+                   int* has_tiled, int* has_raw);
+
+/* LinPath (w4a16_dec/mod.rs:79-84) */
+enum {
+    W4A16_PATH_AUTO = 0,   /* t <= 16 -> DECODE, else PREFILL; LANE when the linear has no tiled copy            */
+    W4A16_PATH_LANE = 1,   /* bit-exact twin of lane.rs (reference: w4a16_gemm_g128, gptq4.cu:825-951)            */
+    W4A16_PATH_DECODE = 2, /* HBM-streaming skinny GEMM, t <= 16 (reference: gemv_t_launch / sk_*_dev)            */
+    W4A16_PATH_PREFILL = 3 /* LDS-staged MFMA GEMM, any t (reference: gemm_launch -> marlin_gemm_try)             */
+};
+
+/* lin_forward (w4a16_dec/kernels/mod.rs:121-144): y[t][n] = x[t][k] * W^T on the launch stream, no host sync.
+ * x_dev: f16 [t][k].  y_dev: f32 [t][n] if out_f16 == 0 else f16 [t][n] (f32 accumulation, one rounding). */
+int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16,
+                      int path);
+
+/* gemv_host (w4a16_dec/mod.rs, host-operand convenience used by probes): lin_forward with host x / y. */
+int w4a16_lin_forward_host(w4a16_ctx* ctx, const char* name, const uint16_t* x_f16, void* y, size_t t, int out_f16,
+                           int path);
+
+/* Dequantised weights of a registered linear as f32 [n][k] = (nibble - 8) * scale
+ * (dequant_row_w4a16_split, crates/core/src/matmul/cpu.rs:167-194).  from_tiled != 0 reads the tiled copy (so the
+ * re-layout is covered), else the as-given copy. */
+int w4a16_dequant_dump(w4a16_ctx* ctx, const char* name, int from_tiled, uint64_t out_f32_dev);
+/* Inverse of the upload re-layout: writes q u32 [n][k/8] and s u16 [n][k/group] in the operand format from the
+ * tiled copy (round-trip check, as repack_roundtrip / scale_perm_roundtrip in crates/core/src/marlin.rs:106-132). */
+int w4a16_lin_untile(w4a16_ctx* ctx, const char* name, uint64_t q_out_dev, uint64_t s_out_dev);
+
+/* Launch-shape override for the decode kernel (0 = choose automatically): rows_per_wave in {16,32,64},
+ * waves_per_block in 1..16.  For tuning sweeps (the reference exposes its split-K factor the same way,
+ * sk_ksp, w4a16_dec/kernels/decode.rs:3-16). */
+int w4a16_set_decode_shape(w4a16_ctx* ctx, int rows_per_wave, int waves_per_block);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* W4A16_HIP_H */

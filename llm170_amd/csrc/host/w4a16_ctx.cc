@@ -1,0 +1,305 @@
+// Driver layer of libw4a16hip.so: context, code-object loading, launches, memory, events.
+// Stands in for CudaCtx over the dlopen'ed CUDA driver table in the reference
+// (crates/backend-gpu/src/rawcuda/ffi.rs:237-459, ctx/mod.rs:62-419, ctx/mem.rs, ctx/prof.rs, assets.rs).
+#include <dlfcn.h>
+
+#include <cctype>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "w4a16_internal.h"
+
+// ------------------------------------------------------------------------------------------------ errors
+static thread_local char g_err[512] = "";
+
+extern "C" const char* w4a16_last_error(void) { return g_err; }
+
+int w4_fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    int off = snprintf(g_err, sizeof g_err, "w4a16hip: ");
+    vsnprintf(g_err + off, sizeof g_err - (size_t)off, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+std::string w4_err_save() { return std::string(g_err); }
+
+void w4_err_restore(const std::string& msg) {
+    strncpy(g_err, msg.c_str(), sizeof g_err - 1);
+    g_err[sizeof g_err - 1] = 0;
+}
+
+int w4_hip(hipError_t e, const char* api) {
+    if (e == hipSuccess) return 0;
+    return w4_fail((int)e, "%s: %s (%d)", api, hipGetErrorString(e), (int)e);
+}
+
+// ------------------------------------------------------------------------------------------------ manifest
+// Asset registry: code object name -> kernel symbols.  Counterpart of assets.rs:276-334 / FATBINS.manifest; a test
+// checks that these lists equal the extern "C" __global__ symbols of the kernel sources (assets.rs:394-443).
+static const char* const kLaneSyms[] = {"w4a16_lane_g128_f16", "w4a16_lane_g128_bf16", "w4a16_lane_g32_f16",
+                                        "w4a16_lane_g32_bf16", nullptr};
+static const char* const kLayoutSyms[] = {"w4a16_tile_q",         "w4a16_tile_s",          "w4a16_untile_q",
+                                          "w4a16_untile_s",       "w4a16_dump_tiled_f16",  "w4a16_dump_tiled_bf16",
+                                          "w4a16_dump_raw_f16",   "w4a16_dump_raw_bf16",   nullptr};
+static const char* const kDecodeSyms[] = {
+    "w4a16_decode_g128_f16_rb1",  "w4a16_decode_g128_f16_rb2",  "w4a16_decode_g128_f16_rb4",
+    "w4a16_decode_g32_f16_rb1",   "w4a16_decode_g32_f16_rb2",   "w4a16_decode_g32_f16_rb4",
+    "w4a16_decode_g128_bf16_rb1", "w4a16_decode_g128_bf16_rb2", "w4a16_decode_g128_bf16_rb4",
+    "w4a16_decode_g32_bf16_rb1",  "w4a16_decode_g32_bf16_rb2",  "w4a16_decode_g32_bf16_rb4",
+    nullptr};
+
+struct W4Asset {
+    const char* name;
+    const char* const* syms;
+};
+static const W4Asset kAssets[] = {
+    {"lane", kLaneSyms},
+    {"layout", kLayoutSyms},
+    {"decode", kDecodeSyms},
+};
+static const size_t kAssetCount = sizeof kAssets / sizeof kAssets[0];
+
+extern "C" size_t w4a16_manifest(size_t asset, const char** name, const char* const** symbols) {
+    if (asset < kAssetCount) {
+        if (name) *name = kAssets[asset].name;
+        if (symbols) *symbols = kAssets[asset].syms;
+    }
+    return kAssetCount;
+}
+
+static std::string default_asset_dir() {
+    Dl_info info;
+    if (dladdr((void*)&w4a16_last_error, &info) && info.dli_fname) {
+        std::string p(info.dli_fname);
+        size_t slash = p.rfind('/');
+        return (slash == std::string::npos ? std::string(".") : p.substr(0, slash)) + "/assets";
+    }
+    return "assets";
+}
+
+static int read_file(const std::string& path, std::vector<char>* out) {
+    FILE* f = fopen(path.c_str(), "rb");
+    if (!f) return w4_fail(W4A16_ERR_ASSET, "asset: cannot open %s (build the gfx950 code objects first)", path.c_str());
+    fseek(f, 0, SEEK_END);
+    long sz = ftell(f);
+    fseek(f, 0, SEEK_SET);
+    out->resize(sz > 0 ? (size_t)sz : 0);
+    size_t got = sz > 0 ? fread(out->data(), 1, (size_t)sz, f) : 0;
+    fclose(f);
+    if (sz <= 0 || got != (size_t)sz) return w4_fail(W4A16_ERR_ASSET, "asset: short read on %s", path.c_str());
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------ context
+extern "C" int w4a16_module_load(w4a16_ctx* ctx, const char* key, const void* image, size_t len,
+                                 const char* const* symbols, size_t nsym) {
+    if (!ctx || !key || !image || len == 0) return w4_fail(W4A16_ERR_ARG, "module_load: null argument");
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    hipModule_t mod = nullptr;
+    hipError_t e = hipModuleLoadData(&mod, image);
+    if (e != hipSuccess) {
+        // the reference's hint on load failure is an architecture mismatch (ctx/mod.rs:207-210)
+        return w4_fail((int)e, "hipModuleLoadData(%s): %s (%d) — the code object must be built for gfx950", key,
+                       hipGetErrorString(e), (int)e);
+    }
+    std::vector<std::pair<std::string, hipFunction_t>> found;
+    for (size_t i = 0; i < nsym; i++) {
+        hipFunction_t f = nullptr;
+        e = hipModuleGetFunction(&f, mod, symbols[i]);
+        if (e != hipSuccess || !f) {
+            hipModuleUnload(mod);
+            return w4_fail(W4A16_ERR_SYMBOL, "module_load(%s): symbol %s not in the code object (%s)", key, symbols[i],
+                           hipGetErrorString(e));
+        }
+        found.emplace_back(symbols[i], f);
+    }
+    ctx->modules.push_back(mod);
+    for (auto& p : found) ctx->functions[p.first] = p.second;
+    return 0;
+}
+
+extern "C" int w4a16_ctx_create(int device_ordinal, const char* asset_dir, w4a16_ctx** out) {
+    if (!out) return w4_fail(W4A16_ERR_ARG, "ctx_create: out is null");
+    *out = nullptr;
+    W4_TRY(w4_hip(hipInit(0), "hipInit"));
+    int count = 0;
+    W4_TRY(w4_hip(hipGetDeviceCount(&count), "hipGetDeviceCount"));
+    if (device_ordinal < 0 || device_ordinal >= count)
+        return w4_fail(W4A16_ERR_ARG, "ctx_create: device %d of %d", device_ordinal, count);
+    W4_TRY(w4_hip(hipSetDevice(device_ordinal), "hipSetDevice"));
+    w4a16_ctx* ctx = new w4a16_ctx();
+    ctx->device = device_ordinal;
+    hipDeviceProp_t prop;
+    int rc = w4_hip(hipGetDeviceProperties(&prop, device_ordinal), "hipGetDeviceProperties");
+    if (!rc && strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        rc = w4_fail(W4A16_ERR_UNSUPPORTED, "ctx_create: device is %s; the kernels are built for gfx950 only",
+                     prop.gcnArchName);
+    if (!rc) ctx->cu_count = prop.multiProcessorCount;
+    // both streams non-blocking, default priority (reference: flag 1 = CU_STREAM_NON_BLOCKING, ctx/mod.rs:366-396)
+    if (!rc) rc = w4_hip(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+    if (!rc) rc = w4_hip(hipStreamCreateWithFlags(&ctx->stream2, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+    std::string dir = asset_dir ? std::string(asset_dir) : default_asset_dir();
+    for (size_t a = 0; a < kAssetCount && !rc; a++) {
+        std::string env = "LLM170_HIP_";
+        for (const char* c = kAssets[a].name; *c; c++) env.push_back((char)toupper((unsigned char)*c));
+        env += "_HSACO_PATH";
+        const char* over = getenv(env.c_str());
+        std::string path = over && *over ? std::string(over) : dir + "/" + kAssets[a].name + ".hsaco";
+        std::vector<char> image;
+        rc = read_file(path, &image);
+        if (rc) break;
+        size_t nsym = 0;
+        while (kAssets[a].syms[nsym]) nsym++;
+        rc = w4a16_module_load(ctx, kAssets[a].name, image.data(), image.size(), kAssets[a].syms, nsym);
+    }
+    if (rc) {
+        const std::string keep = w4_err_save();
+        w4a16_ctx_destroy(ctx);
+        w4_err_restore(keep);
+        return rc;
+    }
+    *out = ctx;
+    return 0;
+}
+
+extern "C" void w4a16_ctx_destroy(w4a16_ctx* ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->stream2) (void)hipStreamSynchronize(ctx->stream2);
+    for (auto& a : ctx->allocs) (void)hipFree((void*)a.first);
+    for (auto m : ctx->modules) (void)hipModuleUnload(m);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    if (ctx->stream2) (void)hipStreamDestroy(ctx->stream2);
+    delete ctx;
+}
+
+extern "C" int w4a16_has_symbol(w4a16_ctx* ctx, const char* symbol) {
+    if (!ctx || !symbol) return w4_fail(W4A16_ERR_ARG, "has_symbol: null argument");
+    if (ctx->functions.find(symbol) == ctx->functions.end())
+        return w4_fail(W4A16_ERR_SYMBOL, "function: symbol %s is not loaded", symbol);
+    return 0;
+}
+
+int w4_launch(w4a16_ctx* ctx, const char* symbol, unsigned gx, unsigned gy, unsigned block, unsigned shmem,
+              void** params) {
+    auto it = ctx->functions.find(symbol);
+    if (it == ctx->functions.end()) return w4_fail(W4A16_ERR_SYMBOL, "function: symbol %s is not loaded", symbol);
+    if (gx == 0 || gy == 0 || block == 0 || block > 1024)
+        return w4_fail(W4A16_ERR_ARG, "launch %s: grid %ux%u block %u", symbol, gx, gy, block);
+    hipError_t e = hipModuleLaunchKernel(it->second, gx, gy, 1, block, 1, 1, shmem, ctx->stream, params, nullptr);
+    if (e != hipSuccess)
+        return w4_fail((int)e, "hipModuleLaunchKernel(%s grid %ux%u block %u shmem %u): %s (%d)", symbol, gx, gy, block,
+                       shmem, hipGetErrorString(e), (int)e);
+    return 0;
+}
+
+extern "C" int w4a16_launch(w4a16_ctx* ctx, const char* symbol, unsigned gx, unsigned gy, unsigned block,
+                            unsigned shmem, void** params) {
+    if (!ctx || !symbol || !params) return w4_fail(W4A16_ERR_ARG, "launch: null argument");
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    return w4_launch(ctx, symbol, gx, gy, block, shmem, params);
+}
+
+// ------------------------------------------------------------------------------------------------ memory
+extern "C" int w4a16_alloc(w4a16_ctx* ctx, size_t bytes, uint64_t* dptr) {
+    if (!ctx || !dptr) return w4_fail(W4A16_ERR_ARG, "alloc: null argument");
+    *dptr = 0;
+    if (bytes == 0) return w4_fail(W4A16_ERR_ARG, "alloc: zero bytes");
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) return w4_fail((int)e, "hipMalloc(%zu): %s (%d)", bytes, hipGetErrorString(e), (int)e);
+    ctx->allocs[(uint64_t)p] = bytes;
+    ctx->allocated += bytes;
+    *dptr = (uint64_t)p;
+    return 0;
+}
+
+extern "C" int w4a16_free(w4a16_ctx* ctx, uint64_t dptr) {
+    if (!ctx) return w4_fail(W4A16_ERR_ARG, "free: null context");
+    if (dptr == 0) return 0;
+    auto it = ctx->allocs.find(dptr);
+    if (it == ctx->allocs.end()) return w4_fail(W4A16_ERR_ARG, "free: %#llx was not allocated by this context",
+                                                (unsigned long long)dptr);
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    // work queued on the launch stream may still use the buffer
+    W4_TRY(w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"));
+    ctx->allocated -= it->second;
+    ctx->allocs.erase(it);
+    return w4_hip(hipFree((void*)dptr), "hipFree");
+}
+
+extern "C" size_t w4a16_allocated_bytes(w4a16_ctx* ctx) { return ctx ? ctx->allocated : 0; }
+
+extern "C" int w4a16_h2d(w4a16_ctx* ctx, uint64_t dst, const void* src, size_t bytes) {
+    if (!ctx || !dst || !src) return w4_fail(W4A16_ERR_ARG, "h2d: null argument");
+    if (bytes == 0) return 0;
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    W4_TRY(w4_hip(hipMemcpyAsync((void*)dst, src, bytes, hipMemcpyHostToDevice, ctx->stream), "hipMemcpyAsync(h2d)"));
+    return w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+extern "C" int w4a16_d2h(w4a16_ctx* ctx, void* dst, uint64_t src, size_t bytes) {
+    if (!ctx || !dst || !src) return w4_fail(W4A16_ERR_ARG, "d2h: null argument");
+    if (bytes == 0) return 0;
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    W4_TRY(w4_hip(hipMemcpyAsync(dst, (const void*)src, bytes, hipMemcpyDeviceToHost, ctx->stream), "hipMemcpyAsync(d2h)"));
+    return w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+extern "C" int w4a16_d2d(w4a16_ctx* ctx, uint64_t dst, uint64_t src, size_t bytes) {
+    if (!ctx || !dst || !src) return w4_fail(W4A16_ERR_ARG, "d2d: null argument");
+    if (bytes == 0) return 0;
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    return w4_hip(hipMemcpyAsync((void*)dst, (const void*)src, bytes, hipMemcpyDeviceToDevice, ctx->stream),
+                  "hipMemcpyAsync(d2d)");
+}
+
+extern "C" int w4a16_memset0(w4a16_ctx* ctx, uint64_t dst, size_t bytes) {
+    if (!ctx || !dst) return w4_fail(W4A16_ERR_ARG, "memset0: null argument");
+    if (bytes == 0) return 0;
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    return w4_hip(hipMemsetAsync((void*)dst, 0, bytes, ctx->stream), "hipMemsetAsync");
+}
+
+extern "C" int w4a16_sync(w4a16_ctx* ctx) {
+    if (!ctx) return w4_fail(W4A16_ERR_ARG, "sync: null context");
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    return w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+// ------------------------------------------------------------------------------------------------ events
+extern "C" int w4a16_event_create(w4a16_ctx* ctx, w4a16_event** out) {
+    if (!ctx || !out) return w4_fail(W4A16_ERR_ARG, "event_create: null argument");
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    w4a16_event* ev = new w4a16_event();
+    int rc = w4_hip(hipEventCreate(&ev->ev), "hipEventCreate");
+    if (rc) {
+        delete ev;
+        return rc;
+    }
+    *out = ev;
+    return 0;
+}
+
+extern "C" int w4a16_event_record(w4a16_ctx* ctx, w4a16_event* ev) {
+    if (!ctx || !ev) return w4_fail(W4A16_ERR_ARG, "event_record: null argument");
+    return w4_hip(hipEventRecord(ev->ev, ctx->stream), "hipEventRecord");
+}
+
+extern "C" int w4a16_event_elapsed_ms(w4a16_ctx* ctx, w4a16_event* start, w4a16_event* stop, float* ms) {
+    if (!ctx || !start || !stop || !ms) return w4_fail(W4A16_ERR_ARG, "event_elapsed_ms: null argument");
+    W4_TRY(w4_hip(hipEventSynchronize(stop->ev), "hipEventSynchronize"));
+    return w4_hip(hipEventElapsedTime(ms, start->ev, stop->ev), "hipEventElapsedTime");
+}
+
+extern "C" void w4a16_event_destroy(w4a16_ctx* ctx, w4a16_event* ev) {
+    (void)ctx;
+    if (!ev) return;
+    (void)hipEventDestroy(ev->ev);
+    delete ev;
+}

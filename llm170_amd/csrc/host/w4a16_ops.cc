@@ -1,0 +1,271 @@
+// Operator layer of libw4a16hip.so: shape contract, weight registration with re-layout, regime dispatch.
+// Stands in for Gptq4 (crates/backend-gpu/src/rawcuda/gptq4.rs) and for the W4a16Dec linear-op entry points
+// upload_lin_g / lin_forward / gemv_t_launch / gemm_launch (w4a16_dec/upload.rs:15-65, kernels/mod.rs:121-144,
+// kernels/gemv.rs:112-187, kernels/gemm.rs:4-51).
+#include <algorithm>
+#include <cstring>
+
+#include "w4a16_internal.h"
+
+static inline unsigned ceil_div(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+
+// ------------------------------------------------------------------------------------------------ contract
+extern "C" int w4a16_check_shapes(size_t t, size_t qlen, size_t slen, size_t xlen, size_t n, size_t k, size_t group) {
+    if ((group != 128 && group != 32) || k == 0 || k % group != 0 || t == 0 || n == 0 || qlen != n * (k / 8) ||
+        slen != n * (k / group) || xlen != t * k) {
+        return w4_fail(W4A16_ERR_SHAPE, "gptq4: shape contract violated q=%zu s=%zu x=%zu n=%zu k=%zu t=%zu group=%zu",
+                       qlen, slen, xlen, n, k, t, group);
+    }
+    return 0;
+}
+
+extern "C" const char* w4a16_kernel_sym(int group, int scale_bf16) {
+    if (group == 128) return scale_bf16 ? "w4a16_lane_g128_bf16" : "w4a16_lane_g128_f16";
+    if (group == 32) return scale_bf16 ? "w4a16_lane_g32_bf16" : "w4a16_lane_g32_f16";
+    w4_fail(W4A16_ERR_UNSUPPORTED, "gptq4: unsupported combination group=%d scale_bf16=%d", group, scale_bf16);
+    return nullptr;
+}
+
+// ------------------------------------------------------------------------------------------------ launches
+static int launch_lane(w4a16_ctx* ctx, uint64_t q, uint64_t s, uint64_t x, uint64_t out, size_t n, size_t k, size_t t,
+                       size_t group, int scale_bf16) {
+    const char* sym = w4a16_kernel_sym((int)group, scale_bf16);
+    if (!sym) return W4A16_ERR_UNSUPPORTED;
+    if (n > 0x7fffffffu || k > 0x7fffffffu || t > 8u * 65535u)
+        return w4_fail(W4A16_ERR_SHAPE, "lane: n=%zu k=%zu t=%zu exceed the launch limits", n, k, t);
+    int ni = (int)n, ki = (int)k, ti = (int)t;
+    void* params[] = {&q, &s, &x, &out, &ni, &ki, &ti};
+    return w4_launch(ctx, sym, ceil_div(n, 4), ceil_div(t, 8), 256, 0, params);
+}
+
+static int pick_decode_shape(const w4a16_ctx* ctx, const W4Lin& L, size_t t, int* rb_out, int* waves_out) {
+    int rb = ctx->decode_rows_per_wave ? ctx->decode_rows_per_wave / 16 : (t <= 4 ? 2 : 4);
+    if (rb != 1 && rb != 2 && rb != 4) return w4_fail(W4A16_ERR_ARG, "decode: rows_per_wave must be 16, 32 or 64");
+    while (rb > 1 && L.row_blocks < (size_t)rb) rb >>= 1;
+    const int kt_n = (int)(L.k / 128);
+    int waves = ctx->decode_waves_per_block;
+    if (waves == 0) {
+        // aim at ~8 KiB of weights per wave (measured best for a read-once stream on MI355X)
+        const int tiles_per_wave = std::max(1, 8 / rb);
+        waves = (kt_n + tiles_per_wave - 1) / tiles_per_wave;
+    }
+    waves = std::max(1, std::min(std::min(waves, 16), kt_n));
+    *rb_out = rb;
+    *waves_out = waves;
+    return 0;
+}
+
+static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16) {
+    if (t == 0 || t > 16) return w4_fail(W4A16_ERR_SHAPE, "decode: t=%zu outside 1..16", t);
+    if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode: linear has no tiled copy (needs k %% 128 == 0)");
+    int rb = 0, waves = 0;
+    W4_TRY(pick_decode_shape(ctx, L, t, &rb, &waves));
+    char sym[64];
+    snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_rb%d", L.group, L.scale_bf16 ? "bf16" : "f16", rb);
+    uint64_t qt = L.q_tiled, st = L.s_tiled;
+    int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
+    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of};
+    unsigned shmem = waves > 1 ? (unsigned)(waves * rb * 64 * 16) : 0;
+    return w4_launch(ctx, sym, ceil_div(L.row_blocks, (size_t)rb), 1, (unsigned)(waves * 64), shmem, params);
+}
+
+// ------------------------------------------------------------------------------------------------ Gptq4::gemm
+extern "C" int w4a16_gemm_host(w4a16_ctx* ctx, const uint16_t* x_f16, size_t t, const uint32_t* q, const uint16_t* s,
+                               size_t n, size_t k, size_t group, int scale_bf16, float* out_f32) {
+    if (!ctx || !x_f16 || !q || !s || !out_f32) return w4_fail(W4A16_ERR_ARG, "gemm_host: null argument");
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    if ((group != 128 && group != 32) || k == 0 || k % group != 0 || t == 0 || n == 0)
+        return w4_fail(W4A16_ERR_SHAPE, "gptq4: shape contract violated n=%zu k=%zu t=%zu group=%zu", n, k, t, group);
+    if (!w4a16_kernel_sym((int)group, scale_bf16)) return W4A16_ERR_UNSUPPORTED;
+    const size_t qb = n * (k / 8) * 4, sb = n * (k / group) * 2, xb = t * k * 2, ob = t * n * 4;
+    uint64_t dq = 0, ds = 0, dx = 0, dout = 0;
+    int rc = w4a16_alloc(ctx, qb, &dq);
+    if (!rc) rc = w4a16_alloc(ctx, sb, &ds);
+    if (!rc) rc = w4a16_alloc(ctx, xb, &dx);
+    if (!rc) rc = w4a16_alloc(ctx, ob, &dout);
+    if (!rc) rc = w4a16_h2d(ctx, dq, q, qb);
+    if (!rc) rc = w4a16_h2d(ctx, ds, s, sb);
+    if (!rc) rc = w4a16_h2d(ctx, dx, x_f16, xb);
+    if (!rc) rc = launch_lane(ctx, dq, ds, dx, dout, n, k, t, group, scale_bf16);
+    if (!rc) rc = w4a16_d2h(ctx, out_f32, dout, ob);
+    const std::string keep = w4_err_save();
+    (void)w4a16_free(ctx, dq);
+    (void)w4a16_free(ctx, ds);
+    (void)w4a16_free(ctx, dx);
+    (void)w4a16_free(ctx, dout);
+    if (rc) w4_err_restore(keep);
+    return rc;
+}
+
+// ------------------------------------------------------------------------------------------------ registration
+static void free_lin(w4a16_ctx* ctx, W4Lin& L) {
+    (void)w4a16_free(ctx, L.q_raw);
+    (void)w4a16_free(ctx, L.s_raw);
+    (void)w4a16_free(ctx, L.q_tiled);
+    (void)w4a16_free(ctx, L.s_tiled);
+    L = W4Lin();
+}
+
+extern "C" int w4a16_upload_lin(w4a16_ctx* ctx, const char* name, const void* q, size_t qlen_bytes, const void* s,
+                                size_t slen_bytes, size_t n, size_t k, size_t group, int scale_bf16) {
+    if (!ctx || !name || !q || !s) return w4_fail(W4A16_ERR_ARG, "upload_lin: null argument");
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    if (group != 128 && group != 32)
+        return w4_fail(W4A16_ERR_UNSUPPORTED, "gptq4: unsupported combination group=%zu scale_bf16=%d", group, scale_bf16);
+    if (n == 0 || k == 0 || k % group != 0 || qlen_bytes != n * (k / 2) || slen_bytes != n * (k / group) * 2)
+        return w4_fail(W4A16_ERR_SHAPE, "upload_lin_g %s: q=%zu s=%zu != n%zu k%zu g%zu contract", name, qlen_bytes,
+                       slen_bytes, n, k, group);
+    if (n > 0x7fffffffu || k > 0x7fffffffu) return w4_fail(W4A16_ERR_SHAPE, "upload_lin_g %s: n or k too large", name);
+    W4Lin L;
+    L.n = n;
+    L.k = k;
+    L.group = group;
+    L.scale_bf16 = scale_bf16 ? 1 : 0;
+    int rc = w4a16_alloc(ctx, qlen_bytes, &L.q_raw);
+    if (!rc) rc = w4a16_alloc(ctx, slen_bytes, &L.s_raw);
+    if (!rc) rc = w4a16_h2d(ctx, L.q_raw, q, qlen_bytes);
+    if (!rc) rc = w4a16_h2d(ctx, L.s_raw, s, slen_bytes);
+    if (!rc && k % 128 == 0) {
+        L.row_blocks = (n + 15) / 16;
+        const size_t kt_n = k / 128, kg_n = k / group;
+        const size_t qt_bytes = L.row_blocks * kt_n * 1024, st_bytes = L.row_blocks * kg_n * 16 * 2;
+        rc = w4a16_alloc(ctx, qt_bytes, &L.q_tiled);
+        if (!rc) rc = w4a16_alloc(ctx, st_bytes, &L.s_tiled);
+        if (!rc) {
+            int ni = (int)n, ki = (int)k, rbi = (int)L.row_blocks, kgi = (int)kg_n;
+            void* pq[] = {&L.q_raw, &L.q_tiled, &ni, &ki, &rbi};
+            rc = w4_launch(ctx, "w4a16_tile_q", ceil_div(qt_bytes / 4, 256), 1, 256, 0, pq);
+            void* ps[] = {&L.s_raw, &L.s_tiled, &ni, &kgi, &rbi};
+            if (!rc) rc = w4_launch(ctx, "w4a16_tile_s", ceil_div(st_bytes / 2, 256), 1, 256, 0, ps);
+            if (!rc) rc = w4a16_sync(ctx);
+        }
+    }
+    if (rc) {
+        const std::string keep = w4_err_save();
+        free_lin(ctx, L);
+        w4_err_restore(keep);
+        return rc;
+    }
+    auto it = ctx->lins.find(name);
+    if (it != ctx->lins.end()) free_lin(ctx, it->second);  // re-registration frees the old buffers (upload.rs:53-56)
+    ctx->lins[name] = L;
+    return 0;
+}
+
+static int find_lin(w4a16_ctx* ctx, const char* name, W4Lin** out) {
+    if (!ctx || !name) return w4_fail(W4A16_ERR_ARG, "lin: null argument");
+    auto it = ctx->lins.find(name);
+    if (it == ctx->lins.end()) return w4_fail(W4A16_ERR_NOT_FOUND, "lin %s: not registered", name);
+    *out = &it->second;
+    return 0;
+}
+
+extern "C" int w4a16_lin_drop_raw(w4a16_ctx* ctx, const char* name) {
+    W4Lin* L = nullptr;
+    W4_TRY(find_lin(ctx, name, &L));
+    if (!L->q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "lin %s: no tiled copy, the operands as given must stay", name);
+    W4_TRY(w4a16_free(ctx, L->q_raw));
+    W4_TRY(w4a16_free(ctx, L->s_raw));
+    L->q_raw = L->s_raw = 0;
+    return 0;
+}
+
+extern "C" int w4a16_lin_info(w4a16_ctx* ctx, const char* name, size_t* n, size_t* k, size_t* group, int* scale_bf16,
+                              int* has_tiled, int* has_raw) {
+    W4Lin* L = nullptr;
+    W4_TRY(find_lin(ctx, name, &L));
+    if (n) *n = L->n;
+    if (k) *k = L->k;
+    if (group) *group = L->group;
+    if (scale_bf16) *scale_bf16 = L->scale_bf16;
+    if (has_tiled) *has_tiled = L->q_tiled != 0;
+    if (has_raw) *has_raw = L->q_raw != 0;
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------ forward
+extern "C" int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16,
+                                 int path) {
+    W4Lin* L = nullptr;
+    W4_TRY(find_lin(ctx, name, &L));
+    if (!x_dev || !y_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward %s: null operand or t=0", name);
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    if (path == W4A16_PATH_AUTO) {
+        if (!L->q_tiled)
+            path = W4A16_PATH_LANE;
+        else
+            path = t <= 16 ? W4A16_PATH_DECODE : W4A16_PATH_PREFILL;
+    }
+    switch (path) {
+        case W4A16_PATH_LANE:
+            if (!L->q_raw) return w4_fail(W4A16_ERR_NOT_FOUND, "lin %s: operands as given were dropped", name);
+            if (out_f16) return w4_fail(W4A16_ERR_UNSUPPORTED, "lin_forward %s: the bit-exact path writes f32 only", name);
+            return launch_lane(ctx, L->q_raw, L->s_raw, x_dev, y_dev, L->n, L->k, t, L->group, L->scale_bf16);
+        case W4A16_PATH_DECODE:
+            return launch_decode(ctx, *L, x_dev, y_dev, t, out_f16);
+        case W4A16_PATH_PREFILL:
+            return w4_fail(W4A16_ERR_UNSUPPORTED, "lin_forward %s: prefill path not built", name);
+        default:
+            return w4_fail(W4A16_ERR_ARG, "lin_forward %s: unknown path %d", name, path);
+    }
+}
+
+extern "C" int w4a16_lin_forward_host(w4a16_ctx* ctx, const char* name, const uint16_t* x_f16, void* y, size_t t,
+                                      int out_f16, int path) {
+    W4Lin* L = nullptr;
+    W4_TRY(find_lin(ctx, name, &L));
+    if (!x_f16 || !y || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_host %s: null operand or t=0", name);
+    const size_t xb = t * L->k * 2, yb = t * L->n * (out_f16 ? 2 : 4);
+    uint64_t dx = 0, dy = 0;
+    int rc = w4a16_alloc(ctx, xb, &dx);
+    if (!rc) rc = w4a16_alloc(ctx, yb, &dy);
+    if (!rc) rc = w4a16_h2d(ctx, dx, x_f16, xb);
+    if (!rc) rc = w4a16_lin_forward(ctx, name, dx, dy, t, out_f16, path);
+    if (!rc) rc = w4a16_d2h(ctx, y, dy, yb);
+    const std::string keep = w4_err_save();
+    (void)w4a16_free(ctx, dx);
+    (void)w4a16_free(ctx, dy);
+    if (rc) w4_err_restore(keep);
+    return rc;
+}
+
+extern "C" int w4a16_dequant_dump(w4a16_ctx* ctx, const char* name, int from_tiled, uint64_t out_f32_dev) {
+    W4Lin* L = nullptr;
+    W4_TRY(find_lin(ctx, name, &L));
+    if (!out_f32_dev) return w4_fail(W4A16_ERR_ARG, "dequant_dump %s: null output", name);
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    int ni = (int)L->n, ki = (int)L->k, gi = (int)L->group, rbi = (int)L->row_blocks;
+    if (from_tiled) {
+        if (!L->q_tiled) return w4_fail(W4A16_ERR_NOT_FOUND, "lin %s: no tiled copy", name);
+        void* p[] = {&L->q_tiled, &L->s_tiled, &out_f32_dev, &ni, &ki, &gi, &rbi};
+        return w4_launch(ctx, L->scale_bf16 ? "w4a16_dump_tiled_bf16" : "w4a16_dump_tiled_f16",
+                         ceil_div(L->row_blocks * (L->k / 128) * 256, 256), 1, 256, 0, p);
+    }
+    if (!L->q_raw) return w4_fail(W4A16_ERR_NOT_FOUND, "lin %s: operands as given were dropped", name);
+    void* p[] = {&L->q_raw, &L->s_raw, &out_f32_dev, &ni, &ki, &gi};
+    return w4_launch(ctx, L->scale_bf16 ? "w4a16_dump_raw_bf16" : "w4a16_dump_raw_f16", ceil_div(L->n * (L->k / 8), 256),
+                     1, 256, 0, p);
+}
+
+extern "C" int w4a16_lin_untile(w4a16_ctx* ctx, const char* name, uint64_t q_out_dev, uint64_t s_out_dev) {
+    W4Lin* L = nullptr;
+    W4_TRY(find_lin(ctx, name, &L));
+    if (!q_out_dev || !s_out_dev) return w4_fail(W4A16_ERR_ARG, "lin_untile %s: null output", name);
+    if (!L->q_tiled) return w4_fail(W4A16_ERR_NOT_FOUND, "lin %s: no tiled copy", name);
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    int ni = (int)L->n, ki = (int)L->k, kgi = (int)(L->k / L->group);
+    void* pq[] = {&L->q_tiled, &q_out_dev, &ni, &ki};
+    W4_TRY(w4_launch(ctx, "w4a16_untile_q", ceil_div(L->n * (L->k / 8), 256), 1, 256, 0, pq));
+    void* ps[] = {&L->s_tiled, &s_out_dev, &ni, &kgi};
+    return w4_launch(ctx, "w4a16_untile_s", ceil_div(L->n * (L->k / L->group), 256), 1, 256, 0, ps);
+}
+
+extern "C" int w4a16_set_decode_shape(w4a16_ctx* ctx, int rows_per_wave, int waves_per_block) {
+    if (!ctx) return w4_fail(W4A16_ERR_ARG, "set_decode_shape: null context");
+    if ((rows_per_wave != 0 && rows_per_wave != 16 && rows_per_wave != 32 && rows_per_wave != 64) ||
+        waves_per_block < 0 || waves_per_block > 16)
+        return w4_fail(W4A16_ERR_ARG, "set_decode_shape: rows_per_wave in {0,16,32,64}, waves_per_block in 0..16");
+    ctx->decode_rows_per_wave = rows_per_wave;
+    ctx->decode_waves_per_block = waves_per_block;
+    return 0;
+}

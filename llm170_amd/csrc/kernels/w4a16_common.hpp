@@ -1,0 +1,83 @@
+// Device helpers shared by the gfx950 W4A16 kernels.
+//
+// Tiled weight layout ("T16x128"), produced at upload from the operand format q u32 [n][k/8]:
+//   a tile covers 16 output rows x 128 k and is 1 KiB, stored as 64 lanes x 16 B; tiles are ordered
+//   [row_block = n/16][k_tile = k/128], so one row block's k range is one contiguous run.
+//   lane l = g*16 + r (r = row in block, g = 0..3) owns dwords w = 0..3; dword w holds the eight weights
+//   k = k_tile*128 + w*32 + g*8 + j, j = 0..7.  With this choice dword w of all 64 lanes is exactly the A operand
+//   (16 rows x 32 k) of one v_mfma_f32_16x16x32_f16, and for group size 32 that MFMA stays inside one scale group.
+//   Inside a dword the nibbles are interleaved: nibble position p holds j = PERM[p], PERM = {0,2,4,6,1,3,5,7}, so
+//   that (dword & 0x000F000F) picks the pair (j=0, j=1) into the two f16 halves of one register, etc.
+// Tiled scale layout: u16 [row_block][k/group][16 rows] (the 4 rows an MFMA result lane owns are 8 contiguous bytes).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef float f16_t __attribute__((ext_vector_type(16)));
+typedef unsigned u2_t __attribute__((ext_vector_type(2)));
+typedef unsigned u4_t __attribute__((ext_vector_type(4)));
+
+#define W4_TILE_ROWS 16
+#define W4_TILE_K 128
+
+// nibble position p (bits 4p..4p+3) of a tiled dword holds element PERM[p]; element j sits at position POS[j]
+__device__ __forceinline__ int w4_perm(int p) { return ((p & 3) << 1) | (p >> 2); }
+__device__ __forceinline__ int w4_pos(int j) { return ((j & 1) << 2) | (j >> 1); }
+
+// Eight weights of one tiled dword as exact f16 integers (nibble - 8), in element order j = 0..7.
+// 0x6400 is f16 1024.0 (mantissa unit 1): or-ing a nibble into bits 0..3 gives 1024 + nibble exactly.
+// 0x5400 is f16 64.0 (mantissa unit 1/16): or-ing a nibble into bits 4..7 gives 64 + nibble exactly.
+__device__ __forceinline__ h8_t w4_deq8(unsigned w) {
+    const h2_t off_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
+    const h2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+    unsigned w1 = w >> 8;
+    unsigned a0 = (w & 0x000F000Fu) | 0x64006400u;
+    unsigned a1 = (w & 0x00F000F0u) | 0x54005400u;
+    unsigned a2 = (w1 & 0x000F000Fu) | 0x64006400u;
+    unsigned a3 = (w1 & 0x00F000F0u) | 0x54005400u;
+    h2_t p0 = __builtin_bit_cast(h2_t, a0) + off_lo;
+    h2_t p1 = __builtin_bit_cast(h2_t, a1) + off_hi;
+    h2_t p2 = __builtin_bit_cast(h2_t, a2) + off_lo;
+    h2_t p3 = __builtin_bit_cast(h2_t, a3) + off_hi;
+    h8_t r;
+    r[0] = p0[0]; r[1] = p0[1]; r[2] = p1[0]; r[3] = p1[1];
+    r[4] = p2[0]; r[5] = p2[1]; r[6] = p3[0]; r[7] = p3[1];
+    return r;
+}
+
+// IEEE binary16 bits -> f32 by integer manipulation (subnormals normalised, Inf/NaN payload shifted), the routine
+// the reference uses on both host and device (crates/core/src/quant/deq.rs:4-27).
+__device__ __forceinline__ float w4_half_bits_to_f32(unsigned h) {
+    unsigned sign = (h >> 15) & 1u, exp = (h >> 10) & 0x1fu, frac = h & 0x3ffu, bits;
+    if (exp == 0) {
+        if (frac == 0) {
+            bits = sign << 31;
+        } else {
+            int sh = __builtin_clz(frac) - 21;  // shifts needed to bring the leading one to bit 10
+            unsigned f = (frac << sh) & 0x3ffu;
+            bits = (sign << 31) | ((unsigned)(127 - 15 + 1 - sh) << 23) | (f << 13);
+        }
+    } else if (exp == 0x1f) {
+        bits = (sign << 31) | (0xffu << 23) | (frac << 13);
+    } else {
+        bits = (sign << 31) | ((exp + 112u) << 23) | (frac << 13);
+    }
+    return __builtin_bit_cast(float, bits);
+}
+
+template <bool SBF>
+__device__ __forceinline__ float w4_scale_to_f32(unsigned bits16) {
+    if (SBF) return __builtin_bit_cast(float, bits16 << 16);  // crates/core/src/quant/deq.rs:29-31
+    return w4_half_bits_to_f32(bits16);
+}
+
+// Fast-path scale conversion: hardware cvt for f16 (identical to the integer routine for every finite value).
+template <bool SBF>
+__device__ __forceinline__ float w4_scale_fast(unsigned bits16) {
+    if (SBF) return __builtin_bit_cast(float, bits16 << 16);
+    return (float)__builtin_bit_cast(_Float16, (unsigned short)bits16);
+}

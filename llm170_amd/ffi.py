@@ -1,0 +1,97 @@
+"""ctypes binding of libw4a16hip.so (include/w4a16_hip.h).  No fallback: if the library or its gfx950 code objects
+are missing, loading fails with an error that says how to build them."""
+import ctypes as C
+import os
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG, "libw4a16hip.so")
+
+ERR_SHAPE, ERR_SYMBOL, ERR_UNSUPPORTED, ERR_NOT_FOUND, ERR_ARG, ERR_ASSET = 10001, 10002, 10003, 10004, 10005, 10006
+PATH_AUTO, PATH_LANE, PATH_DECODE, PATH_PREFILL = 0, 1, 2, 3
+
+
+class W4a16Error(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("%s [code %d]" % (message, code))
+        self.code = code
+        self.message = message
+
+
+_SIGS = {
+    "w4a16_last_error": (C.c_char_p, []),
+    "w4a16_ctx_create": (C.c_int, [C.c_int, C.c_char_p, C.POINTER(C.c_void_p)]),
+    "w4a16_ctx_destroy": (None, [C.c_void_p]),
+    "w4a16_module_load": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_char_p), C.c_size_t]),
+    "w4a16_has_symbol": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "w4a16_launch": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint, C.c_uint, C.c_uint, C.c_uint, C.POINTER(C.c_void_p)]),
+    "w4a16_alloc": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_uint64)]),
+    "w4a16_free": (C.c_int, [C.c_void_p, C.c_uint64]),
+    "w4a16_h2d": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_size_t]),
+    "w4a16_d2h": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_size_t]),
+    "w4a16_d2d": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t]),
+    "w4a16_memset0": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t]),
+    "w4a16_sync": (C.c_int, [C.c_void_p]),
+    "w4a16_allocated_bytes": (C.c_size_t, [C.c_void_p]),
+    "w4a16_event_create": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "w4a16_event_record": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "w4a16_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
+    "w4a16_event_destroy": (None, [C.c_void_p, C.c_void_p]),
+    "w4a16_manifest": (C.c_size_t, [C.c_size_t, C.POINTER(C.c_char_p), C.POINTER(C.POINTER(C.c_char_p))]),
+    "w4a16_check_shapes": (C.c_int, [C.c_size_t] * 7),
+    "w4a16_kernel_sym": (C.c_char_p, [C.c_int, C.c_int]),
+    "w4a16_gemm_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t,
+                                  C.c_size_t, C.c_int, C.c_void_p]),
+    "w4a16_upload_lin": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t,
+                                   C.c_size_t, C.c_size_t, C.c_int]),
+    "w4a16_lin_drop_raw": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "w4a16_lin_info": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t),
+                                 C.POINTER(C.c_size_t), C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "w4a16_lin_forward": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_size_t, C.c_int, C.c_int]),
+    "w4a16_lin_forward_host": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int]),
+    "w4a16_dequant_dump": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int, C.c_uint64]),
+    "w4a16_lin_untile": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64]),
+    "w4a16_set_decode_shape": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the in-tree shared library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libw4a16hip.so is not built: run `python -m llm170_amd.build` (needs hipcc)")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGS.items():
+            fn = getattr(lib, name)  # AttributeError if the library lacks a declared entry point
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def declared_symbols():
+    return sorted(_SIGS)
+
+
+def check(rc):
+    if rc != 0:
+        raise W4a16Error(rc, load().w4a16_last_error().decode("utf-8", "replace"))
+
+
+def manifest():
+    lib = load()
+    out = {}
+    count = lib.w4a16_manifest(1 << 30, None, None)
+    for a in range(count):
+        name = C.c_char_p()
+        syms = C.POINTER(C.c_char_p)()
+        lib.w4a16_manifest(a, C.byref(name), C.byref(syms))
+        lst = []
+        i = 0
+        while syms[i]:
+            lst.append(syms[i].decode())
+            i += 1
+        out[name.value.decode()] = lst
+    return out

@@ -1,0 +1,218 @@
+"""Host-side mirror of the reference's operator interface for the W4A16 linear path, over the C ABI.
+
+  Ctx       <- CudaCtx                      crates/backend-gpu/src/rawcuda/ctx/mod.rs:62-77
+  Gptq4     <- Gptq4 (gemv / gemm)          crates/backend-gpu/src/rawcuda/gptq4.rs:72-190
+  W4a16Dec  <- W4a16Dec linear entry points crates/backend-gpu/src/rawcuda/w4a16_dec/upload.rs:4-65,
+                                            w4a16_dec/kernels/mod.rs:121-144
+
+Same names, argument meaning and error behaviour (errors surface as W4a16Error carrying the library's message).
+numpy arrays stand in for the Rust slices; device pointers are plain ints.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import ffi
+from .ffi import PATH_AUTO, PATH_DECODE, PATH_LANE, PATH_PREFILL, W4a16Error  # noqa: F401
+
+
+def check_shapes(t, qlen, slen, xlen, n, k, group):
+    """gptq4.rs:31-58.  Raises W4a16Error(ERR_SHAPE) on violation."""
+    ffi.check(ffi.load().w4a16_check_shapes(t, qlen, slen, xlen, n, k, group))
+
+
+def kernel_sym(group, scale_bf16):
+    """gptq4.rs:60-70."""
+    r = ffi.load().w4a16_kernel_sym(int(group), int(bool(scale_bf16)))
+    if r is None:
+        ffi.check(ffi.ERR_UNSUPPORTED)
+    return r.decode()
+
+
+def _ptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class Event:
+    def __init__(self, ctx):
+        self.ctx = ctx
+        h = C.c_void_p()
+        ffi.check(ctx.lib.w4a16_event_create(ctx.h, C.byref(h)))
+        self.h = h
+
+    def record(self):
+        ffi.check(self.ctx.lib.w4a16_event_record(self.ctx.h, self.h))
+
+    def elapsed_ms(self, stop):
+        ms = C.c_float()
+        ffi.check(self.ctx.lib.w4a16_event_elapsed_ms(self.ctx.h, self.h, stop.h, C.byref(ms)))
+        return ms.value
+
+    def destroy(self):
+        if self.h:
+            self.ctx.lib.w4a16_event_destroy(self.ctx.h, self.h)
+            self.h = None
+
+
+class Ctx:
+    """Device context: launch stream, loaded gfx950 code objects, tracked allocations."""
+
+    def __init__(self, device=0, asset_dir=None):
+        self.lib = ffi.load()
+        h = C.c_void_p()
+        ffi.check(self.lib.w4a16_ctx_create(device, asset_dir.encode() if asset_dir else None, C.byref(h)))
+        self.h = h
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.lib.w4a16_ctx_destroy(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # ---- CudaCtx::alloc / free / h2d / d2h / d2d / sync
+    def alloc(self, nbytes):
+        p = C.c_uint64()
+        ffi.check(self.lib.w4a16_alloc(self.h, nbytes, C.byref(p)))
+        return p.value
+
+    def free(self, dptr):
+        ffi.check(self.lib.w4a16_free(self.h, dptr))
+
+    def h2d(self, dptr, arr):
+        arr = np.ascontiguousarray(arr)
+        ffi.check(self.lib.w4a16_h2d(self.h, dptr, _ptr(arr), arr.nbytes))
+
+    def d2h(self, dptr, shape, dtype):
+        out = np.empty(shape, dtype)
+        ffi.check(self.lib.w4a16_d2h(self.h, _ptr(out), dptr, out.nbytes))
+        return out
+
+    def d2d(self, dst, src, nbytes):
+        ffi.check(self.lib.w4a16_d2d(self.h, dst, src, nbytes))
+
+    def memset0(self, dptr, nbytes):
+        ffi.check(self.lib.w4a16_memset0(self.h, dptr, nbytes))
+
+    def to_device(self, arr):
+        arr = np.ascontiguousarray(arr)
+        p = self.alloc(arr.nbytes)
+        self.h2d(p, arr)
+        return p
+
+    def sync(self):
+        ffi.check(self.lib.w4a16_sync(self.h))
+
+    def allocated_bytes(self):
+        return self.lib.w4a16_allocated_bytes(self.h)
+
+    def has_symbol(self, name):
+        return self.lib.w4a16_has_symbol(self.h, name.encode()) == 0
+
+    def function(self, name):
+        """CudaCtx::function: raises for an unknown symbol, naming it."""
+        ffi.check(self.lib.w4a16_has_symbol(self.h, name.encode()))
+        return name
+
+    def launch(self, symbol, gx, gy, block, args, shmem=0):
+        """CudaCtx::launch: args is a list of ctypes scalars (kept alive for the call)."""
+        arr = (C.c_void_p * len(args))(*[C.cast(C.byref(a), C.c_void_p) for a in args])
+        ffi.check(self.lib.w4a16_launch(self.h, symbol.encode(), gx, gy, block, shmem, arr))
+
+    def event(self):
+        return Event(self)
+
+
+class Gptq4:
+    """Standalone operator on the bit-exact kernel (upload, launch, download per call)."""
+
+    def __init__(self, ctx=None):
+        self.cc = ctx or Ctx()
+
+    def gemv(self, x, q, s, n, k, group, scale_bf16):
+        return self.gemm(x, 1, q, s, n, k, group, scale_bf16)
+
+    def gemm(self, x, t, q, s, n, k, group, scale_bf16):
+        x = np.ascontiguousarray(x, np.uint16).ravel()
+        q = np.ascontiguousarray(q, np.uint32).ravel()
+        s = np.ascontiguousarray(s, np.uint16).ravel()
+        check_shapes(t, q.size, s.size, x.size, n, k, group)
+        kernel_sym(group, scale_bf16)
+        out = np.empty((t, n), np.float32)
+        ffi.check(self.cc.lib.w4a16_gemm_host(self.cc.h, _ptr(x), t, _ptr(q), _ptr(s), n, k, group,
+                                              int(bool(scale_bf16)), _ptr(out)))
+        return out.ravel()
+
+
+class W4a16Dec:
+    """Resident linears by name and the regime dispatch."""
+
+    def __init__(self, ctx=None):
+        self.cc = ctx or Ctx()
+
+    def upload_lin(self, name, q, s, n, k):
+        return self.upload_lin_g(name, q, s, n, k, 128, False)
+
+    def upload_lin_g(self, name, q, s, n, k, group, scale_bf16):
+        q = np.ascontiguousarray(q)
+        s = np.ascontiguousarray(s)
+        ffi.check(self.cc.lib.w4a16_upload_lin(self.cc.h, name.encode(), _ptr(q), q.nbytes, _ptr(s), s.nbytes, n, k,
+                                               group, int(bool(scale_bf16))))
+
+    def lin_spec(self, name):
+        n, k, g = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        bf, tiled, raw = C.c_int(), C.c_int(), C.c_int()
+        ffi.check(self.cc.lib.w4a16_lin_info(self.cc.h, name.encode(), C.byref(n), C.byref(k), C.byref(g), C.byref(bf),
+                                             C.byref(tiled), C.byref(raw)))
+        return {"n": n.value, "k": k.value, "group": g.value, "scale_bf16": bool(bf.value),
+                "tiled": bool(tiled.value), "raw": bool(raw.value)}
+
+    def drop_raw(self, name):
+        ffi.check(self.cc.lib.w4a16_lin_drop_raw(self.cc.h, name.encode()))
+
+    def lin_forward(self, name, x_dev, dst_dev, t, out_f16=False, path=PATH_AUTO):
+        ffi.check(self.cc.lib.w4a16_lin_forward(self.cc.h, name.encode(), x_dev, dst_dev, t, int(out_f16), path))
+
+    def gemv_host(self, name, x, t=1, out_f16=False, path=PATH_AUTO):
+        """Host operands in, host result out: y [t][n] (f32, or f16 bit patterns when out_f16)."""
+        spec = self.lin_spec(name)
+        x = np.ascontiguousarray(x, np.uint16).ravel()
+        if x.size != t * spec["k"]:
+            raise W4a16Error(ffi.ERR_SHAPE, "gemv_host %s: x has %d halves, want t*k = %d" % (name, x.size, t * spec["k"]))
+        y = np.empty((t, spec["n"]), np.uint16 if out_f16 else np.float32)
+        ffi.check(self.cc.lib.w4a16_lin_forward_host(self.cc.h, name.encode(), _ptr(x), _ptr(y), t, int(out_f16), path))
+        return y
+
+    def dequant(self, name, from_tiled=True):
+        spec = self.lin_spec(name)
+        nbytes = spec["n"] * spec["k"] * 4
+        p = self.cc.alloc(nbytes)
+        try:
+            ffi.check(self.cc.lib.w4a16_dequant_dump(self.cc.h, name.encode(), int(from_tiled), p))
+            return self.cc.d2h(p, (spec["n"], spec["k"]), np.float32)
+        finally:
+            self.cc.free(p)
+
+    def untile(self, name):
+        spec = self.lin_spec(name)
+        n, k, g = spec["n"], spec["k"], spec["group"]
+        pq, ps = self.cc.alloc(n * (k // 8) * 4), self.cc.alloc(n * (k // g) * 2)
+        try:
+            ffi.check(self.cc.lib.w4a16_lin_untile(self.cc.h, name.encode(), pq, ps))
+            return self.cc.d2h(pq, (n, k // 8), np.uint32), self.cc.d2h(ps, (n, k // g), np.uint16)
+        finally:
+            self.cc.free(pq)
+            self.cc.free(ps)
+
+    def set_decode_shape(self, rows_per_wave=0, waves_per_block=0):
+        ffi.check(self.cc.lib.w4a16_set_decode_shape(self.cc.h, rows_per_wave, waves_per_block))

@@ -1,0 +1,75 @@
+"""CPU-side checks of the host library: it loads, exports every declared entry point, its asset manifest matches the
+kernel sources, and the shape contract behaves as the reference's (no GPU calls)."""
+import os
+import re
+
+import pytest
+
+from llm170_amd import ffi, ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ffi.load()
+    header = open(os.path.join(ROOT, "include", "w4a16_hip.h")).read()
+    declared = set(re.findall(r"\b(w4a16_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations parsed"
+    for name in sorted(declared):
+        assert hasattr(lib, name), name
+    assert declared == set(ffi.declared_symbols())
+
+
+def test_manifest_matches_kernel_sources():
+    """Precedent: manifest symbols == extern "C" __global__ symbols of the .cu files (assets.rs:394-443)."""
+    man = ffi.manifest()
+    kdir = os.path.join(ROOT, "llm170_amd", "csrc", "kernels")
+    for asset, syms in man.items():
+        text = open(os.path.join(kdir, asset + ".hip")).read()
+        direct = re.findall(r'extern "C" __global__[^;{]*?\bvoid\s+(w4a16_\w+)\s*\(', text)
+        via_macro = re.findall(r"^[A-Z0-9_]+_KERNEL\((w4a16_\w+)", text, flags=re.M)
+        assert sorted(set(direct + via_macro)) == sorted(syms), asset
+        assert len(set(syms)) == len(syms)
+    hips = sorted(f[:-4] for f in os.listdir(kdir) if f.endswith(".hip"))
+    assert hips == sorted(man), "every kernel source is a manifest asset and vice versa"
+
+
+def test_shapes_accept_contract():
+    # gptq4.rs:196-208
+    ops.check_shapes(1, 8 * 640, 8 * 40, 5120, 8, 5120, 128)
+    ops.check_shapes(8, 8 * 640, 8 * 40, 8 * 5120, 8, 5120, 128)
+    ops.check_shapes(1, 512 * 256, 512 * 64, 2048, 512, 2048, 32)
+    ops.check_shapes(8, 512 * 256, 512 * 64, 8 * 2048, 512, 2048, 32)
+    ops.check_shapes(1, 8 * 1024, 8 * 256, 8192, 8, 8192, 32)
+
+
+def test_shapes_reject_bad_rank_and_misalignment():
+    # gptq4.rs:210-216
+    for args in [(1, 8 * 640, 8 * 40, 5120, 8, 5121, 128), (0, 8 * 640, 8 * 40, 0, 8, 5120, 128),
+                 (1, 7 * 640, 8 * 40, 5120, 8, 5120, 128), (1, 8 * 640, 8 * 40, 5120, 8, 5120, 64)]:
+        with pytest.raises(ops.W4a16Error) as e:
+            ops.check_shapes(*args)
+        assert e.value.code == ffi.ERR_SHAPE and "shape contract" in str(e.value)
+
+
+def test_gemv_k_limit_of_the_reference_is_not_carried_over():
+    # gptq4.rs:218-223 rejects t == 1 with k > 256 * group (shared-memory scale cache); no such cache here
+    ops.check_shapes(1, 8 * 4112, 8 * 257, 32896, 8, 32896, 128)
+    ops.check_shapes(2, 8 * 4112, 8 * 257, 2 * 32896, 8, 32896, 128)
+
+
+def test_kernel_sym_selects_variants():
+    # gptq4.rs:225-233 (the two combinations the reference rejects are served here)
+    assert ops.kernel_sym(128, False) == "w4a16_lane_g128_f16"
+    assert ops.kernel_sym(32, True) == "w4a16_lane_g32_bf16"
+    assert ops.kernel_sym(32, False) == "w4a16_lane_g32_f16"
+    with pytest.raises(ops.W4a16Error) as e:
+        ops.kernel_sym(64, False)
+    assert e.value.code == ffi.ERR_UNSUPPORTED
+
+
+def test_code_objects_are_gfx950():
+    adir = os.path.join(ROOT, "llm170_amd", "assets")
+    for asset in ffi.manifest():
+        blob = open(os.path.join(adir, asset + ".hsaco"), "rb").read()
+        assert blob[:4] == b"\x7fELF" and b"gfx950" in blob, asset
