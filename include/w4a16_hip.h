@@ -112,7 +112,7 @@ int w4a16_gemm_host(w4a16_ctx* ctx, const uint16_t* x_f16, size_t t, const uint3
 
 /* W4a16Dec::upload_lin_g (w4a16_dec/upload.rs:15-65): register a linear by name.  q: n*k/2 bytes, s: n*(k/group)*2
  * bytes in the operand format above; lengths are enforced.  Keeps the operands resident as given and, when
- * n % 16 == 0 and k % 128 == 0, also in the tiled layout the streaming and MFMA kernels read (the reference likewise
+ * k % 128 == 0 (rows are padded to a multiple of 16), also in the tiled layout the streaming and MFMA kernels read (the reference likewise
  * keeps a repacked copy next to the original, upload.rs:99-179).  Re-registering a name frees the old buffers. */
 int w4a16_upload_lin(w4a16_ctx* ctx, const char* name, const void* q, size_t qlen_bytes, const void* s,
                      size_t slen_bytes, size_t n, size_t k, size_t group, int scale_bf16);
@@ -149,9 +149,19 @@ int w4a16_dequant_dump(w4a16_ctx* ctx, const char* name, int from_tiled, uint64_
 int w4a16_lin_untile(w4a16_ctx* ctx, const char* name, uint64_t q_out_dev, uint64_t s_out_dev);
 
 /* Launch-shape override for the decode kernel (0 = choose automatically): rows_per_wave in {16,32,64},
- * waves_per_block in 1..16.  For tuning sweeps (the reference exposes its split-K factor the same way,
+ * waves_per_block in 1..8.  For tuning sweeps (the reference exposes its split-K factor the same way,
  * sk_ksp, w4a16_dec/kernels/decode.rs:3-16). */
 int w4a16_set_decode_shape(w4a16_ctx* ctx, int rows_per_wave, int waves_per_block);
+
+/* run_bench_gemv / run_bench_gemm (crates/server/src/probes/w4a16/gpu/bench.rs:366-433): `warmup` untimed then
+ * `reps` timed back-to-back lin_forward launches on the launch stream, one synchronisation at the end.  Launch i
+ * uses linear names[i % n_names] — rotating over copies whose total size exceeds the last-level caches gives the
+ * cold-HBM figure, a single name the warm one (the reference flushes with a 256 MiB copy instead, probe.rs:1198-1230).
+ * All named linears must have the same shape.  ms_events = elapsed between HIP events recorded on the launch stream
+ * around the timed launches; ms_wall = host wall clock around the same region including the final sync. */
+int w4a16_bench_forward(w4a16_ctx* ctx, const char* const* names, size_t n_names, uint64_t x_dev, uint64_t y_dev,
+                        size_t t, int out_f16, int path, size_t warmup, size_t reps, float* ms_events,
+                        double* ms_wall);
 
 #ifdef __cplusplus
 }

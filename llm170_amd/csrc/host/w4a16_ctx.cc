@@ -3,6 +3,7 @@
 // (crates/backend-gpu/src/rawcuda/ffi.rs:237-459, ctx/mod.rs:62-419, ctx/mem.rs, ctx/prof.rs, assets.rs).
 #include <dlfcn.h>
 
+#include <algorithm>
 #include <cctype>
 #include <cstdio>
 #include <cstdlib>
@@ -45,11 +46,16 @@ static const char* const kLayoutSyms[] = {"w4a16_tile_q",         "w4a16_tile_s"
                                           "w4a16_untile_s",       "w4a16_dump_tiled_f16",  "w4a16_dump_tiled_bf16",
                                           "w4a16_dump_raw_f16",   "w4a16_dump_raw_bf16",   nullptr};
 static const char* const kDecodeSyms[] = {
-    "w4a16_decode_g128_f16_rb1",  "w4a16_decode_g128_f16_rb2",  "w4a16_decode_g128_f16_rb4",
-    "w4a16_decode_g32_f16_rb1",   "w4a16_decode_g32_f16_rb2",   "w4a16_decode_g32_f16_rb4",
-    "w4a16_decode_g128_bf16_rb1", "w4a16_decode_g128_bf16_rb2", "w4a16_decode_g128_bf16_rb4",
-    "w4a16_decode_g32_bf16_rb1",  "w4a16_decode_g32_bf16_rb2",  "w4a16_decode_g32_bf16_rb4",
+    "w4a16_decode_g128_f16_rb1", "w4a16_decode_g128_f16_rb1_xl", "w4a16_decode_g128_f16_rb2",
+    "w4a16_decode_g128_f16_rb2_xl", "w4a16_decode_g128_f16_rb4", "w4a16_decode_g128_f16_rb4_xl",
+    "w4a16_decode_g128_bf16_rb1", "w4a16_decode_g128_bf16_rb1_xl", "w4a16_decode_g128_bf16_rb2",
+    "w4a16_decode_g128_bf16_rb2_xl", "w4a16_decode_g128_bf16_rb4", "w4a16_decode_g128_bf16_rb4_xl",
+    "w4a16_decode_g32_f16_rb1", "w4a16_decode_g32_f16_rb1_xl", "w4a16_decode_g32_f16_rb2",
+    "w4a16_decode_g32_f16_rb2_xl", "w4a16_decode_g32_f16_rb4", "w4a16_decode_g32_f16_rb4_xl",
+    "w4a16_decode_g32_bf16_rb1", "w4a16_decode_g32_bf16_rb1_xl", "w4a16_decode_g32_bf16_rb2",
+    "w4a16_decode_g32_bf16_rb2_xl", "w4a16_decode_g32_bf16_rb4", "w4a16_decode_g32_bf16_rb4_xl",
     nullptr};
+static const char* const kUtilSyms[] = {"w4a16_fill0_u32", "w4a16_copy_u4", nullptr};
 
 struct W4Asset {
     const char* name;
@@ -59,6 +65,7 @@ static const W4Asset kAssets[] = {
     {"lane", kLaneSyms},
     {"layout", kLayoutSyms},
     {"decode", kDecodeSyms},
+    {"util", kUtilSyms},
 };
 static const size_t kAssetCount = sizeof kAssets / sizeof kAssets[0];
 
@@ -262,8 +269,13 @@ extern "C" int w4a16_d2d(w4a16_ctx* ctx, uint64_t dst, uint64_t src, size_t byte
 extern "C" int w4a16_memset0(w4a16_ctx* ctx, uint64_t dst, size_t bytes) {
     if (!ctx || !dst) return w4_fail(W4A16_ERR_ARG, "memset0: null argument");
     if (bytes == 0) return 0;
+    if ((dst & 3) || (bytes & 3)) return w4_fail(W4A16_ERR_ARG, "memset0: address and size must be multiples of 4");
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
-    return w4_hip(hipMemsetAsync((void*)dst, 0, bytes, ctx->stream), "hipMemsetAsync");
+    // a fill kernel rather than a memset node: memset nodes are not replay-safe inside captured graphs here
+    size_t words = bytes / 4;
+    unsigned grid = (unsigned)std::min<size_t>((words + 255) / 256, 4096);
+    void* params[] = {&dst, &words};
+    return w4_launch(ctx, "w4a16_fill0_u32", grid, 1, 256, 0, params);
 }
 
 extern "C" int w4a16_sync(w4a16_ctx* ctx) {

@@ -3,6 +3,7 @@
 // upload_lin_g / lin_forward / gemv_t_launch / gemm_launch (w4a16_dec/upload.rs:15-65, kernels/mod.rs:121-144,
 // kernels/gemv.rs:112-187, kernels/gemm.rs:4-51).
 #include <algorithm>
+#include <chrono>
 #include <cstring>
 
 #include "w4a16_internal.h"
@@ -49,7 +50,7 @@ static int pick_decode_shape(const w4a16_ctx* ctx, const W4Lin& L, size_t t, int
         const int tiles_per_wave = std::max(1, 8 / rb);
         waves = (kt_n + tiles_per_wave - 1) / tiles_per_wave;
     }
-    waves = std::max(1, std::min(std::min(waves, 16), kt_n));
+    waves = std::max(1, std::min(std::min(waves, 8), kt_n));
     *rb_out = rb;
     *waves_out = waves;
     return 0;
@@ -60,12 +61,18 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode: linear has no tiled copy (needs k %% 128 == 0)");
     int rb = 0, waves = 0;
     W4_TRY(pick_decode_shape(ctx, L, t, &rb, &waves));
+    if (L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
+        return w4_fail(W4A16_ERR_SHAPE, "decode: tiled weights of 2 GiB or more exceed the buffer-descriptor range");
+    // x goes through LDS when it fits beside a second resident workgroup (kernels/decode.hip, XLDS variants)
+    const size_t x_lds = t * (L.k + 32) * 2;
+    const bool xl = x_lds <= 64 * 1024;
     char sym[64];
-    snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_rb%d", L.group, L.scale_bf16 ? "bf16" : "f16", rb);
+    snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_rb%d%s", L.group, L.scale_bf16 ? "bf16" : "f16", rb, xl ? "_xl" : "");
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of};
     unsigned shmem = waves > 1 ? (unsigned)(waves * rb * 64 * 16) : 0;
+    if (xl) shmem = std::max(shmem, (unsigned)x_lds);
     return w4_launch(ctx, sym, ceil_div(L.row_blocks, (size_t)rb), 1, (unsigned)(waves * 64), shmem, params);
 }
 
@@ -263,9 +270,47 @@ extern "C" int w4a16_lin_untile(w4a16_ctx* ctx, const char* name, uint64_t q_out
 extern "C" int w4a16_set_decode_shape(w4a16_ctx* ctx, int rows_per_wave, int waves_per_block) {
     if (!ctx) return w4_fail(W4A16_ERR_ARG, "set_decode_shape: null context");
     if ((rows_per_wave != 0 && rows_per_wave != 16 && rows_per_wave != 32 && rows_per_wave != 64) ||
-        waves_per_block < 0 || waves_per_block > 16)
-        return w4_fail(W4A16_ERR_ARG, "set_decode_shape: rows_per_wave in {0,16,32,64}, waves_per_block in 0..16");
+        waves_per_block < 0 || waves_per_block > 8)
+        return w4_fail(W4A16_ERR_ARG, "set_decode_shape: rows_per_wave in {0,16,32,64}, waves_per_block in 0..8");
     ctx->decode_rows_per_wave = rows_per_wave;
     ctx->decode_waves_per_block = waves_per_block;
     return 0;
+}
+
+// ------------------------------------------------------------------------------------------------ bench probe
+extern "C" int w4a16_bench_forward(w4a16_ctx* ctx, const char* const* names, size_t n_names, uint64_t x_dev,
+                                   uint64_t y_dev, size_t t, int out_f16, int path, size_t warmup, size_t reps,
+                                   float* ms_events, double* ms_wall) {
+    if (!ctx || !names || n_names == 0 || reps == 0) return w4_fail(W4A16_ERR_ARG, "bench_forward: null argument");
+    W4Lin* first = nullptr;
+    W4_TRY(find_lin(ctx, names[0], &first));
+    for (size_t i = 1; i < n_names; i++) {
+        W4Lin* L = nullptr;
+        W4_TRY(find_lin(ctx, names[i], &L));
+        if (L->n != first->n || L->k != first->k || L->group != first->group)
+            return w4_fail(W4A16_ERR_SHAPE, "bench_forward: %s and %s differ in shape", names[0], names[i]);
+    }
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    W4_TRY(w4_hip(hipEventCreate(&e0), "hipEventCreate"));
+    int rc = w4_hip(hipEventCreate(&e1), "hipEventCreate");
+    for (size_t i = 0; i < warmup && !rc; i++)
+        rc = w4a16_lin_forward(ctx, names[i % n_names], x_dev, y_dev, t, out_f16, path);
+    if (!rc) rc = w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    auto w0 = std::chrono::steady_clock::now();
+    if (!rc) rc = w4_hip(hipEventRecord(e0, ctx->stream), "hipEventRecord");
+    for (size_t i = 0; i < reps && !rc; i++)
+        rc = w4a16_lin_forward(ctx, names[(warmup + i) % n_names], x_dev, y_dev, t, out_f16, path);
+    if (!rc) rc = w4_hip(hipEventRecord(e1, ctx->stream), "hipEventRecord");
+    if (!rc) rc = w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    auto w1 = std::chrono::steady_clock::now();
+    float ms = 0.f;
+    if (!rc) rc = w4_hip(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+    if (ms_events) *ms_events = ms;
+    if (ms_wall) *ms_wall = std::chrono::duration<double, std::milli>(w1 - w0).count();
+    const std::string keep = w4_err_save();
+    (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (rc) w4_err_restore(keep);
+    return rc;
 }

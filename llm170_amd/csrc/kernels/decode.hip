@@ -1,23 +1,38 @@
 // Decode regime (t = 1..16 activation rows): HBM-streaming skinny GEMM  y[t][n] = x[t][k] * W^T.
 // Role of the reference's gemv_t / split-K decode kernels (assets/gptq4.cu:522-553, assets/decode.cu:46-267),
 // designed for CDNA4 instead:
-//   * weights are read once, as 1 KiB tiles (64 lanes x global_load_dwordx4, non-temporal) of the tiled layout in
+//   * weights are read once, as 1 KiB tiles (64 lanes x buffer_load_dwordx4) of the tiled layout in
 //     w4a16_common.hpp — every wave-level load is one fully used contiguous KiB;
 //   * the int4 -> f16 unpack is 9 VALU ops per 8 weights and stays in registers; the multiply-accumulate runs on
 //     the matrix core: dword w of the 64 lanes is the A operand of v_mfma_f32_16x16x32_f16 (16 rows x 32 k), the
-//     B operand is x (32 k x 16 token columns, columns >= t are zero), so t = 1 and t = 16 cost the same;
+//     B operand is x (32 k x 16 token columns), so t = 1 and t = 16 cost the same arithmetic;
+//   * x: every vector-memory instruction costs the CU's address unit about as much as a full 1 KiB load, however few
+//     lanes are live, so four B-operand loads per k tile would cost more than the weight stream itself.  When
+//     t*k*2 bytes fit (XLDS variants, the normal case for t <= 4) the workgroup copies x into LDS once and the
+//     B operands come from ds_read_b128; token columns >= t read a duplicate row (their results are never stored).
+//     Otherwise x comes from raw buffer loads whose offset is out of range for columns >= t (zeros, no traffic);
 //   * weights enter the MFMA as exact integers; the per-group scale multiplies the f32 group sum, so no weight is
 //     ever rounded to f16 (error vs the f32 lane contract is summation order only);
+//   * each wave keeps DEPTH k-tiles of loads in flight (register ring, software pipelined);
 //   * split-K lives inside the workgroup: the W waves of a block take consecutive k-tile slices of the same RB row
 //     blocks and wave 0 folds the partial tiles through LDS in fixed order (deterministic, no atomics, no second
-//     launch).  The host picks RB and W so that a wave streams about 8 KiB.
+//     launch).  The host picks RB and W.
 #include "w4a16_common.hpp"
 
-template <int G, bool SBF, int RB>
+template <int G, int RB>
+struct DecodeStage {
+    u4_t q[RB];
+    u2_t s[RB][W4_TILE_K / G];
+    u4_t x[4];
+};
+
+#define W4_XLDS_PAD 32  // halves of padding per x row in LDS (rows land 16 banks apart)
+
+template <int G, bool SBF, int RB, int DEPTH, bool XLDS>
 __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                             const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
                                             int k, int n, int t, int out_f16) {
-    extern __shared__ f4_t red[];  // [W][RB][64]
+    extern __shared__ f4_t red[];  // [W][RB][64] partial tiles; XLDS: first holds x as halves [t][k + W4_XLDS_PAD]
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, W = blockDim.x >> 6;
     const int kt_n = k / W4_TILE_K;
@@ -26,35 +41,61 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     const int kt0 = (kt_n * wave) / W, kt1 = (kt_n * (wave + 1)) / W;
     const int m = lane & 15, g = lane >> 4;
     const bool xact = m < t;
-    const uint16_t* xp = x + (size_t)(xact ? m : 0) * k + g * 8;
+    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)t * (unsigned)k * 2u);
+    const unsigned xoff = xact ? ((unsigned)m * (unsigned)k + (unsigned)g * 8u) * 2u : W4_OOB;
 
+    const int xstride = k + W4_XLDS_PAD;
+    if (XLDS) {
+        // cooperative copy of x into LDS, 16 B per thread per step
+        _Float16* xs = reinterpret_cast<_Float16*>(red);
+        const int chunks_per_row = k / 8;
+        for (int c = threadIdx.x; c < t * chunks_per_row; c += blockDim.x) {
+            const int row = c / chunks_per_row, col = (c - row * chunks_per_row) * 8;
+            *reinterpret_cast<u4_t*>(xs + row * xstride + col) =
+                *reinterpret_cast<const u4_t*>(x + (size_t)row * k + col);
+        }
+        __syncthreads();
+    }
+    const _Float16* xl = reinterpret_cast<const _Float16*>(red) + min(m, t - 1) * xstride + g * 8;
+
+    // Every load is a raw buffer load: a k tile at or past kt1 gets an out-of-range offset, returns zeros and costs no
+    // memory traffic, so the pipeline needs no branch around its prefetches.
+    const __amdgpu_buffer_rsrc_t qr = w4_make_rsrc(qt, (unsigned)row_blocks * (unsigned)kt_n * 1024u);
+    const __amdgpu_buffer_rsrc_t sr = w4_make_rsrc(st, (unsigned)row_blocks * (unsigned)kg_n * 32u);
     f4_t acc[RB];
-    const u4_t* qp[RB];
-    const uint16_t* sp[RB];
+    unsigned qoff[RB], soff[RB];
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
         acc[rb] = (f4_t){0.f, 0.f, 0.f, 0.f};
-        const int nb = min(nb0 + rb, row_blocks - 1);  // a tail block re-reads the last row block, never stores it
-        qp[rb] = qt + (size_t)nb * kt_n * 64 + lane;
-        sp[rb] = st + (size_t)nb * kg_n * 16 + 4 * g;
+        const unsigned nb = (unsigned)min(nb0 + rb, row_blocks - 1);  // a tail block re-reads the last row block
+        qoff[rb] = nb * (unsigned)kt_n * 1024u + (unsigned)lane * 16u;
+        soff[rb] = nb * (unsigned)kg_n * 32u + (unsigned)g * 8u;
     }
 
-#pragma unroll 2
-    for (int kt = kt0; kt < kt1; ++kt) {
-        u4_t qv[RB];
-        u2_t sv[RB][GPT];
-        h8_t xb[4];
+    DecodeStage<G, RB> stage[DEPTH];
+    auto load = [&](DecodeStage<G, RB>& s_, int kt) {
+        const bool live = kt < kt1;
 #pragma unroll
-        for (int rb = 0; rb < RB; rb++) qv[rb] = __builtin_nontemporal_load(qp[rb] + (size_t)kt * 64);
+        for (int rb = 0; rb < RB; rb++)
+            s_.q[rb] = __builtin_amdgcn_raw_buffer_load_b128(qr, live ? qoff[rb] + (unsigned)kt * 1024u : W4_OOB, 0,
+                                                             2 /* nt: read-once stream */);
 #pragma unroll
         for (int rb = 0; rb < RB; rb++)
 #pragma unroll
             for (int gi = 0; gi < GPT; gi++)
-                sv[rb][gi] = *reinterpret_cast<const u2_t*>(sp[rb] + ((size_t)kt * GPT + gi) * 16);
+                s_.s[rb][gi] = __builtin_amdgcn_raw_buffer_load_b64(
+                    sr, live ? soff[rb] + (unsigned)(kt * GPT + gi) * 32u : W4_OOB, 0, 0);
+        if (!XLDS) {
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
-            xb[w] = (h8_t){0, 0, 0, 0, 0, 0, 0, 0};
-            if (xact) xb[w] = *reinterpret_cast<const h8_t*>(xp + kt * W4_TILE_K + w * 32);
+            for (int w = 0; w < 4; w++)
+                s_.x[w] = __builtin_amdgcn_raw_buffer_load_b128(
+                    xr, live ? xoff + (unsigned)(kt * W4_TILE_K + w * 32) * 2u : W4_OOB, 0, 0);
+        }
+    };
+    auto compute = [&](DecodeStage<G, RB>& s_, int kt) {
+        if (XLDS) {
+#pragma unroll
+            for (int w = 0; w < 4; w++) s_.x[w] = *reinterpret_cast<const u4_t*>(xl + kt * W4_TILE_K + w * 32);
         }
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
@@ -62,25 +103,47 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                 f4_t part = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int w = 0; w < 4; w++)
-                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(qv[rb][w]), xb[w], part, 0, 0, 0);
+                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
+                                                                  __builtin_bit_cast(h8_t, s_.x[w]), part, 0, 0, 0);
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    acc[rb][i] += w4_scale_fast<SBF>((sv[rb][0][i >> 1] >> (16 * (i & 1))) & 0xFFFFu) * part[i];
+                    acc[rb][i] += w4_scale_fast<SBF>((s_.s[rb][0][i >> 1] >> (16 * (i & 1))) & 0xFFFFu) * part[i];
             } else {
 #pragma unroll
                 for (int w = 0; w < 4; w++) {
                     f4_t part = {0.f, 0.f, 0.f, 0.f};
-                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(qv[rb][w]), xb[w], part, 0, 0, 0);
+                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
+                                                                  __builtin_bit_cast(h8_t, s_.x[w]), part, 0, 0, 0);
 #pragma unroll
                     for (int i = 0; i < 4; i++)
                         acc[rb][i] +=
-                            w4_scale_fast<SBF>((sv[rb][w % GPT][i >> 1] >> (16 * (i & 1))) & 0xFFFFu) * part[i];
+                            w4_scale_fast<SBF>((s_.s[rb][w % GPT][i >> 1] >> (16 * (i & 1))) & 0xFFFFu) * part[i];
                 }
             }
         }
+    };
+
+    // One counted loop does the pipeline fill (round -1, compute skipped) and the steady state, so on every path
+    // into a stage's compute the outstanding loads are in ring order and the wait can be "all but the younger stages'
+    // loads" (s_waitcnt vmcnt(N > 0)).  Tiles past kt1 load zeros (scale 0 => no contribution); the last partial
+    // round is finished by the unrolled tail below.  The scheduling barriers keep each stage's loads together.
+    const int tiles = kt1 - kt0;
+    const int rounds = tiles / DEPTH;
+    for (int r = -1; r < rounds; r++) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            if (r >= 0) compute(stage[d], kt0 + r * DEPTH + d);
+            __builtin_amdgcn_sched_barrier(0);
+            load(stage[d], kt0 + (r + 1) * DEPTH + d);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
+#pragma unroll
+    for (int d = 0; d < DEPTH - 1; d++)
+        if (rounds * DEPTH + d < tiles) compute(stage[d], kt0 + rounds * DEPTH + d);
 
     if (W > 1) {
+        if (XLDS) __syncthreads();  // everyone is done reading x before the partial tiles overwrite it
         if (wave != 0) {
 #pragma unroll
             for (int rb = 0; rb < RB; rb++) red[(wave * RB + rb) * 64 + lane] = acc[rb];
@@ -120,22 +183,27 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     }
 }
 
-#define DECODE_KERNEL(NAME, G, SBF, RB)                                                                     \
-    extern "C" __global__ __launch_bounds__(1024) void NAME(const u4_t* qt, const uint16_t* st,             \
-                                                            const uint16_t* x, void* y, int row_blocks, int k, \
-                                                            int n, int t, int out_f16) {                    \
-        decode_body<G, SBF, RB>(qt, st, x, y, row_blocks, k, n, t, out_f16);                                \
+#define DECODE_KERNEL(NAME, G, SBF, RB, DEPTH)                                                                 \
+    extern "C" __global__ __launch_bounds__(512) void NAME(const u4_t* qt, const uint16_t* st, const uint16_t* x, \
+                                                           void* y, int row_blocks, int k, int n, int t,          \
+                                                           int out_f16) {                                         \
+        decode_body<G, SBF, RB, DEPTH, false>(qt, st, x, y, row_blocks, k, n, t, out_f16);                        \
+    }                                                                                                             \
+    extern "C" __global__ __launch_bounds__(512) void NAME##_xl(const u4_t* qt, const uint16_t* st,               \
+                                                                const uint16_t* x, void* y, int row_blocks,       \
+                                                                int k, int n, int t, int out_f16) {               \
+        decode_body<G, SBF, RB, DEPTH, true>(qt, st, x, y, row_blocks, k, n, t, out_f16);                         \
     }
 
-DECODE_KERNEL(w4a16_decode_g128_f16_rb1, 128, false, 1)
-DECODE_KERNEL(w4a16_decode_g128_f16_rb2, 128, false, 2)
-DECODE_KERNEL(w4a16_decode_g128_f16_rb4, 128, false, 4)
-DECODE_KERNEL(w4a16_decode_g32_f16_rb1, 32, false, 1)
-DECODE_KERNEL(w4a16_decode_g32_f16_rb2, 32, false, 2)
-DECODE_KERNEL(w4a16_decode_g32_f16_rb4, 32, false, 4)
-DECODE_KERNEL(w4a16_decode_g128_bf16_rb1, 128, true, 1)
-DECODE_KERNEL(w4a16_decode_g128_bf16_rb2, 128, true, 2)
-DECODE_KERNEL(w4a16_decode_g128_bf16_rb4, 128, true, 4)
-DECODE_KERNEL(w4a16_decode_g32_bf16_rb1, 32, true, 1)
-DECODE_KERNEL(w4a16_decode_g32_bf16_rb2, 32, true, 2)
-DECODE_KERNEL(w4a16_decode_g32_bf16_rb4, 32, true, 4)
+DECODE_KERNEL(w4a16_decode_g128_f16_rb1, 128, false, 1, 4)
+DECODE_KERNEL(w4a16_decode_g128_f16_rb2, 128, false, 2, 3)
+DECODE_KERNEL(w4a16_decode_g128_f16_rb4, 128, false, 4, 2)
+DECODE_KERNEL(w4a16_decode_g32_f16_rb1, 32, false, 1, 3)
+DECODE_KERNEL(w4a16_decode_g32_f16_rb2, 32, false, 2, 2)
+DECODE_KERNEL(w4a16_decode_g32_f16_rb4, 32, false, 4, 2)
+DECODE_KERNEL(w4a16_decode_g128_bf16_rb1, 128, true, 1, 4)
+DECODE_KERNEL(w4a16_decode_g128_bf16_rb2, 128, true, 2, 3)
+DECODE_KERNEL(w4a16_decode_g128_bf16_rb4, 128, true, 4, 2)
+DECODE_KERNEL(w4a16_decode_g32_bf16_rb1, 32, true, 1, 3)
+DECODE_KERNEL(w4a16_decode_g32_bf16_rb2, 32, true, 2, 2)
+DECODE_KERNEL(w4a16_decode_g32_bf16_rb4, 32, true, 4, 2)

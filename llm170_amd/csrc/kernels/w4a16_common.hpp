@@ -28,17 +28,26 @@ typedef unsigned u4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ int w4_perm(int p) { return ((p & 3) << 1) | (p >> 2); }
 __device__ __forceinline__ int w4_pos(int j) { return ((j & 1) << 2) | (j >> 1); }
 
+// (w & mask) | bits in one VALU op.  The mask travels in an SGPR and the or-constant in a VGPR (one scalar operand
+// per VOP3 instruction on this target); the compiler would otherwise emit v_and + v_or with literals.
+__device__ __forceinline__ unsigned w4_and_or(unsigned w, unsigned mask, unsigned bits) {
+    unsigned r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(w), "s"(mask), "v"(bits));
+    return r;
+}
+
 // Eight weights of one tiled dword as exact f16 integers (nibble - 8), in element order j = 0..7.
 // 0x6400 is f16 1024.0 (mantissa unit 1): or-ing a nibble into bits 0..3 gives 1024 + nibble exactly.
 // 0x5400 is f16 64.0 (mantissa unit 1/16): or-ing a nibble into bits 4..7 gives 64 + nibble exactly.
+// 9 VALU ops per dword: one shift, four and-or, four packed f16 adds.
 __device__ __forceinline__ h8_t w4_deq8(unsigned w) {
     const h2_t off_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
     const h2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
     unsigned w1 = w >> 8;
-    unsigned a0 = (w & 0x000F000Fu) | 0x64006400u;
-    unsigned a1 = (w & 0x00F000F0u) | 0x54005400u;
-    unsigned a2 = (w1 & 0x000F000Fu) | 0x64006400u;
-    unsigned a3 = (w1 & 0x00F000F0u) | 0x54005400u;
+    unsigned a0 = w4_and_or(w, 0x000F000Fu, 0x64006400u);
+    unsigned a1 = w4_and_or(w, 0x00F000F0u, 0x54005400u);
+    unsigned a2 = w4_and_or(w1, 0x000F000Fu, 0x64006400u);
+    unsigned a3 = w4_and_or(w1, 0x00F000F0u, 0x54005400u);
     h2_t p0 = __builtin_bit_cast(h2_t, a0) + off_lo;
     h2_t p1 = __builtin_bit_cast(h2_t, a1) + off_hi;
     h2_t p2 = __builtin_bit_cast(h2_t, a2) + off_lo;
@@ -48,6 +57,13 @@ __device__ __forceinline__ h8_t w4_deq8(unsigned w) {
     r[4] = p2[0]; r[5] = p2[1]; r[6] = p3[0]; r[7] = p3[1];
     return r;
 }
+
+// Raw buffer descriptor over [base, base + bytes): loads whose byte offset falls outside return 0 and touch no
+// memory, which gives branch-free predication of per-lane loads.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t w4_make_rsrc(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+#define W4_OOB 0x80000000u  // a byte offset no buffer here reaches
 
 // IEEE binary16 bits -> f32 by integer manipulation (subnormals normalised, Inf/NaN payload shifted), the routine
 // the reference uses on both host and device (crates/core/src/quant/deq.rs:4-27).

@@ -216,3 +216,12 @@ class W4a16Dec:
 
     def set_decode_shape(self, rows_per_wave=0, waves_per_block=0):
         ffi.check(self.cc.lib.w4a16_set_decode_shape(self.cc.h, rows_per_wave, waves_per_block))
+
+    def bench_forward(self, names, x_dev, y_dev, t, reps, warmup=1, out_f16=False, path=PATH_AUTO):
+        """run_bench_gemv / run_bench_gemm (probes/w4a16/gpu/bench.rs:366-433): returns (ms by events, ms wall) for
+        `reps` back-to-back launches rotating over `names`."""
+        arr = (C.c_char_p * len(names))(*[n.encode() for n in names])
+        ms, wall = C.c_float(), C.c_double()
+        ffi.check(self.cc.lib.w4a16_bench_forward(self.cc.h, arr, len(names), x_dev, y_dev, t, int(out_f16), path, warmup,
+                                                  reps, C.byref(ms), C.byref(wall)))
+        return ms.value, wall.value

@@ -117,7 +117,7 @@ def test_decode_matches_oracle(dec, orc, n, k, group):
         assert np.array_equal(_bits(twin), _bits(want))
 
 
-@pytest.mark.parametrize("rows,waves", [(16, 1), (16, 16), (32, 3), (64, 7), (64, 16), (32, 1)])
+@pytest.mark.parametrize("rows,waves", [(16, 1), (16, 8), (32, 3), (64, 7), (64, 8), (32, 1), (16, 5)])
 def test_decode_launch_shapes_agree(dec, orc, rows, waves):
     n, k, group = 208, 2560, 128  # 13 row blocks: not a multiple of 2 or 4
     q, s, x = gen.make_linear(n, k, group, 16, seed=3)

@@ -26,9 +26,13 @@ def test_manifest_matches_kernel_sources():
     kdir = os.path.join(ROOT, "llm170_amd", "csrc", "kernels")
     for asset, syms in man.items():
         text = open(os.path.join(kdir, asset + ".hip")).read()
-        direct = re.findall(r'extern "C" __global__[^;{]*?\bvoid\s+(w4a16_\w+)\s*\(', text)
-        via_macro = re.findall(r"^[A-Z0-9_]+_KERNEL\((w4a16_\w+)", text, flags=re.M)
-        assert sorted(set(direct + via_macro)) == sorted(syms), asset
+        names = set(re.findall(r'extern "C" __global__[^;{]*?\bvoid\s+(w4a16_\w+)\s*\(', text))
+        # kernels stamped out by a *_KERNEL(NAME, ...) macro: one symbol per `void NAME` / `void NAME##suffix` in its body
+        for macro, body in re.findall(r"#define\s+([A-Z0-9_]+_KERNEL)\(NAME[^)]*\)((?:.*\\\n)*.*)", text):
+            suffixes = re.findall(r"\bvoid\s+NAME(?:##(\w+))?\s*\(", body)
+            for inst in re.findall(r"^%s\((w4a16_\w+)" % macro, text, flags=re.M):
+                names.update(inst + suf for suf in suffixes)
+        assert sorted(names) == sorted(syms), asset
         assert len(set(syms)) == len(syms)
     hips = sorted(f[:-4] for f in os.listdir(kdir) if f.endswith(".hip"))
     assert hips == sorted(man), "every kernel source is a manifest asset and vice versa"
