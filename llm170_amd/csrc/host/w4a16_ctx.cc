@@ -46,14 +46,18 @@ static const char* const kLayoutSyms[] = {"w4a16_tile_q",         "w4a16_tile_s"
                                           "w4a16_untile_s",       "w4a16_dump_tiled_f16",  "w4a16_dump_tiled_bf16",
                                           "w4a16_dump_raw_f16",   "w4a16_dump_raw_bf16",   nullptr};
 static const char* const kDecodeSyms[] = {
-    "w4a16_decode_g128_f16_rb1", "w4a16_decode_g128_f16_rb1_xl", "w4a16_decode_g128_f16_rb2",
-    "w4a16_decode_g128_f16_rb2_xl", "w4a16_decode_g128_f16_rb4", "w4a16_decode_g128_f16_rb4_xl",
-    "w4a16_decode_g128_bf16_rb1", "w4a16_decode_g128_bf16_rb1_xl", "w4a16_decode_g128_bf16_rb2",
-    "w4a16_decode_g128_bf16_rb2_xl", "w4a16_decode_g128_bf16_rb4", "w4a16_decode_g128_bf16_rb4_xl",
-    "w4a16_decode_g32_f16_rb1", "w4a16_decode_g32_f16_rb1_xl", "w4a16_decode_g32_f16_rb2",
-    "w4a16_decode_g32_f16_rb2_xl", "w4a16_decode_g32_f16_rb4", "w4a16_decode_g32_f16_rb4_xl",
-    "w4a16_decode_g32_bf16_rb1", "w4a16_decode_g32_bf16_rb1_xl", "w4a16_decode_g32_bf16_rb2",
-    "w4a16_decode_g32_bf16_rb2_xl", "w4a16_decode_g32_bf16_rb4", "w4a16_decode_g32_bf16_rb4_xl",
+    "w4a16_decode_g128_f16_rb1_x1", "w4a16_decode_g128_f16_rb1_x2", "w4a16_decode_g128_f16_rb1_x4",
+    "w4a16_decode_g128_f16_rb2_x1", "w4a16_decode_g128_f16_rb2_x2", "w4a16_decode_g128_f16_rb2_x4",
+    "w4a16_decode_g128_f16_rb4_x1", "w4a16_decode_g128_f16_rb4_x2", "w4a16_decode_g128_f16_rb4_x4",
+    "w4a16_decode_g128_bf16_rb1_x1", "w4a16_decode_g128_bf16_rb1_x2", "w4a16_decode_g128_bf16_rb1_x4",
+    "w4a16_decode_g128_bf16_rb2_x1", "w4a16_decode_g128_bf16_rb2_x2", "w4a16_decode_g128_bf16_rb2_x4",
+    "w4a16_decode_g128_bf16_rb4_x1", "w4a16_decode_g128_bf16_rb4_x2", "w4a16_decode_g128_bf16_rb4_x4",
+    "w4a16_decode_g32_f16_rb1_x1", "w4a16_decode_g32_f16_rb1_x2", "w4a16_decode_g32_f16_rb1_x4",
+    "w4a16_decode_g32_f16_rb2_x1", "w4a16_decode_g32_f16_rb2_x2", "w4a16_decode_g32_f16_rb2_x4",
+    "w4a16_decode_g32_f16_rb4_x1", "w4a16_decode_g32_f16_rb4_x2", "w4a16_decode_g32_f16_rb4_x4",
+    "w4a16_decode_g32_bf16_rb1_x1", "w4a16_decode_g32_bf16_rb1_x2", "w4a16_decode_g32_bf16_rb1_x4",
+    "w4a16_decode_g32_bf16_rb2_x1", "w4a16_decode_g32_bf16_rb2_x2", "w4a16_decode_g32_bf16_rb2_x4",
+    "w4a16_decode_g32_bf16_rb4_x1", "w4a16_decode_g32_bf16_rb4_x2", "w4a16_decode_g32_bf16_rb4_x4",
     nullptr};
 static const char* const kUtilSyms[] = {"w4a16_fill0_u32", "w4a16_copy_u4", nullptr};
 

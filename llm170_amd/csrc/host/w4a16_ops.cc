@@ -64,15 +64,14 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     if (L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
         return w4_fail(W4A16_ERR_SHAPE, "decode: tiled weights of 2 GiB or more exceed the buffer-descriptor range");
     // x goes through LDS when it fits beside a second resident workgroup (kernels/decode.hip, XLDS variants)
-    const size_t x_lds = t * (L.k + 32) * 2;
-    const bool xl = x_lds <= 64 * 1024;
+    // x loads per k tile: one serves up to 4 token rows, two up to 8, four up to 16 (kernels/decode.hip)
+    const int xl = t <= 4 ? 1 : t <= 8 ? 2 : 4;
     char sym[64];
-    snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_rb%d%s", L.group, L.scale_bf16 ? "bf16" : "f16", rb, xl ? "_xl" : "");
+    snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_rb%d_x%d", L.group, L.scale_bf16 ? "bf16" : "f16", rb, xl);
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of};
     unsigned shmem = waves > 1 ? (unsigned)(waves * rb * 64 * 16) : 0;
-    if (xl) shmem = std::max(shmem, (unsigned)x_lds);
     return w4_launch(ctx, sym, ceil_div(L.row_blocks, (size_t)rb), 1, (unsigned)(waves * 64), shmem, params);
 }
 

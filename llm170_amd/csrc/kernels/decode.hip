@@ -6,11 +6,11 @@
 //   * the int4 -> f16 unpack is 9 VALU ops per 8 weights and stays in registers; the multiply-accumulate runs on
 //     the matrix core: dword w of the 64 lanes is the A operand of v_mfma_f32_16x16x32_f16 (16 rows x 32 k), the
 //     B operand is x (32 k x 16 token columns), so t = 1 and t = 16 cost the same arithmetic;
-//   * x: every vector-memory instruction costs the CU's address unit about as much as a full 1 KiB load, however few
-//     lanes are live, so four B-operand loads per k tile would cost more than the weight stream itself.  When
-//     t*k*2 bytes fit (XLDS variants, the normal case for t <= 4) the workgroup copies x into LDS once and the
-//     B operands come from ds_read_b128; token columns >= t read a duplicate row (their results are never stored).
-//     Otherwise x comes from raw buffer loads whose offset is out of range for columns >= t (zeros, no traffic);
+//   * x: every vector-memory instruction costs the CU's address unit about as much as a full 1 KiB load however few
+//     lanes are live, so one B-operand load per MFMA would cost more than the weight stream.  For t <= 4 a single
+//     buffer load per k tile brings all four 32-k chunks (lane m fetches chunk m/4 of token m%4; lanes for tokens
+//     >= t are out of range: zeros, no traffic) and v_mov_b32_dpp row_shl moves chunk c to the token's column;
+//     t <= 8 takes two loads, t <= 16 four (no shuffles).  No LDS and no barrier on the streaming path;
 //   * weights enter the MFMA as exact integers; the per-group scale multiplies the f32 group sum, so no weight is
 //     ever rounded to f16 (error vs the f32 lane contract is summation order only);
 //   * each wave keeps DEPTH k-tiles of loads in flight (register ring, software pipelined);
@@ -19,49 +19,47 @@
 //     launch).  The host picks RB and W.
 #include "w4a16_common.hpp"
 
-template <int G, int RB>
+// One pipeline stage = the loads of one k tile: RB weight tiles, their scales, and XL loads of x.
+template <int G, int RB, int XL>
 struct DecodeStage {
     u4_t q[RB];
     u2_t s[RB][W4_TILE_K / G];
-    u4_t x[4];
+    u4_t x[XL];
 };
 
-#define W4_XLDS_PAD 32  // halves of padding per x row in LDS (rows land 16 banks apart)
+// Data of lane (i + SH) of the same 16-lane row (zero past the row end): v_mov_b32_dpp row_shl.
+template <int SH>
+__device__ __forceinline__ u4_t w4_row_shl(u4_t v) {
+    u4_t r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = __builtin_amdgcn_update_dpp(0u, v[i], 0x100 + SH, 0xF, 0xF, true);
+    return r;
+}
 
-template <int G, bool SBF, int RB, int DEPTH, bool XLDS>
+// XL = vector loads of x per k tile: 1 serves t <= 4, 2 serves t <= 8, 4 serves t <= 16.
+template <int G, bool SBF, int RB, int DEPTH, int XL>
 __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                             const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
                                             int k, int n, int t, int out_f16) {
-    extern __shared__ f4_t red[];  // [W][RB][64] partial tiles; XLDS: first holds x as halves [t][k + W4_XLDS_PAD]
+    extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
+    constexpr int C = 4 / XL;           // 32-k chunks (MFMAs) served by one x load
+    constexpr int TPL = 16 / C;         // token columns served by one x load
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, W = blockDim.x >> 6;
     const int kt_n = k / W4_TILE_K;
     const int kg_n = kt_n * GPT;
     const int nb0 = blockIdx.x * RB;
     const int kt0 = (kt_n * wave) / W, kt1 = (kt_n * (wave + 1)) / W;
     const int m = lane & 15, g = lane >> 4;
-    const bool xact = m < t;
-    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)t * (unsigned)k * 2u);
-    const unsigned xoff = xact ? ((unsigned)m * (unsigned)k + (unsigned)g * 8u) * 2u : W4_OOB;
 
-    const int xstride = k + W4_XLDS_PAD;
-    if (XLDS) {
-        // cooperative copy of x into LDS, 16 B per thread per step
-        _Float16* xs = reinterpret_cast<_Float16*>(red);
-        const int chunks_per_row = k / 8;
-        for (int c = threadIdx.x; c < t * chunks_per_row; c += blockDim.x) {
-            const int row = c / chunks_per_row, col = (c - row * chunks_per_row) * 8;
-            *reinterpret_cast<u4_t*>(xs + row * xstride + col) =
-                *reinterpret_cast<const u4_t*>(x + (size_t)row * k + col);
-        }
-        __syncthreads();
-    }
-    const _Float16* xl = reinterpret_cast<const _Float16*>(red) + min(m, t - 1) * xstride + g * 8;
-
-    // Every load is a raw buffer load: a k tile at or past kt1 gets an out-of-range offset, returns zeros and costs no
-    // memory traffic, so the pipeline needs no branch around its prefetches.
+    // Every load is a raw buffer load: an out-of-range offset returns zeros and costs no memory traffic, which
+    // predicates tiles past kt1 and token columns >= t without a branch.
     const __amdgpu_buffer_rsrc_t qr = w4_make_rsrc(qt, (unsigned)row_blocks * (unsigned)kt_n * 1024u);
     const __amdgpu_buffer_rsrc_t sr = w4_make_rsrc(st, (unsigned)row_blocks * (unsigned)kg_n * 32u);
+    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)t * (unsigned)k * 2u);
+    // x load l of a tile: lane (m, g) fetches, for token m % TPL, the 8 halves of chunk l*C + m / TPL at k offset g*8
+    const int xtok = m % TPL, xchunk = m / TPL;
+    const unsigned xoff = xtok < t ? ((unsigned)xtok * (unsigned)k + (unsigned)(xchunk * 32 + g * 8)) * 2u : W4_OOB;
     f4_t acc[RB];
     unsigned qoff[RB], soff[RB];
 #pragma unroll
@@ -72,8 +70,8 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
         soff[rb] = nb * (unsigned)kg_n * 32u + (unsigned)g * 8u;
     }
 
-    DecodeStage<G, RB> stage[DEPTH];
-    auto load = [&](DecodeStage<G, RB>& s_, int kt) {
+    DecodeStage<G, RB, XL> stage[DEPTH];
+    auto load = [&](DecodeStage<G, RB, XL>& s_, int kt) {
         const bool live = kt < kt1;
 #pragma unroll
         for (int rb = 0; rb < RB; rb++)
@@ -85,17 +83,22 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
             for (int gi = 0; gi < GPT; gi++)
                 s_.s[rb][gi] = __builtin_amdgcn_raw_buffer_load_b64(
                     sr, live ? soff[rb] + (unsigned)(kt * GPT + gi) * 32u : W4_OOB, 0, 0);
-        if (!XLDS) {
 #pragma unroll
-            for (int w = 0; w < 4; w++)
-                s_.x[w] = __builtin_amdgcn_raw_buffer_load_b128(
-                    xr, live ? xoff + (unsigned)(kt * W4_TILE_K + w * 32) * 2u : W4_OOB, 0, 0);
-        }
+        for (int l = 0; l < XL; l++)
+            s_.x[l] = __builtin_amdgcn_raw_buffer_load_b128(
+                xr, live ? xoff + (unsigned)(kt * W4_TILE_K + l * C * 32) * 2u : W4_OOB, 0, 0);
     };
-    auto compute = [&](DecodeStage<G, RB>& s_, int kt) {
-        if (XLDS) {
+    auto compute = [&](const DecodeStage<G, RB, XL>& s_) {
+        // B operand of MFMA w = chunk w of x for token column m: held by lane (m + (w % C) * TPL) of load w / C
+        u4_t xb[4];
 #pragma unroll
-            for (int w = 0; w < 4; w++) s_.x[w] = *reinterpret_cast<const u4_t*>(xl + kt * W4_TILE_K + w * 32);
+        for (int l = 0; l < XL; l++) {
+            xb[l * C] = s_.x[l];
+            if (C >= 2) xb[l * C + 1] = w4_row_shl<TPL>(s_.x[l]);
+            if (C == 4) {
+                xb[2] = w4_row_shl<2 * TPL>(s_.x[l]);
+                xb[3] = w4_row_shl<3 * TPL>(s_.x[l]);
+            }
         }
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
@@ -104,7 +107,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
 #pragma unroll
                 for (int w = 0; w < 4; w++)
                     part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
-                                                                  __builtin_bit_cast(h8_t, s_.x[w]), part, 0, 0, 0);
+                                                                  __builtin_bit_cast(h8_t, xb[w]), part, 0, 0, 0);
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     acc[rb][i] += w4_scale_fast<SBF>((s_.s[rb][0][i >> 1] >> (16 * (i & 1))) & 0xFFFFu) * part[i];
@@ -113,7 +116,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                 for (int w = 0; w < 4; w++) {
                     f4_t part = {0.f, 0.f, 0.f, 0.f};
                     part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
-                                                                  __builtin_bit_cast(h8_t, s_.x[w]), part, 0, 0, 0);
+                                                                  __builtin_bit_cast(h8_t, xb[w]), part, 0, 0, 0);
 #pragma unroll
                     for (int i = 0; i < 4; i++)
                         acc[rb][i] +=
@@ -124,15 +127,15 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     };
 
     // One counted loop does the pipeline fill (round -1, compute skipped) and the steady state, so on every path
-    // into a stage's compute the outstanding loads are in ring order and the wait can be "all but the younger stages'
-    // loads" (s_waitcnt vmcnt(N > 0)).  Tiles past kt1 load zeros (scale 0 => no contribution); the last partial
-    // round is finished by the unrolled tail below.  The scheduling barriers keep each stage's loads together.
+    // into a stage's compute the outstanding loads are in ring order and the wait can leave the younger stages' loads
+    // in flight (s_waitcnt vmcnt(N > 0)).  Tiles past kt1 load zeros and are never computed; the last partial round
+    // is finished by the unrolled tail.  The scheduling barriers keep each stage's loads together.
     const int tiles = kt1 - kt0;
     const int rounds = tiles / DEPTH;
     for (int r = -1; r < rounds; r++) {
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
-            if (r >= 0) compute(stage[d], kt0 + r * DEPTH + d);
+            if (r >= 0) compute(stage[d]);
             __builtin_amdgcn_sched_barrier(0);
             load(stage[d], kt0 + (r + 1) * DEPTH + d);
             __builtin_amdgcn_sched_barrier(0);
@@ -140,10 +143,9 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     }
 #pragma unroll
     for (int d = 0; d < DEPTH - 1; d++)
-        if (rounds * DEPTH + d < tiles) compute(stage[d], kt0 + rounds * DEPTH + d);
+        if (rounds * DEPTH + d < tiles) compute(stage[d]);
 
     if (W > 1) {
-        if (XLDS) __syncthreads();  // everyone is done reading x before the partial tiles overwrite it
         if (wave != 0) {
 #pragma unroll
             for (int rb = 0; rb < RB; rb++) red[(wave * RB + rb) * 64 + lane] = acc[rb];
@@ -155,7 +157,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
             for (int rb = 0; rb < RB; rb++) acc[rb] += red[(w * RB + rb) * 64 + lane];
         }
     }
-    if (!xact) return;
+    if (m >= t) return;
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
         if (nb0 + rb >= row_blocks) break;
@@ -183,27 +185,28 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     }
 }
 
-#define DECODE_KERNEL(NAME, G, SBF, RB, DEPTH)                                                                 \
-    extern "C" __global__ __launch_bounds__(512) void NAME(const u4_t* qt, const uint16_t* st, const uint16_t* x, \
-                                                           void* y, int row_blocks, int k, int n, int t,          \
-                                                           int out_f16) {                                         \
-        decode_body<G, SBF, RB, DEPTH, false>(qt, st, x, y, row_blocks, k, n, t, out_f16);                        \
-    }                                                                                                             \
-    extern "C" __global__ __launch_bounds__(512) void NAME##_xl(const u4_t* qt, const uint16_t* st,               \
-                                                                const uint16_t* x, void* y, int row_blocks,       \
-                                                                int k, int n, int t, int out_f16) {               \
-        decode_body<G, SBF, RB, DEPTH, true>(qt, st, x, y, row_blocks, k, n, t, out_f16);                         \
-    }
+// ring depth: as many stages as ~96 VGPRs of load buffers allow
+#define DECODE_DEPTH(G, RB, XL) \
+    ((96 / (4 * RB + 2 * RB * (W4_TILE_K / G) + 4 * XL)) < 2 ? 2 : (96 / (4 * RB + 2 * RB * (W4_TILE_K / G) + 4 * XL)) > 8 ? 8 : (96 / (4 * RB + 2 * RB * (W4_TILE_K / G) + 4 * XL)))
 
-DECODE_KERNEL(w4a16_decode_g128_f16_rb1, 128, false, 1, 4)
-DECODE_KERNEL(w4a16_decode_g128_f16_rb2, 128, false, 2, 3)
-DECODE_KERNEL(w4a16_decode_g128_f16_rb4, 128, false, 4, 2)
-DECODE_KERNEL(w4a16_decode_g32_f16_rb1, 32, false, 1, 3)
-DECODE_KERNEL(w4a16_decode_g32_f16_rb2, 32, false, 2, 2)
-DECODE_KERNEL(w4a16_decode_g32_f16_rb4, 32, false, 4, 2)
-DECODE_KERNEL(w4a16_decode_g128_bf16_rb1, 128, true, 1, 4)
-DECODE_KERNEL(w4a16_decode_g128_bf16_rb2, 128, true, 2, 3)
-DECODE_KERNEL(w4a16_decode_g128_bf16_rb4, 128, true, 4, 2)
-DECODE_KERNEL(w4a16_decode_g32_bf16_rb1, 32, true, 1, 3)
-DECODE_KERNEL(w4a16_decode_g32_bf16_rb2, 32, true, 2, 2)
-DECODE_KERNEL(w4a16_decode_g32_bf16_rb4, 32, true, 4, 2)
+#define DECODE_KERNEL_X(NAME, G, SBF, RB, XL)                                                                        \
+    extern "C" __global__ __launch_bounds__(512) void NAME##_x##XL(const u4_t* qt, const uint16_t* st,               \
+                                                                   const uint16_t* x, void* y, int row_blocks,       \
+                                                                   int k, int n, int t, int out_f16) {               \
+        decode_body<G, SBF, RB, DECODE_DEPTH(G, RB, XL), XL>(qt, st, x, y, row_blocks, k, n, t, out_f16);            \
+    }
+#define DECODE_KERNEL(NAME, G, SBF, RB) \
+    DECODE_KERNEL_X(NAME, G, SBF, RB, 1) DECODE_KERNEL_X(NAME, G, SBF, RB, 2) DECODE_KERNEL_X(NAME, G, SBF, RB, 4)
+
+DECODE_KERNEL(w4a16_decode_g128_f16_rb1, 128, false, 1)
+DECODE_KERNEL(w4a16_decode_g128_f16_rb2, 128, false, 2)
+DECODE_KERNEL(w4a16_decode_g128_f16_rb4, 128, false, 4)
+DECODE_KERNEL(w4a16_decode_g32_f16_rb1, 32, false, 1)
+DECODE_KERNEL(w4a16_decode_g32_f16_rb2, 32, false, 2)
+DECODE_KERNEL(w4a16_decode_g32_f16_rb4, 32, false, 4)
+DECODE_KERNEL(w4a16_decode_g128_bf16_rb1, 128, true, 1)
+DECODE_KERNEL(w4a16_decode_g128_bf16_rb2, 128, true, 2)
+DECODE_KERNEL(w4a16_decode_g128_bf16_rb4, 128, true, 4)
+DECODE_KERNEL(w4a16_decode_g32_bf16_rb1, 32, true, 1)
+DECODE_KERNEL(w4a16_decode_g32_bf16_rb2, 32, true, 2)
+DECODE_KERNEL(w4a16_decode_g32_bf16_rb4, 32, true, 4)

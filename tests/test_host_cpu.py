@@ -20,6 +20,36 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(ffi.declared_symbols())
 
 
+def expand_kernel_macros(text):
+    """Kernel names produced by function-like macros whose body contains `extern "C" __global__ ... void NAME...(`;
+    macros may call other macros and paste suffixes with ##."""
+    text = re.sub(r"\\\n", " ", text)
+    macros = {}
+    for m in re.finditer(r"^#define\s+(\w+)\(([^)]*)\)\s+(.*)$", text, flags=re.M):
+        macros[m.group(1)] = ([a.strip() for a in m.group(2).split(",")], m.group(3))
+    body_lines = [ln for ln in text.split("\n") if not ln.startswith("#define")]
+
+    def expand(line, depth=0):
+        out = line
+        for name, (params, body) in macros.items():
+            for call in list(re.finditer(r"\b%s\(([^()]*)\)" % name, out)):
+                args = [a.strip() for a in call.group(1).split(",")]
+                if len(args) != len(params):
+                    continue
+                rep = body
+                for p_, a_ in zip(params, args):
+                    rep = re.sub(r"\b%s\b" % p_, a_, rep)
+                rep = re.sub(r"\s*##\s*", "", rep)
+                out = out.replace(call.group(0), rep)
+        return expand(out, depth + 1) if out != line and depth < 8 else out
+
+    names = set()
+    for ln in body_lines:
+        if re.match(r"^[A-Z0-9_]+\(", ln):
+            names.update(re.findall(r'__global__[^;{]*?\bvoid\s+(w4a16_\w+)\s*\(', expand(ln)))
+    return names
+
+
 def test_manifest_matches_kernel_sources():
     """Precedent: manifest symbols == extern "C" __global__ symbols of the .cu files (assets.rs:394-443)."""
     man = ffi.manifest()
@@ -27,11 +57,8 @@ def test_manifest_matches_kernel_sources():
     for asset, syms in man.items():
         text = open(os.path.join(kdir, asset + ".hip")).read()
         names = set(re.findall(r'extern "C" __global__[^;{]*?\bvoid\s+(w4a16_\w+)\s*\(', text))
-        # kernels stamped out by a *_KERNEL(NAME, ...) macro: one symbol per `void NAME` / `void NAME##suffix` in its body
-        for macro, body in re.findall(r"#define\s+([A-Z0-9_]+_KERNEL)\(NAME[^)]*\)((?:.*\\\n)*.*)", text):
-            suffixes = re.findall(r"\bvoid\s+NAME(?:##(\w+))?\s*\(", body)
-            for inst in re.findall(r"^%s\((w4a16_\w+)" % macro, text, flags=re.M):
-                names.update(inst + suf for suf in suffixes)
+        # kernels stamped out by macros: expand `#define M(...) body` textually until only `void <name>(` remain
+        names |= expand_kernel_macros(text)
         assert sorted(names) == sorted(syms), asset
         assert len(set(syms)) == len(syms)
     hips = sorted(f[:-4] for f in os.listdir(kdir) if f.endswith(".hip"))
