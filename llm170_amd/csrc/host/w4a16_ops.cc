@@ -39,17 +39,16 @@ static int launch_lane(w4a16_ctx* ctx, uint64_t q, uint64_t s, uint64_t x, uint6
     return w4_launch(ctx, sym, ceil_div(n, 4), ceil_div(t, 8), 256, 0, params);
 }
 
+// Launch shape of the row-block decode kernel.  Measured on MI355X at the 27B layer shapes: two row blocks per
+// wave and four waves per block (in-block split-K by 4) is best or within 2 % of best for t <= 8 and for narrow
+// outputs; for 9..16 token rows on wide outputs four row blocks per wave halve the x operand traffic.
 static int pick_decode_shape(const w4a16_ctx* ctx, const W4Lin& L, size_t t, int* rb_out, int* waves_out) {
-    int rb = ctx->decode_rows_per_wave ? ctx->decode_rows_per_wave / 16 : (t <= 4 ? 2 : 4);
+    const bool wide16 = t > 8 && L.row_blocks >= 1024;
+    int rb = ctx->decode_rows_per_wave ? ctx->decode_rows_per_wave / 16 : (wide16 ? 4 : 2);
     if (rb != 1 && rb != 2 && rb != 4) return w4_fail(W4A16_ERR_ARG, "decode: rows_per_wave must be 16, 32 or 64");
     while (rb > 1 && L.row_blocks < (size_t)rb) rb >>= 1;
     const int kt_n = (int)(L.k / 128);
-    int waves = ctx->decode_waves_per_block;
-    if (waves == 0) {
-        // aim at ~8 KiB of weights per wave (measured best for a read-once stream on MI355X)
-        const int tiles_per_wave = std::max(1, 8 / rb);
-        waves = (kt_n + tiles_per_wave - 1) / tiles_per_wave;
-    }
+    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : (wide16 ? 2 : 4);
     waves = std::max(1, std::min(std::min(waves, 8), kt_n));
     *rb_out = rb;
     *waves_out = waves;
@@ -63,7 +62,6 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     W4_TRY(pick_decode_shape(ctx, L, t, &rb, &waves));
     if (L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
         return w4_fail(W4A16_ERR_SHAPE, "decode: tiled weights of 2 GiB or more exceed the buffer-descriptor range");
-    // x goes through LDS when it fits beside a second resident workgroup (kernels/decode.hip, XLDS variants)
     // x loads per k tile: one serves up to 4 token rows, two up to 8, four up to 16 (kernels/decode.hip)
     const int xl = t <= 4 ? 1 : t <= 8 ? 2 : 4;
     char sym[64];

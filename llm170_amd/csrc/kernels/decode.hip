@@ -45,7 +45,9 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
     constexpr int C = 4 / XL;           // 32-k chunks (MFMAs) served by one x load
     constexpr int TPL = 16 / C;         // token columns served by one x load
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, W = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, W = blockDim.x >> 6;
+    // the wave index is uniform across the wave: keep it (and everything derived from it) in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kt_n = k / W4_TILE_K;
     const int kg_n = kt_n * GPT;
     const int nb0 = blockIdx.x * RB;
