@@ -59,6 +59,8 @@ static const char* const kDecodeSyms[] = {
     "w4a16_decode_g32_bf16_rb2_x1", "w4a16_decode_g32_bf16_rb2_x2", "w4a16_decode_g32_bf16_rb2_x4",
     "w4a16_decode_g32_bf16_rb4_x1", "w4a16_decode_g32_bf16_rb4_x2", "w4a16_decode_g32_bf16_rb4_x4",
     nullptr};
+static const char* const kPrefillSyms[] = {"w4a16_prefill_g128_f16", "w4a16_prefill_g128_bf16", "w4a16_prefill_g32_f16",
+                                           "w4a16_prefill_g32_bf16", nullptr};
 static const char* const kUtilSyms[] = {"w4a16_fill0_u32", "w4a16_copy_u4", nullptr};
 
 struct W4Asset {
@@ -69,6 +71,7 @@ static const W4Asset kAssets[] = {
     {"lane", kLaneSyms},
     {"layout", kLayoutSyms},
     {"decode", kDecodeSyms},
+    {"prefill", kPrefillSyms},
     {"util", kUtilSyms},
 };
 static const size_t kAssetCount = sizeof kAssets / sizeof kAssets[0];

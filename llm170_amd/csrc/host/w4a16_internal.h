@@ -20,6 +20,7 @@ struct W4Lin {
     size_t n = 0, k = 0, group = 0;
     int scale_bf16 = 0;
     size_t row_blocks = 0;
+    bool scales_regular = true;  // every scale finite and non-zero (the MFMA prefill kernel divides by them)
 };
 
 struct w4a16_event {

@@ -73,6 +73,33 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     return w4_launch(ctx, sym, ceil_div(L.row_blocks, (size_t)rb), 1, (unsigned)(waves * 64), shmem, params);
 }
 
+// Prefill GEMM (kernels/prefill.hip): 256 x 256 block tiles, 8 waves, grid padded to a multiple of 8 so that block
+// b % 8 (the XCD it lands on) owns a contiguous run of tiles.
+static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16) {
+    if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has no tiled copy (needs k %% 128 == 0)");
+    if (!L.scales_regular)
+        return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has a zero or non-finite scale (use the decode path)");
+    if (t * L.k * 2 >= 0x80000000ull || L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
+        return w4_fail(W4A16_ERR_SHAPE, "prefill: x or the tiled weights reach 2 GiB, beyond the buffer-descriptor range");
+    const size_t tiles = ((t + 255) / 256) * ((L.n + 255) / 256);
+    const size_t per_xcd = (tiles + 7) / 8;
+    char sym[64];
+    snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s", L.group, L.scale_bf16 ? "bf16" : "f16");
+    uint64_t qt = L.q_tiled, st = L.s_tiled;
+    int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
+    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of};
+    return w4_launch(ctx, sym, (unsigned)(per_xcd * 8), 1, 512, 2 * 256 * 72 * 2, params);
+}
+
+// t > 16 without the prefill kernel (irregular scales): the decode kernel over chunks of 16 rows.
+static int launch_decode_chunked(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16) {
+    for (size_t t0 = 0; t0 < t; t0 += 16) {
+        const size_t tc = std::min<size_t>(16, t - t0);
+        W4_TRY(launch_decode(ctx, L, x + t0 * L.k * 2, y + t0 * L.n * (out_f16 ? 2 : 4), tc, out_f16));
+    }
+    return 0;
+}
+
 // ------------------------------------------------------------------------------------------------ Gptq4::gemm
 extern "C" int w4a16_gemm_host(w4a16_ctx* ctx, const uint16_t* x_f16, size_t t, const uint32_t* q, const uint16_t* s,
                                size_t n, size_t k, size_t group, int scale_bf16, float* out_f32) {
@@ -125,6 +152,18 @@ extern "C" int w4a16_upload_lin(w4a16_ctx* ctx, const char* name, const void* q,
     L.k = k;
     L.group = group;
     L.scale_bf16 = scale_bf16 ? 1 : 0;
+    {
+        const uint16_t* sp = static_cast<const uint16_t*>(s);
+        const size_t ns = slen_bytes / 2;
+        const unsigned expmask = scale_bf16 ? 0x7F80u : 0x7C00u;
+        for (size_t i = 0; i < ns; i++) {
+            const unsigned b = sp[i];
+            if ((b & 0x7FFFu) == 0 || (b & expmask) == expmask) {
+                L.scales_regular = false;
+                break;
+            }
+        }
+    }
     int rc = w4a16_alloc(ctx, qlen_bytes, &L.q_raw);
     if (!rc) rc = w4a16_alloc(ctx, slen_bytes, &L.s_raw);
     if (!rc) rc = w4a16_h2d(ctx, L.q_raw, q, qlen_bytes);
@@ -197,8 +236,12 @@ extern "C" int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_de
     if (path == W4A16_PATH_AUTO) {
         if (!L->q_tiled)
             path = W4A16_PATH_LANE;
+        else if (t <= 16)
+            path = W4A16_PATH_DECODE;
+        else if (L->scales_regular)
+            path = W4A16_PATH_PREFILL;
         else
-            path = t <= 16 ? W4A16_PATH_DECODE : W4A16_PATH_PREFILL;
+            return launch_decode_chunked(ctx, *L, x_dev, y_dev, t, out_f16);
     }
     switch (path) {
         case W4A16_PATH_LANE:
@@ -208,7 +251,7 @@ extern "C" int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_de
         case W4A16_PATH_DECODE:
             return launch_decode(ctx, *L, x_dev, y_dev, t, out_f16);
         case W4A16_PATH_PREFILL:
-            return w4_fail(W4A16_ERR_UNSUPPORTED, "lin_forward %s: prefill path not built", name);
+            return launch_prefill(ctx, *L, x_dev, y_dev, t, out_f16);
         default:
             return w4_fail(W4A16_ERR_ARG, "lin_forward %s: unknown path %d", name, path);
     }

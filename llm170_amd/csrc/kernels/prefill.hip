@@ -1,0 +1,190 @@
+// Prefill regime (t > 16 activation rows): tiled GEMM  y[t][n] = x[t][k] * W^T  on v_mfma_f32_32x32x16_f16.
+// Role of the reference's prefill path gemm_launch -> marlin_gemm_try / w4a16_gemm_g128_mma
+// (w4a16_dec/kernels/gemm.rs:4-51, kernels/marlin.rs:94-213, assets/gptq4.cu:984-1147), designed for CDNA4:
+//   * workgroup = 8 waves (2 along m x 4 along n), block tile 256 (m) x 256 (n), wave tile 128 x 64 = 4 x 2 MFMA tiles
+//     of 32 x 32 with f32 accumulators in arch VGPRs (128 registers), two waves per SIMD;
+//   * x (the A operand) is staged through LDS in k slabs of 64, double buffered, rows padded to 72 halves so the
+//     ds_read_b128 fragment reads are bank-conflict free; rows >= t come from out-of-range buffer loads (zeros);
+//   * the weights (B operand) never touch LDS: the tiled layout of w4a16_common.hpp already is the MFMA B layout —
+//     lane (n = l % 32, khalf = l / 32) reads 16 B of tile lane g = 2h + khalf, r = n % 16 of its row block, dword w of
+//     which is the k16 block (w, h) of the k tile — so each wave fetches its 64 x 128 weights with four coalesced
+//     dwordx4 loads per k tile (one k tile ahead) and unpacks them in registers (9 VALU ops per MFMA operand);
+//   * weights enter the MFMA as exact integers.  The per-group scale is carried as a running unit: the accumulator
+//     holds sum / s_g; at each group boundary it is multiplied by s_prev / s_cur and the new group's integer products
+//     are added by the MFMA itself; the epilogue multiplies by the last scale.  No weight is rounded to f16 and no
+//     second accumulator set is needed.  (Linears with a zero or non-finite scale are not routed here.)
+//   * workgroups are numbered so that each XCD works on a contiguous run of n tiles, m fastest: the sixteen m tiles
+//     that share a weight panel run on the same L2.
+#include "w4a16_common.hpp"
+
+#define PF_BM 256
+#define PF_BN 256
+#define PF_KS 64          // k per LDS stage
+#define PF_LDA 72         // halves per staged x row (64 + 8 padding)
+#define PF_THREADS 512
+
+template <int G, bool SBF>
+__device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
+                                             const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
+                                             int k, int n, int t, int out_f16) {
+    extern __shared__ _Float16 lds[];  // 2 stages x [PF_BM][PF_LDA]
+    constexpr int GPT = W4_TILE_K / G;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & 1, wn = wave >> 1;  // 2 x 4 waves
+    const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
+
+    // XCD-aware tile numbering: block b runs on XCD b % 8; give each XCD a contiguous run of tiles, m fastest.
+    const int tiles_m = (t + PF_BM - 1) / PF_BM, tiles_n = (n + PF_BN - 1) / PF_BN;
+    const int n_tiles = tiles_m * tiles_n;
+    const int per_xcd = (n_tiles + 7) / 8;
+    const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per_xcd || tile >= n_tiles) return;  // uniform for the whole block
+    const int m0 = (tile % tiles_m) * PF_BM, n0 = (tile / tiles_m) * PF_BN;
+
+    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)t * (unsigned)k * 2u);
+    const __amdgpu_buffer_rsrc_t qr = w4_make_rsrc(qt, (unsigned)row_blocks * (unsigned)kt_n * 1024u);
+    const __amdgpu_buffer_rsrc_t sr = w4_make_rsrc(st, (unsigned)row_blocks * (unsigned)kg_n * 32u);
+
+    // ---- x staging: 256 rows x 64 k per stage = 2048 chunks of 16 B, 4 per thread
+    unsigned xa_off[4];
+    int xa_lds[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int c = tid + i * PF_THREADS, row = c >> 3, col = (c & 7) * 8;
+        xa_off[i] = (m0 + row < t) ? ((unsigned)(m0 + row) * (unsigned)k + (unsigned)col) * 2u : W4_OOB;
+        xa_lds[i] = row * PF_LDA + col;
+    }
+    u4_t xa[4];
+    auto load_a = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            xa[i] = __builtin_amdgcn_raw_buffer_load_b128(xr, xa_off[i] + (unsigned)s * (PF_KS * 2u), 0, 0);  // an out-of-range row stays out of range
+    };
+    auto store_a = [&](int buf) {
+        _Float16* base = lds + buf * (PF_BM * PF_LDA);
+#pragma unroll
+        for (int i = 0; i < 4; i++) *reinterpret_cast<u4_t*>(base + xa_lds[i]) = xa[i];
+    };
+
+    // ---- weights: lane (nl = l % 32, khalf = l / 32); per n sub-tile ni and half h one dwordx4 per k tile
+    const int nl = lane & 31, khalf = lane >> 5;
+    unsigned q_off[2][2], s_off[2];
+#pragma unroll
+    for (int ni = 0; ni < 2; ni++) {
+        const int nrow = n0 + wn * 64 + ni * 32 + nl;
+        const unsigned rb = (unsigned)min(nrow >> 4, row_blocks - 1);  // rows past n re-read the last block, never stored
+        const unsigned r = (unsigned)(nrow & 15);
+#pragma unroll
+        for (int h = 0; h < 2; h++) q_off[ni][h] = (rb * (unsigned)kt_n * 64u + (unsigned)(2 * h + khalf) * 16u + r) * 16u;
+        s_off[ni] = (rb * (unsigned)kg_n * 16u + r) * 2u;
+    }
+    u4_t bq[2][2], bqn[2][2];
+    unsigned sc[2][GPT], scn[2][GPT];
+    auto load_b = [&](u4_t (&dst)[2][2], unsigned (&sdst)[2][GPT], int kt) {
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++) {
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                dst[ni][h] = __builtin_amdgcn_raw_buffer_load_b128(qr, q_off[ni][h] + (unsigned)kt * 1024u, 0, 0);
+#pragma unroll
+            for (int gi = 0; gi < GPT; gi++)
+                sdst[ni][gi] = __builtin_amdgcn_raw_buffer_load_b16(sr, s_off[ni] + (unsigned)(kt * GPT + gi) * 32u, 0, 0);
+        }
+    };
+
+    f16_t acc[4][2];
+#pragma unroll
+    for (int mi = 0; mi < 4; mi++)
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[mi][ni][e] = 0.f;
+    float unit[2] = {1.f, 1.f};  // scale the accumulator of sub-tile ni is currently expressed in
+
+    const int a_row = wm * 128 + nl;  // + mi * 32
+    const int stages = k / PF_KS;
+
+    load_a(0);
+    load_b(bq, sc, 0);
+    store_a(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < kt_n; kt++) {
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int s = kt * 2 + half;
+            if (s + 1 < stages) load_a(s + 1);
+            if (half == 0 && kt + 1 < kt_n) load_b(bqn, scn, kt + 1);
+            const _Float16* abuf = lds + (s & 1) * (PF_BM * PF_LDA) + a_row * PF_LDA + khalf * 8;
+#pragma unroll
+            for (int kbl = 0; kbl < 4; kbl++) {
+                const int kb = half * 4 + kbl, w = kb >> 1, h = kb & 1;
+                // group boundary: re-express the accumulators in the new group's scale
+                if ((G == 128 && kb == 0) || (G == 32 && h == 0)) {
+#pragma unroll
+                    for (int ni = 0; ni < 2; ni++) {
+                        const float s_cur = w4_scale_fast<SBF>(sc[ni][G == 128 ? 0 : w]);
+                        const float ratio = unit[ni] / s_cur;
+                        unit[ni] = s_cur;
+#pragma unroll
+                        for (int mi = 0; mi < 4; mi++) acc[mi][ni] *= ratio;
+                    }
+                }
+                h8_t a[4];
+#pragma unroll
+                for (int mi = 0; mi < 4; mi++)
+                    a[mi] = *reinterpret_cast<const h8_t*>(abuf + mi * 32 * PF_LDA + kbl * 16);
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) {
+                    const h8_t b = w4_deq8(bq[ni][h][w]);
+#pragma unroll
+                    for (int mi = 0; mi < 4; mi++)
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b, acc[mi][ni], 0, 0, 0);
+                }
+            }
+            if (s + 1 < stages) store_a((s + 1) & 1);
+            __syncthreads();
+        }
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) bq[ni][h] = bqn[ni][h];
+#pragma unroll
+            for (int gi = 0; gi < GPT; gi++) sc[ni][gi] = scn[ni][gi];
+        }
+    }
+
+    // ---- epilogue: y[m][n] = acc * unit; D register e of lane (nl, khalf) is row 8*(e/4) + 4*khalf + e%4, column nl
+#pragma unroll
+    for (int ni = 0; ni < 2; ni++) {
+        const int col = n0 + wn * 64 + ni * 32 + nl;
+        if (col >= n) continue;
+#pragma unroll
+        for (int mi = 0; mi < 4; mi++) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int row = m0 + wm * 128 + mi * 32 + 8 * (e >> 2) + 4 * khalf + (e & 3);
+                if (row < t) {
+                    const float v = acc[mi][ni][e] * unit[ni];
+                    if (out_f16)
+                        reinterpret_cast<_Float16*>(y)[(size_t)row * n + col] = (_Float16)v;
+                    else
+                        reinterpret_cast<float*>(y)[(size_t)row * n + col] = v;
+                }
+            }
+        }
+    }
+}
+
+#define PREFILL_KERNEL(NAME, G, SBF)                                                                               \
+    extern "C" __global__ __launch_bounds__(PF_THREADS) void NAME(const u4_t* qt, const uint16_t* st,              \
+                                                                  const uint16_t* x, void* y, int row_blocks,      \
+                                                                  int k, int n, int t, int out_f16) {              \
+        prefill_body<G, SBF>(qt, st, x, y, row_blocks, k, n, t, out_f16);                                          \
+    }
+
+PREFILL_KERNEL(w4a16_prefill_g128_f16, 128, false)
+PREFILL_KERNEL(w4a16_prefill_g128_bf16, 128, true)
+PREFILL_KERNEL(w4a16_prefill_g32_f16, 32, false)
+PREFILL_KERNEL(w4a16_prefill_g32_bf16, 32, true)

@@ -193,3 +193,67 @@ def test_error_paths(dec):
     assert dec.lin_spec("ok") == {"n": 16, "k": 256, "group": 128, "scale_bf16": False, "tiled": True, "raw": False}
     with pytest.raises(ops.W4a16Error):
         dec.gemv_host("ok", np.zeros((1, 256), np.uint16), path=ops.PATH_LANE)
+
+
+# ------------------------------------------------------------------ prefill regime (MFMA GEMM)
+def _device_forward(dec, name, x, t, path, out_f16=False):
+    spec = dec.lin_spec(name)
+    xd = dec.cc.to_device(np.ascontiguousarray(x[:t]))
+    yd = dec.cc.alloc(t * spec["n"] * (2 if out_f16 else 4))
+    try:
+        dec.lin_forward(name, xd, yd, t, out_f16=out_f16, path=path)
+        return dec.cc.d2h(yd, (t, spec["n"]), np.uint16 if out_f16 else np.float32)
+    finally:
+        dec.cc.free(xd)
+        dec.cc.free(yd)
+
+
+@pytest.mark.parametrize("n,k,group,t,bf16", [
+    (256, 256, 128, 256, False), (272, 384, 128, 70, False), (48, 128, 128, 17, False), (1000, 512, 128, 300, False),
+    (512, 256, 32, 100, False), (1536, 2048, 32, 33, False), (2048, 768, 32, 512, False), (320, 256, 128, 64, True),
+    (4096, 4096, 128, 128, False),
+])
+def test_prefill_matches_oracle(dec, orc, n, k, group, t, bf16):
+    say("prefill", n, k, group, t, bf16)
+    q, s, x = gen.make_linear(n, k, group, t, seed=21)
+    if bf16:
+        s = (gen.f16_bits_to_f32(s).view(np.uint32) >> 16).astype(np.uint16)
+    dec.upload_lin_g("pf", q, s, n, k, group, bf16)
+    want = orc.gemm_lane(x, t, q, s, n, k, group, scale_bf16=bf16, threads=16)
+    got = _device_forward(dec, "pf", x, t, ops.PATH_PREFILL)
+    m = parity.assert_close(got, want, "prefill n%d k%d g%d t%d" % (n, k, group, t))
+    say("   ", {a: m[a] for a in ("rel_l2", "max_ulp", "max_ulp_strict", "strict_pass_frac", "clamped")})
+    got16 = _device_forward(dec, "pf", x, t, ops.PATH_PREFILL, out_f16=True)
+    assert np.array_equal(got16, gen.f32_to_f16_bits(got))
+    auto = _device_forward(dec, "pf", x, t, ops.PATH_AUTO)
+    assert np.array_equal(_bits(auto), _bits(got))  # t > 16 routes to the prefill kernel
+
+
+@pytest.mark.parametrize("n,k,t", [(34816, 5120, 512), (5120, 17408, 512), (34816, 5120, 4096)])
+def test_prefill_full_shapes_against_device_twin_and_sampled_oracle(dec, orc, n, k, t):
+    """Layer shapes: every output against the bit-exact device twin (itself pinned to the CPU oracle above and on a
+    seeded sample here), because the CPU needs ~1e12 scalar MACs for the full matrix."""
+    say("prefill full", n, k, t)
+    group = 128
+    q, s, x = gen.make_linear(n, k, group, t, seed=5)
+    dec.upload_lin_g("pfull", q, s, n, k, group, False)
+    got = _device_forward(dec, "pfull", x, t, ops.PATH_PREFILL)
+    twin = _device_forward(dec, "pfull", x, t, ops.PATH_LANE)
+    rows = (gen.stream(1, 3000) % np.uint64(n)).astype(np.uint32)
+    toks = (gen.stream(2, 3000) % np.uint64(t)).astype(np.uint32)
+    smp = orc.gemm_lane_sample(x, q, s, k, group, rows, toks)
+    assert np.array_equal(_bits(twin[toks, rows]), _bits(smp))
+    m = parity.assert_close(got, twin, "prefill full n%d k%d t%d" % (n, k, t))
+    say("   ", {a: m[a] for a in ("rel_l2", "max_ulp", "max_ulp_strict", "strict_pass_frac", "clamped")})
+
+
+def test_prefill_refuses_irregular_scales_and_auto_falls_back(dec, orc):
+    n, k, group, t = 64, 256, 128, 40
+    q, s, x = gen.make_linear(n, k, group, t, seed=9)
+    s[3, 1] = 0  # a zero scale: the running-unit rescale of the MFMA kernel would divide by it
+    dec.upload_lin_g("irr", q, s, n, k, group, False)
+    with pytest.raises(ops.W4a16Error) as e:
+        _device_forward(dec, "irr", x, t, ops.PATH_PREFILL)
+    assert e.value.code == ffi.ERR_UNSUPPORTED
+    want = orc.gemm_lane(x, t, q, s, n, k, group, threads=8)
+    parity.assert_close(_device_forward(dec, "irr", x, t, ops.PATH_AUTO), want, "auto fallback")
