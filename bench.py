@@ -45,6 +45,19 @@ def make_copies(dec, gen, n, k, g, copies, prefix):
     return names, first
 
 
+def measured_traffic(kernel):
+    """HBM bytes per launch of `kernel` measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the plain-copy
+    calibration), as recorded in the committed summary profiles/pmc_traffic.txt; None if no record."""
+    path = os.path.join(ROOT, "profiles", "pmc_traffic.txt")
+    if not os.path.exists(path):
+        return None
+    for ln in open(path):
+        f = ln.split()
+        if len(f) >= 3 and f[0] == kernel and f[1] == "traffic_bytes_per_launch":
+            return int(float(f[2]))
+    return None
+
+
 def time_forward(dec, names, xd, yd, t, steps, warmup, path, out_f16=True):
     ms, wall = dec.bench_forward(names, xd, yd, t, steps, warmup=warmup, out_f16=out_f16, path=path)
     return ms / steps, wall / steps
@@ -119,6 +132,26 @@ def main():
              "parity_f32_out": {a: par_f32[a] for a in ("rel_l2", "max_ulp", "max_ulp_strict", "strict_pass_frac", "clamped")},
              "peaks": {"hbm_GBps": HBM_PEAK_GBPS, "mfma_f16_TFLOPs": MFMA_F16_PEAK_TFLOPS}}
 
+    # ---------------------------------------------------------------- prefill GEMM, M=4096 (second half of the metric)
+    mp = 4096
+    xp = gen.normal_f16(gen.shape_seed(n, k, tensor=4), (mp, k))
+    xpd = cc.to_device(xp)
+    ypd = cc.alloc(mp * n * 2)
+    psteps = max(5, args.steps // 20)
+    pf_ms, _ = time_forward(dec, names, xpd, ypd, mp, psteps, 3, ops.PATH_PREFILL)
+    pf_flops = 2.0 * mp * n * k
+    pf_tf = pf_flops / (pf_ms * 1e-3) / 1e12
+    # parity of the prefill result: a seeded sample of outputs against the CPU oracle
+    rows = (gen.stream(11, 2048) % np.uint64(n)).astype(np.uint32)
+    toks = (gen.stream(12, 2048) % np.uint64(mp)).astype(np.uint32)
+    dec.lin_forward(names[0], xpd, ypd, mp, out_f16=True, path=ops.PATH_PREFILL)
+    yp = cc.d2h(ypd, (mp, n), np.uint16)
+    ref_s = oracle.gemm_lane_sample(xp, q0, s0, k, g, rows, toks)
+    par_pf = parity.compare(gen.f16_bits_to_f32(yp[toks, rows]), gen.f16_bits_to_f32(gen.f32_to_f16_bits(ref_s)))
+    cc.free(xpd)
+    cc.free(ypd)
+    extra["parity_prefill_f16_sample2048"] = {a: par_pf[a] for a in ("rel_l2", "max_ulp", "max_ulp_strict", "strict_pass_frac", "clamped")}
+
     if not args.no_extra:
         table = []
         for mm in (4, 16):
@@ -135,6 +168,18 @@ def main():
             table.append({"shape": "down K17408 N5120 g128", "M": mm, "us": round(ms_m * 1e3, 2),
                           "GBps": round(b / (ms_m * 1e-3) / 1e9, 1), "hbm_frac": round(b / (ms_m * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
         extra["decode_table"] = table
+        ptable = []
+        xp2 = cc.to_device(gen.normal_f16(gen.shape_seed(n2, k2, tensor=4), (mp, k2)))
+        yp2 = cc.alloc(mp * max(n, n2) * 2)
+        xp1 = cc.to_device(xp)
+        for (nm, kk, nn, xdev, shape) in ((names, k, n, xp1, "gate_up K5120 N34816 g128"),
+                                          (names2, k2, n2, xp2, "down K17408 N5120 g128")):
+            for mm in (512, 1024, 4096):
+                ms_m, _ = time_forward(dec, nm, xdev, yp2, mm, psteps, 3, ops.PATH_PREFILL)
+                tf = 2.0 * mm * nn * kk / (ms_m * 1e-3) / 1e12
+                ptable.append({"shape": shape, "M": mm, "ms": round(ms_m, 4), "TFLOPs": round(tf, 1),
+                               "mfma_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4)})
+        extra["prefill_table"] = ptable
 
     line = {
         "metric": "W4A16 GEMM: decode GB/s (M=1) & prefill TFLOP/s (M=4096) vs MI355X peak",
@@ -152,8 +197,13 @@ def main():
         "config": {"workload": "decode GEMV M=1 K=5120 N=34816 g128 (27B dense gate+up), cold HBM: %d weight copies "
                                "rotated" % args.copies, "M": m, "K": k, "N": n, "group": g},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "w4a16_decode_g128_f16_rb2", "algorithmic_bytes_per_launch": nbytes},
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": measured_traffic("w4a16_decode_g128_f16_rb2_x1"),
+                     "kernel": "w4a16_decode_g128_f16_rb2_x1", "algorithmic_bytes_per_launch": nbytes},
+        "roofline_prefill": {"bound": "mfma", "achieved": round(pf_tf, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                             "unit": "TFLOP/s", "frac": round(pf_tf / MFMA_F16_PEAK_TFLOPS, 4),
+                             "traffic": measured_traffic("w4a16_prefill_g128_f16"),
+                             "kernel": "w4a16_prefill_g128_f16", "workload": "prefill GEMM M=4096 K=5120 N=34816 g128",
+                             "ms_per_launch": round(pf_ms, 4), "algorithmic_flops_per_launch": pf_flops},
         "cpu_baseline": cpu,
         "extra": extra,
     }
