@@ -73,22 +73,23 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     return w4_launch(ctx, sym, ceil_div(L.row_blocks, (size_t)rb), 1, (unsigned)(waves * 64), shmem, params);
 }
 
-// Prefill GEMM (kernels/prefill.hip): 256 x 256 block tiles, 8 waves, grid padded to a multiple of 8 so that block
-// b % 8 (the XCD it lands on) owns a contiguous run of tiles.
+// Prefill GEMM (kernels/prefill.hip).
 static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16) {
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has no tiled copy (needs k %% 128 == 0)");
     if (!L.scales_regular)
         return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has a zero or non-finite scale (use the decode path)");
     if (t * L.k * 2 >= 0x80000000ull || L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
         return w4_fail(W4A16_ERR_SHAPE, "prefill: x or the tiled weights reach 2 GiB, beyond the buffer-descriptor range");
-    const size_t tiles = ((t + 255) / 256) * ((L.n + 255) / 256);
-    const size_t per_xcd = (tiles + 7) / 8;
+    // block tile 128 (m) x 256 (n); 8 x 8 super-tiles dealt round-robin to the 8 XCDs (kernels/prefill.hip)
+    const size_t tiles_m = (t + 127) / 128, tiles_n = (L.n + 255) / 256;
+    const size_t supers = ((tiles_m + 7) / 8) * ((tiles_n + 7) / 8);
+    const size_t grid = ((supers + 7) / 8) * 64 * 8;
     char sym[64];
     snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s", L.group, L.scale_bf16 ? "bf16" : "f16");
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of};
-    return w4_launch(ctx, sym, (unsigned)(per_xcd * 8), 1, 512, 2 * 256 * 72 * 2, params);
+    return w4_launch(ctx, sym, (unsigned)grid, 1, 256, 2 * 128 * 72 * 2, params);
 }
 
 // t > 16 without the prefill kernel (irregular scales): the decode kernel over chunks of 16 rows.

@@ -1,8 +1,9 @@
 // Prefill regime (t > 16 activation rows): tiled GEMM  y[t][n] = x[t][k] * W^T  on v_mfma_f32_32x32x16_f16.
 // Role of the reference's prefill path gemm_launch -> marlin_gemm_try / w4a16_gemm_g128_mma
 // (w4a16_dec/kernels/gemm.rs:4-51, kernels/marlin.rs:94-213, assets/gptq4.cu:984-1147), designed for CDNA4:
-//   * workgroup = 8 waves (2 along m x 4 along n), block tile 256 (m) x 256 (n), wave tile 128 x 64 = 4 x 2 MFMA tiles
-//     of 32 x 32 with f32 accumulators in arch VGPRs (128 registers), two waves per SIMD;
+//   * workgroup = 4 waves along n, block tile 128 (m) x 256 (n), wave tile 128 x 64 = 4 x 2 MFMA tiles of 32 x 32 with
+//     f32 accumulators in arch VGPRs (128 registers); two workgroups per CU, so one block's barriers and LDS writes
+//     overlap the other's MFMAs;
 //   * x (the A operand) is staged through LDS in k slabs of 64, double buffered, rows padded to 72 halves so the
 //     ds_read_b128 fragment reads are bank-conflict free; rows >= t come from out-of-range buffer loads (zeros);
 //   * the weights (B operand) never touch LDS: the tiled layout of w4a16_common.hpp already is the MFMA B layout —
@@ -13,15 +14,19 @@
 //     holds sum / s_g; at each group boundary it is multiplied by s_prev / s_cur and the new group's integer products
 //     are added by the MFMA itself; the epilogue multiplies by the last scale.  No weight is rounded to f16 and no
 //     second accumulator set is needed.  (Linears with a zero or non-finite scale are not routed here.)
-//   * workgroups are numbered so that each XCD works on a contiguous run of n tiles, m fastest: the sixteen m tiles
-//     that share a weight panel run on the same L2.
+//   * workgroups are numbered so that the ~64 blocks resident on one XCD form an 8 x 8 super-tile: each x slab and
+//     each weight panel is fetched into that L2 once per eight uses.
 #include "w4a16_common.hpp"
 
-#define PF_BM 256
+#ifndef PF_WM
+#define PF_WM 1           // waves along m (1: block tile 128 x 256, 4 waves; 2: 256 x 256, 8 waves)
+#endif
+#define PF_BM (128 * PF_WM)
 #define PF_BN 256
 #define PF_KS 64          // k per LDS stage
 #define PF_LDA 72         // halves per staged x row (64 + 8 padding)
-#define PF_THREADS 512
+#define PF_THREADS (256 * PF_WM)
+#define PF_SUPER 8        // super-tile edge: 8 x 8 block tiles run together on one XCD
 
 template <int G, bool SBF>
 __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
@@ -31,22 +36,27 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     constexpr int GPT = W4_TILE_K / G;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave & 1, wn = wave >> 1;  // 2 x 4 waves
+    const int wm = wave % PF_WM, wn = wave / PF_WM;  // PF_WM x 4 waves
     const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
 
-    // XCD-aware tile numbering: block b runs on XCD b % 8; give each XCD a contiguous run of tiles, m fastest.
+    // XCD-aware tile numbering.  Block b runs on XCD b % 8 and is the (b / 8)-th block of that XCD; consecutive
+    // blocks of an XCD walk one super-tile of PF_SUPER x PF_SUPER block tiles (m fastest), so the ~64 blocks resident
+    // on an XCD at a time share 8 x slabs and 8 weight panels through its L2.  Super-tiles are dealt round-robin
+    // to the XCDs.
     const int tiles_m = (t + PF_BM - 1) / PF_BM, tiles_n = (n + PF_BN - 1) / PF_BN;
-    const int n_tiles = tiles_m * tiles_n;
-    const int per_xcd = (n_tiles + 7) / 8;
-    const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if ((int)(blockIdx.x >> 3) >= per_xcd || tile >= n_tiles) return;  // uniform for the whole block
-    const int m0 = (tile % tiles_m) * PF_BM, n0 = (tile / tiles_m) * PF_BN;
+    const int sm_n = (tiles_m + PF_SUPER - 1) / PF_SUPER, sn_n = (tiles_n + PF_SUPER - 1) / PF_SUPER;
+    const int j = blockIdx.x >> 3;
+    const int super = (blockIdx.x & 7) + 8 * (j / (PF_SUPER * PF_SUPER)), within = j % (PF_SUPER * PF_SUPER);
+    if (super >= sm_n * sn_n) return;  // uniform for the whole block
+    const int tm = (super % sm_n) * PF_SUPER + within % PF_SUPER, tn = (super / sm_n) * PF_SUPER + within / PF_SUPER;
+    if (tm >= tiles_m || tn >= tiles_n) return;
+    const int m0 = tm * PF_BM, n0 = tn * PF_BN;
 
     const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)t * (unsigned)k * 2u);
     const __amdgpu_buffer_rsrc_t qr = w4_make_rsrc(qt, (unsigned)row_blocks * (unsigned)kt_n * 1024u);
     const __amdgpu_buffer_rsrc_t sr = w4_make_rsrc(st, (unsigned)row_blocks * (unsigned)kg_n * 32u);
 
-    // ---- x staging: 256 rows x 64 k per stage = 2048 chunks of 16 B, 4 per thread
+    // ---- x staging: PF_BM rows x 64 k per stage = PF_BM * 8 chunks of 16 B, 4 per thread
     unsigned xa_off[4];
     int xa_lds[4];
 #pragma unroll
@@ -120,15 +130,17 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
 #pragma unroll
             for (int kbl = 0; kbl < 4; kbl++) {
                 const int kb = half * 4 + kbl, w = kb >> 1, h = kb & 1;
-                // group boundary: re-express the accumulators in the new group's scale
-                if ((G == 128 && kb == 0) || (G == 32 && h == 0)) {
+                // group boundary: re-express the accumulators in the new group's scale.  The multiply of each
+                // accumulator tile sits right before that tile's first MFMA of the group, so the VALU work of one tile
+                // overlaps the matrix-core time of the previous one.
+                const bool boundary = (G == 128 && kb == 0) || (G == 32 && h == 0);
+                float ratio[2] = {1.f, 1.f};
+                if (boundary) {
 #pragma unroll
                     for (int ni = 0; ni < 2; ni++) {
                         const float s_cur = w4_scale_fast<SBF>(sc[ni][G == 128 ? 0 : w]);
-                        const float ratio = unit[ni] / s_cur;
+                        ratio[ni] = unit[ni] / s_cur;
                         unit[ni] = s_cur;
-#pragma unroll
-                        for (int mi = 0; mi < 4; mi++) acc[mi][ni] *= ratio;
                     }
                 }
                 h8_t a[4];
@@ -139,8 +151,10 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
                 for (int ni = 0; ni < 2; ni++) {
                     const h8_t b = w4_deq8(bq[ni][h][w]);
 #pragma unroll
-                    for (int mi = 0; mi < 4; mi++)
+                    for (int mi = 0; mi < 4; mi++) {
+                        if (boundary) acc[mi][ni] *= ratio[ni];
                         acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b, acc[mi][ni], 0, 0, 0);
+                    }
                 }
             }
             if (s + 1 < stages) store_a((s + 1) & 1);
@@ -178,7 +192,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
 }
 
 #define PREFILL_KERNEL(NAME, G, SBF)                                                                               \
-    extern "C" __global__ __launch_bounds__(PF_THREADS) void NAME(const u4_t* qt, const uint16_t* st,              \
+    extern "C" __global__ __launch_bounds__(PF_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void NAME(const u4_t* qt, const uint16_t* st, \
                                                                   const uint16_t* x, void* y, int row_blocks,      \
                                                                   int k, int n, int t, int out_f16) {              \
         prefill_body<G, SBF>(qt, st, x, y, row_blocks, k, n, t, out_f16);                                          \
