@@ -163,6 +163,63 @@ int w4a16_bench_forward(w4a16_ctx* ctx, const char* const* names, size_t n_names
                         size_t t, int out_f16, int path, size_t warmup, size_t reps, float* ms_events,
                         double* ms_wall);
 
+/* ------------------------------------------------------------------------------------------------------------
+ * MoE expert FFN (grouped / ragged W4A16 GEMM)
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* build_marlin_moe_arenas (w4a16_dec/upload.rs:1116-1235): register the experts of one MoE layer by name.
+ *   q13: u32 [n_experts][2*n_ff][h/8]      fused gate|up projection, rows 0..n_ff gate, n_ff..2*n_ff up
+ *   s13: u16 [n_experts][2*n_ff][h/group]
+ *   q2 : u32 [n_experts][h][n_ff/8]        down projection
+ *   s2 : u16 [n_experts][h][n_ff/group]
+ * Byte lengths are enforced.  Needs h % 128 == 0, n_ff % 128 == 0 (whole k tiles) — true of the reference's MoE
+ * shapes.  The experts are kept only in the tiled layout, one arena per projection, experts at a fixed stride. */
+int w4a16_upload_experts(w4a16_ctx* ctx, const char* name, size_t n_experts, const void* q13, size_t q13_bytes,
+                         const void* s13, size_t s13_bytes, const void* q2, size_t q2_bytes, const void* s2,
+                         size_t s2_bytes, size_t h, size_t n_ff, size_t group, int scale_bf16);
+int w4a16_experts_info(w4a16_ctx* ctx, const char* name, size_t* n_experts, size_t* h, size_t* n_ff, size_t* group,
+                       int* scale_bf16);
+/* Dequantised weights of one expert's projection (which: 0 = gate|up [2*n_ff][h], 1 = down [h][n_ff]) as f32,
+ * read back from the arena (covers the arena re-layout bit for bit). */
+int w4a16_experts_dequant_dump(w4a16_ctx* ctx, const char* name, int which, size_t expert, uint64_t out_f32_dev);
+
+/* moe_topk (w4a16_dec/mod.rs:168-185): host routing of t tokens.  Softmax over all n_exp logits in f32, the top_k
+ * largest probabilities with ties to the lower index, weights renormalised by the selected sum.
+ * idx: int32 [t][top_k], w: f32 [t][top_k]. */
+int w4a16_moe_topk_host(const float* logits, size_t t, size_t n_exp, size_t top_k, int32_t* idx, float* w);
+/* Device kernel w4a16_moe_topk_t, assets/moe.cu:686-759: the same rule on the device, logits f32 [t][n_exp] already resident.
+ * n_exp <= 1024, top_k <= 64.  The exponential and the softmax sum are evaluated in a different order than on the
+ * host, so weights agree to rounding, not bit for bit. */
+int w4a16_moe_route(w4a16_ctx* ctx, uint64_t logits_dev, size_t t, size_t n_exp, size_t top_k, uint64_t idx_dev,
+                    uint64_t wt_dev);
+/* Device kernels w4a16_moe_align2 and w4a16_moe_align_marlin, assets/moe.cu:860-908 and 1599-1633: stable counting sort of the
+ * ns = t*top_k slots by expert, every expert's run padded to a multiple of `block` with the sentinel ns.
+ *   sorted_dev: int32, capacity >= ns + n_exp*block; expert_ids_dev: int32 per block of `block` sorted entries,
+ *   capacity >= ns/block + n_exp + 1; num_post_dev: int32 [2] = {padded total, experts hit}. */
+int w4a16_moe_align(w4a16_ctx* ctx, uint64_t idx_dev, size_t ns, size_t n_exp, size_t block, uint64_t sorted_dev,
+                    uint64_t expert_ids_dev, uint64_t num_post_dev);
+
+/* marlin_moe_ffn_dev (w4a16_dec/kernels/marlin_moe.rs:290-422): the routed-expert FFN of t tokens on the launch
+ * stream, no host synchronisation:
+ *   align slots -> act[slot] = f16(silu(f16(gate)) * f16(up)), gate|up = W13[expert] * x[token]
+ *               -> c2[slot] = f16(wt[slot] * (W2[expert] * act[slot]))
+ *               -> y[token] = sum over the token's slots of c2, in slot order, f32.
+ *   x_dev f16 [t][h]; idx_dev int32 [t*top_k]; wt_dev f32 [t*top_k]; y_dev f32 [t][h].
+ * Scratch (sorted ids, act, c2) is owned by the context and grown on demand. */
+int w4a16_moe_ffn(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t idx_dev, uint64_t wt_dev, size_t t,
+                  size_t top_k, uint64_t y_dev);
+/* Scratch of the last w4a16_moe_ffn call, for stage-by-stage checks (the reference exposes the same buffers to
+ * its moe_selfcheck, w4a16_dec/probe.rs:153): which = 0 sorted ids (int32), 1 expert ids (int32), 2 num_post
+ * (int32 [2]), 3 act (f16 [ns][n_ff]), 4 c2 (f16 [ns][h]).  Also reports the segment size used. */
+int w4a16_moe_scratch(w4a16_ctx* ctx, int which, uint64_t* dptr, size_t* bytes, size_t* block);
+/* Launch-shape override for the MoE GEMMs (0 = automatic): block = slots per segment (4, 16, 32, 48, 64);
+ * waves = waves per workgroup (k split for segments of <= 16 slots, output-row units otherwise). */
+int w4a16_set_moe_shape(w4a16_ctx* ctx, int block, int waves);
+/* Timed back-to-back w4a16_moe_ffn calls (as w4a16_bench_forward); call i uses experts names[i % n_names]. */
+int w4a16_bench_moe(w4a16_ctx* ctx, const char* const* names, size_t n_names, uint64_t x_dev, uint64_t idx_dev,
+                    uint64_t wt_dev, size_t t, size_t top_k, uint64_t y_dev, size_t warmup, size_t reps,
+                    float* ms_events, double* ms_wall);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,24 @@ struct W4Lin {
     bool scales_regular = true;  // every scale finite and non-zero (the MFMA prefill kernel divides by them)
 };
 
+// The experts of one MoE layer: two arenas in the tiled layout, experts at a fixed stride
+// (reference: moe_m13 / moe_s13 / moe_m2 / moe_s2, w4a16_dec/upload.rs:1116-1235).
+struct W4Experts {
+    uint64_t q13 = 0, s13 = 0, q2 = 0, s2 = 0;
+    size_t n_exp = 0, h = 0, n_ff = 0, group = 0;
+    int scale_bf16 = 0;
+    size_t q13_stride = 0, s13_stride = 0, q2_stride = 0, s2_stride = 0;  // bytes per expert
+};
+
+// Scratch of the MoE FFN, grown on demand (reference: moe_msorted / moe_mexp / moe_mnpost / moe_mact / moe_mc2,
+// kernels/marlin_moe.rs:322-342).
+struct W4MoeScratch {
+    uint64_t sorted = 0, expert_ids = 0, num_post = 0, act = 0, c2 = 0;
+    size_t sorted_cap = 0, expert_cap = 0, act_cap = 0, c2_cap = 0;       // bytes
+    size_t sorted_len = 0, expert_len = 0, act_len = 0, c2_len = 0;       // bytes used by the last call
+    size_t block = 0;
+};
+
 struct w4a16_event {
     hipEvent_t ev;
 };
@@ -36,6 +54,9 @@ struct w4a16_ctx {
     std::unordered_map<uint64_t, size_t> allocs;
     size_t allocated = 0;
     std::map<std::string, W4Lin> lins;
+    std::map<std::string, W4Experts> experts;
+    W4MoeScratch moe;
+    int moe_block = 0, moe_waves = 0;  // 0 = automatic
     int decode_rows_per_wave = 0, decode_waves_per_block = 0;  // 0 = automatic
     int cu_count = 0;
 };

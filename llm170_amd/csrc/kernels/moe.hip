@@ -1,0 +1,623 @@
+// MoE expert FFN on W4A16 experts: routing, slot alignment, grouped/ragged expert GEMMs, top-k reduction.
+// Role of the reference's route -> align -> grouped gate+up -> SiLU*up -> grouped down (x top-k weight) -> sum
+// sequence (w4a16_dec/kernels/marlin_moe.rs:290-422 over assets/moe.cu:686-759, 860-908, 1599-1674 and the vendored
+// grouped Marlin kernels), designed for CDNA4:
+//   * a "slot" is one (token, chosen expert) pair, slot j = token * top_k + choice.  The align kernel sorts slots by
+//     expert (stable) and pads every expert's run to a multiple of the segment size; a segment = up to BLK slots of
+//     one expert.  Workgroups are numbered (segment, output-row group); segments past the padded total exit at once.
+//   * expert weights live in one arena in the tiled layout of w4a16_common.hpp, experts at a fixed stride; the
+//     gate and up projections are one fused matrix (rows 0..n_ff gate, n_ff..2 n_ff up; upload.rs:1116-1235).
+//   * both regimes multiply on v_mfma_f32_16x16x32_f16 with weights as exact integers (A operand = one dword of the
+//     64 lanes of a tile) and apply the group scale to the f32 group sum, like the dense decode kernel.
+//       - moe_dec (segments of <= 4 or <= 16 slots, decode steps): HBM streaming, in-block split-K over the waves,
+//         x gathered straight from global memory (one load + DPP row shifts for <= 4 slots);
+//       - moe_mm (segments of 16..64 slots, prefill chunks): the waves of a block take different output rows of the
+//         same segment and share the gathered x rows through LDS (double buffered, one k tile per stage), so x is
+//         fetched once per block instead of once per wave.
+//   * GLU epilogue: a wave owns gate row block u and up row block u + n_ff/16, rounds both sums to f16 (the reference
+//     materialises them as f16, moe.cu:1649-1660) and writes silu(g)*u as f16 — the intermediate never reaches
+//     memory.  LIN epilogue: optional multiply by the slot's routing weight, f16 or f32 rows scattered by slot id.
+//   * for group size 32 the four scale groups of a k tile come with ONE load per row block: lane c of each quad
+//     fetches group c % 4 and v_mov_b32_dpp quad_perm broadcasts group w when MFMA w needs it.
+#include <type_traits>
+
+#include "w4a16_common.hpp"
+
+#define MOE_LDX 136  // halves per staged x row: 128 + 8 padding (272-byte stride: 16-lane b128 reads hit all banks once)
+
+template <int W>
+__device__ __forceinline__ unsigned w4_quad_bcast(unsigned v) {
+    return __builtin_amdgcn_update_dpp(0u, v, W * 0x55, 0xF, 0xF, true);
+}
+
+template <int SH>
+__device__ __forceinline__ u4_t moe_row_shl(u4_t v) {
+    u4_t r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = __builtin_amdgcn_update_dpp(0u, v[i], 0x100 + SH, 0xF, 0xF, true);
+    return r;
+}
+
+// The four scales (rows 4q..4q+3 of the row block) of scale group W of the current k tile, as f32.
+// s = the lane's b64 scale load: for G = 128 the tile's only group, for G = 32 group (lane % 4).
+template <int G, bool SBF, int W>
+__device__ __forceinline__ f4_t moe_scale4(u2_t s) {
+    unsigned d0 = s[0], d1 = s[1];
+    if (G == 32) {
+        d0 = w4_quad_bcast<W>(d0);
+        d1 = w4_quad_bcast<W>(d1);
+    }
+    f4_t r;
+    r[0] = w4_scale_fast<SBF>(d0 & 0xFFFFu);
+    r[1] = w4_scale_fast<SBF>(d0 >> 16);
+    r[2] = w4_scale_fast<SBF>(d1 & 0xFFFFu);
+    r[3] = w4_scale_fast<SBF>(d1 >> 16);
+    return r;
+}
+
+__device__ __forceinline__ float moe_round_f16(float v) { return (float)(_Float16)v; }
+
+// Epilogue of one 16 x 16 result tile pair for one token column.  a0/a1: the lane's four rows of row blocks 0/1 of
+// the unit.  GLU: a0 = gate, a1 = up -> act[slot][u*16 + 4q + i] = f16(silu(f16(g)) * f16(u)).
+// LIN: rows of row blocks rbA / rbB, scaled by wgt, as f16 or f32.
+template <bool GLU>
+__device__ __forceinline__ void moe_store(f4_t a0, f4_t a1, int slot, int q, int u, int rbA, int rbB, bool haveB,
+                                          void* __restrict__ y, int y_f16, float wgt, int n) {
+    if (GLU) {
+        const int n_ff = n >> 1;
+        h4_t o;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float g = moe_round_f16(a0[i]), up = moe_round_f16(a1[i]);
+            o[i] = (_Float16)((g / (1.0f + expf(-g))) * up);
+        }
+        *reinterpret_cast<h4_t*>(reinterpret_cast<_Float16*>(y) + (size_t)slot * n_ff + u * 16 + 4 * q) = o;
+    } else {
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++) {
+            if (rb == 1 && !haveB) break;
+            const f4_t a = (rb == 0 ? a0 : a1) * wgt;
+            const int row = (rb == 0 ? rbA : rbB) * 16 + 4 * q;
+            if (y_f16) {
+                _Float16* yo = reinterpret_cast<_Float16*>(y) + (size_t)slot * n + row;
+                if (row + 3 < n) {
+                    h4_t v = {(_Float16)a[0], (_Float16)a[1], (_Float16)a[2], (_Float16)a[3]};
+                    *reinterpret_cast<h4_t*>(yo) = v;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (row + i < n) yo[i] = (_Float16)a[i];
+                }
+            } else {
+                float* yo = reinterpret_cast<float*>(y) + (size_t)slot * n + row;
+                if (row + 3 < n) {
+                    *reinterpret_cast<f4_t*>(yo) = a;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (row + i < n) yo[i] = a[i];
+                }
+            }
+        }
+    }
+}
+
+// Arguments shared by the two grouped kernels.
+//   qa/sa: arena bases, expert e at qa + e*q_stride / sa + e*s_stride (bytes); each expert is row_blocks x k/128
+//          tiles and [row_blocks][k/G][16] scales.  x: f16 [x_rows][k]; slot j reads row j / x_div.
+//   y: GLU -> f16 [ns][n/2]; LIN -> f16 or f32 [ns][n].  topw: null or f32 [ns] (LIN only).
+//   sorted_ids[seg*blk + i]: slot id or the sentinel ns; expert_ids[seg]; num_post[0] = padded slot total.
+#define MOE_PARAMS                                                                                                  \
+    const char *__restrict__ qa, const char *__restrict__ sa, unsigned long long q_stride,                          \
+        unsigned long long s_stride, const uint16_t *__restrict__ x, int x_rows, int x_div, void *__restrict__ y,   \
+        int y_f16, const float *__restrict__ topw, const int *__restrict__ sorted_ids,                              \
+        const int *__restrict__ expert_ids, const int *__restrict__ num_post, int blk, int ns, int row_blocks, int k, \
+        int n
+#define MOE_ARGS \
+    qa, sa, q_stride, s_stride, x, x_rows, x_div, y, y_f16, topw, sorted_ids, expert_ids, num_post, blk, ns, row_blocks, k, n
+
+// ---------------------------------------------------------------------------------------------------- moe_dec
+template <int RB, int XL>
+struct MoeDecStage {
+    u4_t q[RB];
+    u2_t s[RB];
+    u4_t x[XL];
+};
+
+// One block = (segment, unit of two row blocks); its W waves split k.  XL = 1: blk <= 4; XL = 4: blk <= 16.
+template <int G, bool SBF, bool GLU, int XL, int DEPTH>
+__device__ __forceinline__ void moe_dec_body(MOE_PARAMS) {
+    extern __shared__ f4_t red[];  // [W][2][64]
+    constexpr int GPT = W4_TILE_K / G;
+    constexpr int C = 4 / XL, TPL = 16 / C;
+    const int lane = threadIdx.x & 63, W = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int units = GLU ? row_blocks >> 1 : (row_blocks + 1) >> 1;
+    const int seg = blockIdx.x / units, u = blockIdx.x % units;
+    if (seg * blk >= num_post[0]) return;
+    const int e = __builtin_amdgcn_readfirstlane(expert_ids[seg]);
+    const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
+    const int kt0 = (kt_n * wave) / W, kt1 = (kt_n * (wave + 1)) / W;
+    const int m = lane & 15, g = lane >> 4;
+    const int rbA = GLU ? u : 2 * u, rbB = GLU ? u + units : min(2 * u + 1, row_blocks - 1);
+    const bool haveB = GLU || 2 * u + 1 < row_blocks;
+
+    const __amdgpu_buffer_rsrc_t qr =
+        w4_make_rsrc(qa + (unsigned long long)e * q_stride, (unsigned)row_blocks * (unsigned)kt_n * 1024u);
+    const __amdgpu_buffer_rsrc_t sr =
+        w4_make_rsrc(sa + (unsigned long long)e * s_stride, (unsigned)row_blocks * (unsigned)kg_n * 32u);
+    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)x_rows * (unsigned)k * 2u);
+
+    const int xtok = m % TPL, xchunk = m / TPL;
+    const int xslot = xtok < blk ? sorted_ids[seg * blk + xtok] : ns;
+    const unsigned xoff =
+        xslot < ns ? ((unsigned)(xslot / x_div) * (unsigned)k + (unsigned)(xchunk * 32 + g * 8)) * 2u : W4_OOB;
+    const unsigned qoff[2] = {(unsigned)rbA * (unsigned)kt_n * 1024u + (unsigned)lane * 16u,
+                              (unsigned)rbB * (unsigned)kt_n * 1024u + (unsigned)lane * 16u};
+    // scale load: G = 128 -> the tile's group; G = 32 -> group (lane % 4) of the tile's four
+    const unsigned sg = G == 32 ? (unsigned)(lane & 3) * 32u : 0u;
+    const unsigned soff[2] = {(unsigned)rbA * (unsigned)kg_n * 32u + sg + (unsigned)g * 8u,
+                              (unsigned)rbB * (unsigned)kg_n * 32u + sg + (unsigned)g * 8u};
+    f4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+
+    MoeDecStage<2, XL> stage[DEPTH];
+    auto load = [&](MoeDecStage<2, XL>& s_, int kt) {
+        const bool live = kt < kt1;
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+            s_.q[rb] = __builtin_amdgcn_raw_buffer_load_b128(qr, live ? qoff[rb] + (unsigned)kt * 1024u : W4_OOB, 0, 2);
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+            s_.s[rb] = __builtin_amdgcn_raw_buffer_load_b64(sr, live ? soff[rb] + (unsigned)kt * (GPT * 32u) : W4_OOB, 0, 0);
+#pragma unroll
+        for (int l = 0; l < XL; l++)
+            s_.x[l] = __builtin_amdgcn_raw_buffer_load_b128(
+                xr, live ? xoff + (unsigned)(kt * W4_TILE_K + l * C * 32) * 2u : W4_OOB, 0, 0);
+    };
+    auto compute = [&](const MoeDecStage<2, XL>& s_) {
+        u4_t xb[4];
+#pragma unroll
+        for (int l = 0; l < XL; l++) {
+            xb[l * C] = s_.x[l];
+            if (C == 4) {
+                xb[1] = moe_row_shl<TPL>(s_.x[l]);
+                xb[2] = moe_row_shl<2 * TPL>(s_.x[l]);
+                xb[3] = moe_row_shl<3 * TPL>(s_.x[l]);
+            }
+        }
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++) {
+            const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+            if (G == 128) {
+                f4_t part = zero;
+#pragma unroll
+                for (int w = 0; w < 4; w++)
+                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
+                                                                  __builtin_bit_cast(h8_t, xb[w]), part, 0, 0, 0);
+                acc[rb] += moe_scale4<G, SBF, 0>(s_.s[rb]) * part;
+            } else {
+                f4_t p0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][0]), __builtin_bit_cast(h8_t, xb[0]), zero, 0, 0, 0);
+                f4_t p1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][1]), __builtin_bit_cast(h8_t, xb[1]), zero, 0, 0, 0);
+                f4_t p2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][2]), __builtin_bit_cast(h8_t, xb[2]), zero, 0, 0, 0);
+                f4_t p3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][3]), __builtin_bit_cast(h8_t, xb[3]), zero, 0, 0, 0);
+                acc[rb] += moe_scale4<G, SBF, 0>(s_.s[rb]) * p0;
+                acc[rb] += moe_scale4<G, SBF, 1>(s_.s[rb]) * p1;
+                acc[rb] += moe_scale4<G, SBF, 2>(s_.s[rb]) * p2;
+                acc[rb] += moe_scale4<G, SBF, 3>(s_.s[rb]) * p3;
+            }
+        }
+    };
+
+    // counted loop: round -1 fills the ring with compute skipped, so the loads outstanding at every stage's wait are
+    // in ring order (see the dense decode kernel)
+    const int tiles = kt1 - kt0;
+    const int rounds = tiles / DEPTH;
+    for (int r = -1; r < rounds; r++) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            if (r >= 0) compute(stage[d]);
+            __builtin_amdgcn_sched_barrier(0);
+            load(stage[d], kt0 + (r + 1) * DEPTH + d);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < DEPTH - 1; d++)
+        if (rounds * DEPTH + d < tiles) compute(stage[d]);
+
+    if (W > 1) {
+        if (wave != 0) {
+            red[(wave * 2 + 0) * 64 + lane] = acc[0];
+            red[(wave * 2 + 1) * 64 + lane] = acc[1];
+        }
+        __syncthreads();
+        if (wave != 0) return;
+        for (int w = 1; w < W; w++) {
+            acc[0] += red[(w * 2 + 0) * 64 + lane];
+            acc[1] += red[(w * 2 + 1) * 64 + lane];
+        }
+    }
+    const int slot = m < blk ? sorted_ids[seg * blk + m] : ns;
+    if (slot >= ns) return;
+    const float wgt = (!GLU && topw) ? topw[slot] : 1.0f;
+    moe_store<GLU>(acc[0], acc[1], slot, g, u, rbA, rbB, haveB, y, y_f16, wgt, n);
+}
+
+// ---------------------------------------------------------------------------------------------------- moe_mm
+template <int RB>
+struct MoeMmStage {
+    u4_t q[RB];
+    u2_t s[RB];
+};
+
+// One block = (segment of blk = 16*TT slots, group of W units); wave w owns unit group*W + w over the whole k range.
+template <int G, bool SBF, bool GLU, int TT, int DEPTH>
+__device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
+    extern __shared__ _Float16 xs[];  // [2][16*TT][MOE_LDX]
+    constexpr int GPT = W4_TILE_K / G;
+    constexpr int ROWS = 16 * TT;
+    const int tid = threadIdx.x, lane = tid & 63, W = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int units = GLU ? row_blocks >> 1 : (row_blocks + 1) >> 1;
+    const int groups = (units + W - 1) / W;
+    const int seg = blockIdx.x / groups;
+    if (seg * blk >= num_post[0]) return;  // uniform for the block, before any barrier
+    const int u_raw = (blockIdx.x % groups) * W + wave;
+    const bool active = u_raw < units;  // a surplus wave repeats the last unit and stores nothing
+    const int u = min(u_raw, units - 1);
+    const int e = __builtin_amdgcn_readfirstlane(expert_ids[seg]);
+    const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
+    const int c = lane & 15, q = lane >> 4;
+    const int rbA = GLU ? u : 2 * u, rbB = GLU ? u + units : min(2 * u + 1, row_blocks - 1);
+    const bool haveB = GLU || 2 * u + 1 < row_blocks;
+
+    const __amdgpu_buffer_rsrc_t qr =
+        w4_make_rsrc(qa + (unsigned long long)e * q_stride, (unsigned)row_blocks * (unsigned)kt_n * 1024u);
+    const __amdgpu_buffer_rsrc_t sr =
+        w4_make_rsrc(sa + (unsigned long long)e * s_stride, (unsigned)row_blocks * (unsigned)kg_n * 32u);
+    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)x_rows * (unsigned)k * 2u);
+
+    // x staging: one k tile of the segment's rows = ROWS x 256 B; 16 threads cover a row, 4*W rows per pass
+    const int rows_pp = 4 * W;
+    unsigned xg_off[TT];
+    int xl_off[TT];
+#pragma unroll
+    for (int p = 0; p < TT; p++) {
+        const int row = p * rows_pp + (tid >> 4);
+        const int slot = row < ROWS ? sorted_ids[seg * blk + row] : ns;
+        xg_off[p] = slot < ns ? ((unsigned)(slot / x_div) * (unsigned)k + (unsigned)(tid & 15) * 8u) * 2u : W4_OOB;
+        xl_off[p] = row < ROWS ? row * MOE_LDX + (tid & 15) * 8 : -1;
+    }
+    u4_t xreg[TT];
+    auto load_x = [&](int kt) {
+#pragma unroll
+        for (int p = 0; p < TT; p++)
+            xreg[p] = __builtin_amdgcn_raw_buffer_load_b128(
+                xr, (kt < kt_n && xg_off[p] != W4_OOB) ? xg_off[p] + (unsigned)kt * (W4_TILE_K * 2u) : W4_OOB, 0, 0);
+    };
+    auto store_x = [&](int buf) {
+        _Float16* base = xs + buf * (ROWS * MOE_LDX);
+#pragma unroll
+        for (int p = 0; p < TT; p++)
+            if (xl_off[p] >= 0) *reinterpret_cast<u4_t*>(base + xl_off[p]) = xreg[p];
+    };
+
+    const unsigned qoff[2] = {(unsigned)rbA * (unsigned)kt_n * 1024u + (unsigned)lane * 16u,
+                              (unsigned)rbB * (unsigned)kt_n * 1024u + (unsigned)lane * 16u};
+    const unsigned sg = G == 32 ? (unsigned)(lane & 3) * 32u : 0u;
+    const unsigned soff[2] = {(unsigned)rbA * (unsigned)kg_n * 32u + sg + (unsigned)q * 8u,
+                              (unsigned)rbB * (unsigned)kg_n * 32u + sg + (unsigned)q * 8u};
+    MoeMmStage<2> stage[DEPTH];
+    auto load_w = [&](MoeMmStage<2>& s_, int kt) {
+        const bool live = kt < kt_n;
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+            s_.q[rb] = __builtin_amdgcn_raw_buffer_load_b128(qr, live ? qoff[rb] + (unsigned)kt * 1024u : W4_OOB, 0, 2);
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+            s_.s[rb] = __builtin_amdgcn_raw_buffer_load_b64(sr, live ? soff[rb] + (unsigned)kt * (GPT * 32u) : W4_OOB, 0, 0);
+    };
+
+    f4_t acc[2][TT];
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++) acc[rb][tt] = (f4_t){0.f, 0.f, 0.f, 0.f};
+
+    auto compute = [&](const MoeMmStage<2>& s_, int buf) {
+        const _Float16* xb = xs + buf * (ROWS * MOE_LDX) + c * MOE_LDX + q * 8;
+        const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+        f4_t part[2][TT];
+        auto step = [&](auto wc) {
+            constexpr int w = decltype(wc)::value;
+            h8_t b[TT];
+#pragma unroll
+            for (int tt = 0; tt < TT; tt++) b[tt] = *reinterpret_cast<const h8_t*>(xb + tt * 16 * MOE_LDX + w * 32);
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++) {
+                const h8_t a = w4_deq8(s_.q[rb][w]);
+                if (G == 32) {
+                    const f4_t sc = moe_scale4<G, SBF, w>(s_.s[rb]);
+#pragma unroll
+                    for (int tt = 0; tt < TT; tt++)
+                        acc[rb][tt] += sc * __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], zero, 0, 0, 0);
+                } else {
+#pragma unroll
+                    for (int tt = 0; tt < TT; tt++)
+                        part[rb][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], w == 0 ? zero : part[rb][tt], 0, 0, 0);
+                }
+            }
+        };
+        step(std::integral_constant<int, 0>{});
+        step(std::integral_constant<int, 1>{});
+        step(std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 3>{});
+        if (G == 128) {
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++) {
+                const f4_t sc = moe_scale4<G, SBF, 0>(s_.s[rb]);
+#pragma unroll
+                for (int tt = 0; tt < TT; tt++) acc[rb][tt] += sc * part[rb][tt];
+            }
+        }
+    };
+
+    // prologue: x tile 0 into LDS buffer 0, DEPTH weight stages in flight
+    load_x(0);
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) load_w(stage[d], d);
+    store_x(0);
+    __syncthreads();
+    for (int kt0 = 0; kt0 < kt_n; kt0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            const int kt = kt0 + d;
+            load_x(kt + 1);  // out of range past the last tile: zeros, no traffic
+            if (kt < kt_n) compute(stage[d], d & 1);
+            load_w(stage[d], kt + DEPTH);
+            store_x((d + 1) & 1);
+            __syncthreads();
+        }
+    }
+
+    if (!active) return;
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) {
+        const int slot = sorted_ids[seg * blk + tt * 16 + c];
+        if (slot >= ns) continue;
+        const float wgt = (!GLU && topw) ? topw[slot] : 1.0f;
+        moe_store<GLU>(acc[0][tt], acc[1][tt], slot, q, u, rbA, rbB, haveB, y, y_f16, wgt, n);
+    }
+}
+
+#define MOE_DEC_KERNEL(NAME, G, SBF, GLU, XL, DEPTH)                                  \
+    extern "C" __global__ __launch_bounds__(512) void NAME(MOE_PARAMS) {              \
+        moe_dec_body<G, SBF, GLU, XL, DEPTH>(MOE_ARGS);                               \
+    }
+#define MOE_MM_KERNEL(NAME, G, SBF, GLU, TT, DEPTH)                                   \
+    extern "C" __global__ __launch_bounds__(512) void NAME(MOE_PARAMS) {              \
+        moe_mm_body<G, SBF, GLU, TT, DEPTH>(MOE_ARGS);                                \
+    }
+#define MOE_FAMILY(PFX, G, SBF)                              \
+    MOE_DEC_KERNEL(PFX##_dec_glu_x1, G, SBF, true, 1, 4)     \
+    MOE_DEC_KERNEL(PFX##_dec_glu_x4, G, SBF, true, 4, 3)     \
+    MOE_DEC_KERNEL(PFX##_dec_lin_x1, G, SBF, false, 1, 4)    \
+    MOE_DEC_KERNEL(PFX##_dec_lin_x4, G, SBF, false, 4, 3)    \
+    MOE_MM_KERNEL(PFX##_mm_glu_t1, G, SBF, true, 1, 4)       \
+    MOE_MM_KERNEL(PFX##_mm_glu_t2, G, SBF, true, 2, 4)       \
+    MOE_MM_KERNEL(PFX##_mm_glu_t3, G, SBF, true, 3, 4)       \
+    MOE_MM_KERNEL(PFX##_mm_glu_t4, G, SBF, true, 4, 4)       \
+    MOE_MM_KERNEL(PFX##_mm_lin_t1, G, SBF, false, 1, 4)      \
+    MOE_MM_KERNEL(PFX##_mm_lin_t2, G, SBF, false, 2, 4)      \
+    MOE_MM_KERNEL(PFX##_mm_lin_t3, G, SBF, false, 3, 4)      \
+    MOE_MM_KERNEL(PFX##_mm_lin_t4, G, SBF, false, 4, 4)
+
+MOE_FAMILY(w4a16_moe_g32_f16, 32, false)
+MOE_FAMILY(w4a16_moe_g32_bf16, 32, true)
+MOE_FAMILY(w4a16_moe_g128_f16, 128, false)
+MOE_FAMILY(w4a16_moe_g128_bf16, 128, true)
+
+// ---------------------------------------------------------------------------------------------------- routing
+// Softmax over all experts, k largest probabilities with ties to the lower index, weights renormalised by the
+// selected sum (w4a16_dec/mod.rs:168-185; device counterpart assets/moe.cu:686-759).  One wave per token, n <= 1024.
+extern "C" __global__ __launch_bounds__(256) void w4a16_moe_topk_t(const float* __restrict__ lg, int* __restrict__ idx,
+                                                                   float* __restrict__ wt, int t, int n, int k) {
+    const int lane = threadIdx.x & 63;
+    const int ti = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (ti >= t) return;
+    const float* l = lg + (size_t)ti * n;
+    float pv[16];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const int i = lane + 64 * j;
+        pv[j] = i < n ? l[i] : -INFINITY;
+        mx = fmaxf(mx, pv[j]);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        pv[j] = (lane + 64 * j) < n ? expf(pv[j] - mx) : -1.0f;  // -1 marks absent or already taken
+        if (pv[j] > 0.f) sum += pv[j];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+#pragma unroll
+    for (int j = 0; j < 16; j++)
+        if (pv[j] >= 0.f) pv[j] = pv[j] / sum;
+    float wsum = 0.f, mine = 0.f;  // lane r keeps the r-th selected probability
+    for (int r = 0; r < k; r++) {
+        float bv = -1.0f;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < 16; j++)
+            if (pv[j] > bv) {  // strict: the lower index wins inside a lane
+                bv = pv[j];
+                bi = lane + 64 * j;
+            }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off);
+            const int oi = __shfl_xor(bi, off);
+            if (ov > bv || (ov == bv && oi < bi)) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 16; j++)
+            if (lane + 64 * j == bi) pv[j] = -1.0f;
+        if (lane == 0) idx[(size_t)ti * k + r] = bi;
+        if (lane == (r & 63)) mine = bv;
+        wsum += bv;
+    }
+    if (lane < k) wt[(size_t)ti * k + lane] = mine / wsum;
+}
+
+// Stable counting sort of slots by expert with every expert's run padded to a multiple of `block`
+// (assets/moe.cu:860-908 + 1599-1633 in one launch).  One workgroup of 512 threads, n_exp <= 1024.
+//   sorted_ids: slot ids in expert order, padding = sentinel ns; expert_ids[b]: expert of segment b;
+//   num_post[0] = padded total, num_post[1] = number of distinct experts hit.
+// Wave w owns the contiguous slot range [w*chunk, (w+1)*chunk): per-wave counts, an exclusive prefix over the
+// waves per expert, a two-level scan over the experts' padded counts, then every wave places its slots in order.
+// An out-of-range expert id is dropped (its slot is never placed).
+#define MOE_ALIGN_WAVES 8
+#define MOE_ALIGN_KEEP 8  // 64-slot steps of a wave whose expert ids stay in registers between the two passes
+extern "C" __global__ __launch_bounds__(512) void w4a16_moe_align(const int* __restrict__ idx, int ns, int n_exp,
+                                                                  int block, int* __restrict__ sorted_ids,
+                                                                  int* __restrict__ expert_ids, int* __restrict__ num_post) {
+    __shared__ unsigned cnt[MOE_ALIGN_WAVES][1024];  // per wave count, then exclusive prefix over the waves
+    __shared__ unsigned tot[1024], poff[1024];
+    __shared__ unsigned wsum[MOE_ALIGN_WAVES], whit[MOE_ALIGN_WAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int i = tid; i < MOE_ALIGN_WAVES * n_exp; i += 512) cnt[i / n_exp][i % n_exp] = 0;
+    const int chunk = ((ns + MOE_ALIGN_WAVES * 64 - 1) / (MOE_ALIGN_WAVES * 64)) * 64;  // slots per wave, multiple of 64
+    const int j0 = wave * chunk, steps = chunk / 64;
+    int keep[MOE_ALIGN_KEEP];
+#pragma unroll
+    for (int s = 0; s < MOE_ALIGN_KEEP; s++) {
+        const int j = j0 + s * 64 + lane;
+        int e = (s < steps && j < ns) ? idx[j] : -1;
+        keep[s] = (unsigned)e < (unsigned)n_exp ? e : -1;
+    }
+    auto expert_of = [&](int s) -> int {
+        int e = -1;
+#pragma unroll
+        for (int i = 0; i < MOE_ALIGN_KEEP; i++)
+            if (i == s) e = keep[i];
+        if (s >= MOE_ALIGN_KEEP) {
+            const int j = j0 + s * 64 + lane;
+            e = j < ns ? idx[j] : -1;
+            if ((unsigned)e >= (unsigned)n_exp) e = -1;
+        }
+        return e;
+    };
+    __syncthreads();
+    for (int s = 0; s < steps; s++) {
+        const int e = expert_of(s);
+        if (e >= 0) atomicAdd(&cnt[wave][e], 1u);
+    }
+    __syncthreads();
+    // thread i owns experts 2i, 2i+1: totals, then a scan of the padded totals over all threads
+    unsigned padded[2], hits = 0, local = 0;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const int e = 2 * tid + h;
+        unsigned run = 0;
+        if (e < n_exp) {
+            for (int w = 0; w < MOE_ALIGN_WAVES; w++) {
+                const unsigned c = cnt[w][e];
+                cnt[w][e] = run;
+                run += c;
+            }
+            tot[e] = run;
+        }
+        padded[h] = ((run + block - 1) / block) * block;
+        hits += run != 0;
+        local += padded[h];
+    }
+    unsigned incl = local, hincl = hits;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned v = __shfl_up(incl, off), hv = __shfl_up(hincl, off);
+        if (lane >= off) {
+            incl += v;
+            hincl += hv;
+        }
+    }
+    if (lane == 63) {
+        wsum[wave] = incl;
+        whit[wave] = hincl;
+    }
+    __syncthreads();
+    unsigned base = 0, all = 0, allhit = 0;
+#pragma unroll
+    for (int w = 0; w < MOE_ALIGN_WAVES; w++) {
+        if (w < wave) base += wsum[w];
+        all += wsum[w];
+        allhit += whit[w];
+    }
+    if (tid == 0) {
+        num_post[0] = (int)all;
+        num_post[1] = (int)allhit;
+    }
+    unsigned pos = base + incl - local;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const int e = 2 * tid + h;
+        if (e < n_exp) {
+            poff[e] = pos;
+            const unsigned c = tot[e];
+            for (unsigned p = c; p < padded[h]; p++) sorted_ids[pos + p] = ns;
+            for (unsigned b = 0; b < padded[h] / block; b++) expert_ids[pos / block + b] = e;
+            pos += padded[h];
+        }
+    }
+    __syncthreads();
+    // placement in slot order: every wave walks its range 64 slots at a time; rank among equal experts in the step
+    for (int s = 0; s < steps; s++) {
+        const int e = expert_of(s);
+        unsigned rank = 0, same = 0;
+        for (int i = 0; i < 64; i++) {
+            const int ei = __shfl(e, i);
+            same += ei == e;
+            rank += (ei == e) && (i < lane);
+        }
+        if (e >= 0) sorted_ids[poff[e] + cnt[wave][e] + rank] = j0 + s * 64 + lane;
+        __syncthreads();
+        if (e >= 0 && rank + 1 == same) cnt[wave][e] += same;
+        __syncthreads();
+    }
+}
+
+// out[t][c] = sum over the token's k slots of f16 c2[slot][c], added in slot order in f32 (assets/moe.cu:1662-1674).
+// Eight columns per thread when h % 8 == 0 (16-byte loads), one otherwise.
+extern "C" __global__ __launch_bounds__(256) void w4a16_moe_topk_sum_f16(const uint16_t* __restrict__ c2,
+                                                                         float* __restrict__ out, int t, int h, int top_k) {
+    if ((h & 7) == 0) {
+        const size_t total = (size_t)t * h / 8;
+        for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+            const size_t r = (i * 8) / h, c = (i * 8) % h;
+            float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            for (int kk = 0; kk < top_k; kk++) {
+                const h8_t v = *reinterpret_cast<const h8_t*>(c2 + (r * top_k + kk) * h + c);
+#pragma unroll
+                for (int j = 0; j < 8; j++) acc[j] += (float)v[j];
+            }
+            f4_t* o = reinterpret_cast<f4_t*>(out + i * 8);
+            o[0] = (f4_t){acc[0], acc[1], acc[2], acc[3]};
+            o[1] = (f4_t){acc[4], acc[5], acc[6], acc[7]};
+        }
+        return;
+    }
+    const size_t total = (size_t)t * h;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / h, c = i % h;
+        float acc = 0.f;
+        for (int kk = 0; kk < top_k; kk++)
+            acc += (float)__builtin_bit_cast(_Float16, c2[(r * top_k + kk) * h + c]);
+        out[i] = acc;
+    }
+}

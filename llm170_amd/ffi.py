@@ -54,6 +54,24 @@ _SIGS = {
     "w4a16_bench_forward": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.c_size_t, C.c_uint64, C.c_uint64, C.c_size_t,
                                       C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.POINTER(C.c_float),
                                       C.POINTER(C.c_double)]),
+    "w4a16_upload_experts": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
+                                       C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t,
+                                       C.c_int]),
+    "w4a16_experts_info": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t),
+                                     C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_int)]),
+    "w4a16_experts_dequant_dump": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int, C.c_size_t, C.c_uint64]),
+    "w4a16_moe_topk_host": (C.c_int, [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p]),
+    "w4a16_moe_route": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint64, C.c_uint64]),
+    "w4a16_moe_align": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint64, C.c_uint64,
+                                  C.c_uint64]),
+    "w4a16_moe_ffn": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t, C.c_size_t,
+                                C.c_uint64]),
+    "w4a16_moe_scratch": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_size_t),
+                                    C.POINTER(C.c_size_t)]),
+    "w4a16_set_moe_shape": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
+    "w4a16_bench_moe": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.c_size_t, C.c_uint64, C.c_uint64, C.c_uint64,
+                                  C.c_size_t, C.c_size_t, C.c_uint64, C.c_size_t, C.c_size_t, C.POINTER(C.c_float),
+                                  C.POINTER(C.c_double)]),
 }
 
 _lib = None

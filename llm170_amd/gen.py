@@ -140,3 +140,18 @@ def make_linear(n, k, group, t, seed=GATE_SEED, x_dist="normal"):
     else:
         x = gate_x(n, k, t, seed)
     return q, s, x
+
+
+def make_experts(n_exp, h, n_ff, group, seed=GATE_SEED):
+    """Synthetic experts of one MoE layer: q13 u32 [E][2*n_ff][h/8] (gate rows then up rows), s13 u16 [E][2*n_ff][h/g],
+    q2 u32 [E][h][n_ff/8], s2 u16 [E][h][n_ff/g]; distributions as for a dense linear."""
+    q13 = weights_q(shape_seed(2 * n_ff, h, seed, 11), n_exp * 2 * n_ff, h).reshape(n_exp, 2 * n_ff, h // 8)
+    s13 = scales_f16(shape_seed(2 * n_ff, h, seed, 12), n_exp * 2 * n_ff, h, group).reshape(n_exp, 2 * n_ff, h // group)
+    q2 = weights_q(shape_seed(h, n_ff, seed, 13), n_exp * h, n_ff).reshape(n_exp, h, n_ff // 8)
+    s2 = scales_f16(shape_seed(h, n_ff, seed, 14), n_exp * h, n_ff, group).reshape(n_exp, h, n_ff // group)
+    return q13, s13, q2, s2
+
+
+def router_logits(t, n_exp, seed=GATE_SEED):
+    """Router logits f32 [t][n_exp], N(0,1)."""
+    return normal_f32(shape_seed(n_exp, t, seed, 15), (t, n_exp))

@@ -4,6 +4,8 @@
   Gptq4     <- Gptq4 (gemv / gemm)          crates/backend-gpu/src/rawcuda/gptq4.rs:72-190
   W4a16Dec  <- W4a16Dec linear entry points crates/backend-gpu/src/rawcuda/w4a16_dec/upload.rs:4-65,
                                             w4a16_dec/kernels/mod.rs:121-144
+               MoE entry points             w4a16_dec/upload.rs:1116-1235, w4a16_dec/mod.rs:168-185,
+                                            w4a16_dec/kernels/marlin_moe.rs:290-422
 
 Same names, argument meaning and error behaviour (errors surface as W4a16Error carrying the library's message).
 numpy arrays stand in for the Rust slices; device pointers are plain ints.
@@ -225,3 +227,69 @@ class W4a16Dec:
         ffi.check(self.cc.lib.w4a16_bench_forward(self.cc.h, arr, len(names), x_dev, y_dev, t, int(out_f16), path, warmup,
                                                   reps, C.byref(ms), C.byref(wall)))
         return ms.value, wall.value
+
+    # ---- MoE expert FFN
+    def upload_experts(self, name, q13, s13, q2, s2, n_experts, h, n_ff, group=32, scale_bf16=False):
+        """build_marlin_moe_arenas (upload.rs:1116-1235).  q13 u32 [E][2*n_ff][h/8] (gate rows then up rows),
+        s13 u16 [E][2*n_ff][h/group], q2 u32 [E][h][n_ff/8], s2 u16 [E][h][n_ff/group]."""
+        arrs = [np.ascontiguousarray(a) for a in (q13, s13, q2, s2)]
+        ffi.check(self.cc.lib.w4a16_upload_experts(self.cc.h, name.encode(), n_experts, _ptr(arrs[0]), arrs[0].nbytes,
+                                                   _ptr(arrs[1]), arrs[1].nbytes, _ptr(arrs[2]), arrs[2].nbytes,
+                                                   _ptr(arrs[3]), arrs[3].nbytes, h, n_ff, group, int(bool(scale_bf16))))
+
+    def experts_spec(self, name):
+        e, h, f, g = C.c_size_t(), C.c_size_t(), C.c_size_t(), C.c_size_t()
+        bf = C.c_int()
+        ffi.check(self.cc.lib.w4a16_experts_info(self.cc.h, name.encode(), C.byref(e), C.byref(h), C.byref(f),
+                                                 C.byref(g), C.byref(bf)))
+        return {"n_experts": e.value, "h": h.value, "n_ff": f.value, "group": g.value, "scale_bf16": bool(bf.value)}
+
+    def experts_dequant(self, name, which, expert):
+        spec = self.experts_spec(name)
+        n, k = (2 * spec["n_ff"], spec["h"]) if which == 0 else (spec["h"], spec["n_ff"])
+        p = self.cc.alloc(n * k * 4)
+        try:
+            ffi.check(self.cc.lib.w4a16_experts_dequant_dump(self.cc.h, name.encode(), which, expert, p))
+            return self.cc.d2h(p, (n, k), np.float32)
+        finally:
+            self.cc.free(p)
+
+    def moe_route(self, logits_dev, t, n_exp, top_k, idx_dev, wt_dev):
+        """w4a16_moe_topk_t (assets/moe.cu:686-759) on resident logits."""
+        ffi.check(self.cc.lib.w4a16_moe_route(self.cc.h, logits_dev, t, n_exp, top_k, idx_dev, wt_dev))
+
+    def moe_align(self, idx_dev, ns, n_exp, block, sorted_dev, expert_ids_dev, num_post_dev):
+        ffi.check(self.cc.lib.w4a16_moe_align(self.cc.h, idx_dev, ns, n_exp, block, sorted_dev, expert_ids_dev,
+                                              num_post_dev))
+
+    def moe_ffn(self, name, x_dev, idx_dev, wt_dev, t, top_k, y_dev):
+        """marlin_moe_ffn_dev (kernels/marlin_moe.rs:290-422)."""
+        ffi.check(self.cc.lib.w4a16_moe_ffn(self.cc.h, name.encode(), x_dev, idx_dev, wt_dev, t, top_k, y_dev))
+
+    def moe_scratch(self, which, dtype):
+        """Scratch buffer of the last moe_ffn call as a flat numpy array, plus the segment size used."""
+        p, nb, blk = C.c_uint64(), C.c_size_t(), C.c_size_t()
+        ffi.check(self.cc.lib.w4a16_moe_scratch(self.cc.h, which, C.byref(p), C.byref(nb), C.byref(blk)))
+        return self.cc.d2h(p.value, (nb.value // np.dtype(dtype).itemsize,), dtype), blk.value
+
+    def set_moe_shape(self, block=0, waves=0):
+        ffi.check(self.cc.lib.w4a16_set_moe_shape(self.cc.h, block, waves))
+
+    def bench_moe(self, names, x_dev, idx_dev, wt_dev, t, top_k, y_dev, reps, warmup=1):
+        arr = (C.c_char_p * len(names))(*[n.encode() for n in names])
+        ms, wall = C.c_float(), C.c_double()
+        ffi.check(self.cc.lib.w4a16_bench_moe(self.cc.h, arr, len(names), x_dev, idx_dev, wt_dev, t, top_k, y_dev,
+                                              warmup, reps, C.byref(ms), C.byref(wall)))
+        return ms.value, wall.value
+
+
+def moe_topk(logits, top_k):
+    """moe_topk (w4a16_dec/mod.rs:168-185) on the host: logits f32 [t][n_exp] -> (idx int32 [t][top_k], w f32)."""
+    logits = np.ascontiguousarray(logits, np.float32)
+    if logits.ndim == 1:
+        logits = logits[None, :]
+    t, n_exp = logits.shape
+    idx = np.empty((t, top_k), np.int32)
+    w = np.empty((t, top_k), np.float32)
+    ffi.check(ffi.load().w4a16_moe_topk_host(_ptr(logits), t, n_exp, top_k, _ptr(idx), _ptr(w)))
+    return idx, w

@@ -21,6 +21,10 @@
  *   orc_tree64 ............ math.fsum on exactly-summable inputs + a pairing-order vector that distinguishes orders
  *   orc_moe_topk .......... KATs qwen35/stages/moe.rs:135-155
  *   orc_exact_dot ......... exact-rational brute force (quant/exact.rs:77-135 precedent)
+ *   orc_moe_act_silu_f16 .. float64 evaluation of g/(1+exp(-g))*u within one f16 step; special cases g = 0, u = 0,
+ *                           large |g| (silu -> g, -> 0)
+ *   orc_moe_topk_sum_f16 .. numpy float32 sequential sum; exactly-summable inputs
+ *   orc_moe_align ......... numpy stable argsort by expert + padding arithmetic; tiny hand-worked case
  * No function here is "parity unpinned".
  */
 #include <math.h>
@@ -337,4 +341,57 @@ void orc_moe_topk(const float* logits, size_t n, size_t k, uint32_t* idx_out, fl
 uint16_t orc_silu_mul_f16(float g, float u) {
     float sg = g / (1.0f + expf(-g));
     return orc_f32_to_f16(sg * u);
+}
+
+/* ---- w4a16_moe_act_silu_f16 (crates/backend-gpu/src/rawcuda/assets/moe.cu:1649-1660): c13 is f16 [ns][2*n_ff],
+ * gate in columns 0..n_ff, up in n_ff..2*n_ff; act[r][c] = f16(silu(gate) * up) with f32 arithmetic. ---- */
+void orc_moe_act_silu_f16(const uint16_t* c13, size_t ns, size_t n_ff, uint16_t* act) {
+    for (size_t r = 0; r < ns; r++)
+        for (size_t c = 0; c < n_ff; c++) {
+            const float g = orc_half_to_f32(c13[r * 2 * n_ff + c]);
+            const float u = orc_half_to_f32(c13[r * 2 * n_ff + n_ff + c]);
+            act[r * n_ff + c] = orc_silu_mul_f16(g, u);
+        }
+}
+
+/* ---- w4a16_moe_topk_sum_f16 (assets/moe.cu:1662-1674): out[r][c] = sum over the token's top_k slots of
+ * f16 c2[(r*top_k + kk)][c], added in slot order in f32. ---- */
+void orc_moe_topk_sum_f16(const uint16_t* c2, size_t t, size_t h, size_t top_k, float* out) {
+    for (size_t r = 0; r < t; r++)
+        for (size_t c = 0; c < h; c++) {
+            float acc = 0.0f;
+            for (size_t kk = 0; kk < top_k; kk++) acc = acc + orc_half_to_f32(c2[(r * top_k + kk) * h + c]);
+            out[r * h + c] = acc;
+        }
+}
+
+/* ---- w4a16_moe_align2 + w4a16_moe_align_marlin (assets/moe.cu:860-908, 1599-1633): slots sorted by expert,
+ * stable in slot order; each expert's run padded to a multiple of `block` with the sentinel ns; expert_ids holds
+ * the expert of every block; returns the padded total (num_post). ---- */
+size_t orc_moe_align(const int32_t* idx, size_t ns, size_t n_exp, size_t block, int32_t* sorted_ids,
+                     int32_t* expert_ids) {
+    size_t* cnt = (size_t*)calloc(n_exp, sizeof(size_t));
+    size_t* base = (size_t*)calloc(n_exp, sizeof(size_t));
+    for (size_t j = 0; j < ns; j++) cnt[idx[j]]++;
+    size_t pos = 0;
+    for (size_t e = 0; e < n_exp; e++) {
+        base[e] = pos;
+        const size_t padded = (cnt[e] + block - 1) / block * block;
+        for (size_t p = 0; p < padded; p++) sorted_ids[pos + p] = (int32_t)ns;
+        for (size_t b = 0; b < padded / block; b++) expert_ids[pos / block + b] = (int32_t)e;
+        pos += padded;
+    }
+    memset(cnt, 0, n_exp * sizeof(size_t));
+    for (size_t j = 0; j < ns; j++) {
+        const size_t e = (size_t)idx[j];
+        sorted_ids[base[e] + cnt[e]++] = (int32_t)j;
+    }
+    free(cnt);
+    free(base);
+    return pos;
+}
+
+/* Array form of orc_f32_to_f16 (same routine, element by element). */
+void orc_f32_to_f16_array(const float* v, size_t n, uint16_t* out) {
+    for (size_t i = 0; i < n; i++) out[i] = orc_f32_to_f16(v[i]);
 }

@@ -53,6 +53,11 @@ def lib():
         L.orc_gemm_lane_sample.restype = C.c_int
         L.orc_moe_topk.argtypes, L.orc_moe_topk.restype = [f32p, sz, sz, u32p, f32p], None
         L.orc_silu_mul_f16.argtypes, L.orc_silu_mul_f16.restype = [C.c_float, C.c_float], C.c_uint16
+        L.orc_f32_to_f16_array.argtypes, L.orc_f32_to_f16_array.restype = [f32p, sz, u16p], None
+        i32p = C.POINTER(C.c_int32)
+        L.orc_moe_act_silu_f16.argtypes, L.orc_moe_act_silu_f16.restype = [u16p, sz, sz, u16p], None
+        L.orc_moe_topk_sum_f16.argtypes, L.orc_moe_topk_sum_f16.restype = [u16p, sz, sz, sz, f32p], None
+        L.orc_moe_align.argtypes, L.orc_moe_align.restype = [i32p, sz, sz, sz, i32p, i32p], sz
         _lib = L
     return _lib
 
@@ -85,8 +90,9 @@ def half_to_f32_bits_all():
 
 def f32_to_f16_array(v):
     v = _c(v, np.float32).ravel()
-    L = lib()
-    return np.fromiter((L.orc_f32_to_f16(float(x)) for x in v), dtype=np.uint16, count=v.size)
+    out = np.empty(v.size, np.uint16)
+    lib().orc_f32_to_f16_array(_p(v, C.c_float), v.size, _p(out, C.c_uint16))
+    return out
 
 
 def tree64(v):
@@ -186,3 +192,73 @@ def moe_topk(logits, k):
 
 def silu_mul_f16(g, u):
     return int(lib().orc_silu_mul_f16(float(np.float32(g)), float(np.float32(u))))
+
+
+def moe_act_silu_f16(c13, ns, n_ff):
+    """f16 bits [ns][2*n_ff] (gate | up) -> f16 bits [ns][n_ff]."""
+    c13 = _c(c13, np.uint16).reshape(ns, 2 * n_ff)
+    act = np.empty((ns, n_ff), np.uint16)
+    lib().orc_moe_act_silu_f16(_p(c13, C.c_uint16), ns, n_ff, _p(act, C.c_uint16))
+    return act
+
+
+def moe_topk_sum_f16(c2, t, h, top_k):
+    c2 = _c(c2, np.uint16).reshape(t * top_k, h)
+    out = np.empty((t, h), np.float32)
+    lib().orc_moe_topk_sum_f16(_p(c2, C.c_uint16), t, h, top_k, _p(out, C.c_float))
+    return out
+
+
+def moe_align(idx, n_exp, block):
+    """-> (sorted_ids int32 [num_post], expert_ids int32 [num_post/block], num_post)."""
+    idx = _c(idx, np.int32).ravel()
+    ns = idx.size
+    sorted_ids = np.empty(ns + n_exp * block, np.int32)
+    expert_ids = np.empty(ns // block + n_exp + 1, np.int32)
+    n_post = lib().orc_moe_align(_p(idx, C.c_int32), ns, n_exp, block, _p(sorted_ids, C.c_int32),
+                                 _p(expert_ids, C.c_int32))
+    return sorted_ids[:n_post].copy(), expert_ids[:n_post // block].copy(), int(n_post)
+
+
+def moe_topk_batch(logits, k):
+    logits = _c(logits, np.float32)
+    t = logits.shape[0]
+    idx = np.empty((t, k), np.int32)
+    w = np.empty((t, k), np.float32)
+    for i in range(t):
+        a, b = moe_topk(logits[i], k)
+        idx[i], w[i] = a.astype(np.int32), b
+    return idx, w
+
+
+def moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, scale_bf16=False, threads=1, act_in=None):
+    """The routed-expert FFN of the reference's device path (kernels/marlin_moe.rs:290-422) with every GEMM done by
+    the lane contract: per slot j (token j // top_k, expert idx[j])
+        c13 = f16(lane(W13[e], x[token]));  act = f16(silu(gate) * up)
+        c2  = f16(wt[j] * lane(W2[e], act));  y[token] = sum_k c2 in slot order (f32).
+    x: f16 bits [t][h]; idx int32 [t][top_k]; wt f32 [t][top_k]; q13 u32 [E][2*n_ff][h/8] ...
+    act_in (f16 bits [ns][n_ff]) replaces the first stage's result when given (stage-wise checks).
+    Returns dict(c13, act, c2, y)."""
+    x = _c(x, np.uint16).reshape(-1, h)
+    t, top_k = idx.shape
+    ns = t * top_k
+    flat = _c(idx, np.int32).ravel()
+    wflat = _c(wt, np.float32).ravel()
+    c13 = np.zeros((ns, 2 * n_ff), np.uint16)
+    c2 = np.zeros((ns, h), np.uint16)
+    act = np.zeros((ns, n_ff), np.uint16) if act_in is None else _c(act_in, np.uint16).reshape(ns, n_ff).copy()
+    order = np.argsort(flat, kind="stable")
+    bounds = np.flatnonzero(np.diff(flat[order], prepend=-1, append=1 << 30))
+    for b0, b1 in zip(bounds[:-1], bounds[1:]):
+        slots = order[b0:b1]
+        e = int(flat[slots[0]])
+        if act_in is None:
+            xs = x[slots // top_k]
+            y13 = gemm_lane(xs, len(slots), q13[e], s13[e], 2 * n_ff, h, group, scale_bf16, threads)
+            c13[slots] = f32_to_f16_array(y13).reshape(len(slots), 2 * n_ff)
+            act[slots] = moe_act_silu_f16(c13[slots], len(slots), n_ff)
+        y2 = gemm_lane(act[slots], len(slots), q2[e], s2[e], h, n_ff, group, scale_bf16, threads)
+        y2 = (y2 * wflat[slots][:, None]).astype(np.float32)
+        c2[slots] = f32_to_f16_array(y2).reshape(len(slots), h)
+    y = moe_topk_sum_f16(c2, t, h, top_k)
+    return {"c13": c13, "act": act, "c2": c2, "y": y}

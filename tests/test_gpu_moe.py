@@ -1,0 +1,248 @@
+"""GPU parity tests of the MoE expert FFN (grouped / ragged W4A16 GEMM) through the C ABI against the CPU oracle."""
+import numpy as np
+import pytest
+
+from llm170_amd import gen, ops
+from tests import parity
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def dec():
+    d = ops.W4a16Dec()
+    yield d
+    d.cc.close()
+
+
+def _f16(bits):
+    return np.asarray(bits, np.uint16).view(np.float16).astype(np.float32)
+
+
+def _bf16_scales(s):
+    return (gen.f16_bits_to_f32(s).view(np.uint32) >> 16).astype(np.uint16)
+
+
+SMALL = dict(E=8, h=256, n_ff=128, k=2)
+
+
+@pytest.fixture(scope="module")
+def small_experts(dec):
+    out = {}
+    for group in (32, 128):
+        for bf in (False, True):
+            q13, s13, q2, s2 = gen.make_experts(SMALL["E"], SMALL["h"], SMALL["n_ff"], group, seed=gen.GATE_SEED + group)
+            if bf:
+                s13, s2 = _bf16_scales(s13), _bf16_scales(s2)
+            name = "small_g%d_%s" % (group, "bf16" if bf else "f16")
+            dec.upload_experts(name, q13, s13, q2, s2, SMALL["E"], SMALL["h"], SMALL["n_ff"], group, bf)
+            out[(group, bf)] = (name, q13, s13, q2, s2)
+    return out
+
+
+# ------------------------------------------------------------------ arena re-layout, bit exact
+def test_experts_arena_dequant_bit_exact(dec, orc, small_experts):
+    for (group, bf), (name, q13, s13, q2, s2) in small_experts.items():
+        for e in (0, 3, SMALL["E"] - 1):
+            got = dec.experts_dequant(name, 0, e)
+            want = orc.dequant_matrix(q13[e], s13[e], 2 * SMALL["n_ff"], SMALL["h"], group, bf)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (group, bf, e, "w13")
+            got = dec.experts_dequant(name, 1, e)
+            want = orc.dequant_matrix(q2[e], s2[e], SMALL["h"], SMALL["n_ff"], group, bf)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (group, bf, e, "w2")
+
+
+# ------------------------------------------------------------------ routing on the device
+@pytest.mark.parametrize("t,n_exp,k", [(1, 128, 8), (4, 128, 8), (512, 128, 8), (7, 8, 2), (33, 200, 5), (3, 1024, 64)])
+def test_route_matches_host_rule(dec, orc, t, n_exp, k):
+    say("route", t, n_exp, k)
+    lg = gen.router_logits(t, n_exp)
+    cc = dec.cc
+    pl, pi, pw = cc.to_device(lg), cc.alloc(t * k * 4), cc.alloc(t * k * 4)
+    dec.moe_route(pl, t, n_exp, k, pi, pw)
+    idx, w = cc.d2h(pi, (t, k), np.int32), cc.d2h(pw, (t, k), np.float32)
+    for p in (pl, pi, pw):
+        cc.free(p)
+    oi, ow = orc.moe_topk_batch(lg, k)
+    assert np.array_equal(idx, oi)
+    assert np.allclose(w, ow, rtol=2e-6, atol=0)
+    assert np.allclose(w.sum(1), 1.0, atol=1e-6)
+
+
+def test_route_ties_go_to_lower_index(dec):
+    cc = dec.cc
+    lg = np.ones((2, 130), np.float32)
+    lg[1, 70] = 2.0
+    pl, pi, pw = cc.to_device(lg), cc.alloc(2 * 4 * 4), cc.alloc(2 * 4 * 4)
+    dec.moe_route(pl, 2, 130, 4, pi, pw)
+    idx = cc.d2h(pi, (2, 4), np.int32)
+    for p in (pl, pi, pw):
+        cc.free(p)
+    assert idx[0].tolist() == [0, 1, 2, 3] and idx[1].tolist() == [70, 0, 1, 2]
+
+
+# ------------------------------------------------------------------ align on the device
+@pytest.mark.parametrize("ns,n_exp,block", [(8, 128, 4), (32, 128, 4), (128, 128, 16), (4096, 128, 48), (4096, 128, 32),
+                                            (4096, 128, 64), (1000, 7, 64), (130, 1024, 16), (1, 1, 4), (777, 33, 16)])
+def test_align_matches_oracle(dec, orc, ns, n_exp, block):
+    say("align", ns, n_exp, block)
+    rng = np.random.default_rng(ns * 7 + n_exp)
+    idx = rng.integers(0, n_exp, ns).astype(np.int32)
+    if ns == 4096:
+        idx[:64] = 5  # one step of one wave entirely on one expert
+    cc = dec.cc
+    cap_s, cap_e = ns + n_exp * block, ns // block + n_exp + 1
+    pi, ps, pe, pn = cc.to_device(idx), cc.alloc(cap_s * 4), cc.alloc(cap_e * 4), cc.alloc(8)
+    dec.moe_align(pi, ns, n_exp, block, ps, pe, pn)
+    n_post, hit = cc.d2h(pn, (2,), np.int32)
+    s, e = cc.d2h(ps, (cap_s,), np.int32), cc.d2h(pe, (cap_e,), np.int32)
+    for p in (pi, ps, pe, pn):
+        cc.free(p)
+    ws, we, wn = orc.moe_align(idx, n_exp, block)
+    assert n_post == wn and hit == np.unique(idx).size
+    assert np.array_equal(s[:wn], ws) and np.array_equal(e[:wn // block], we)
+
+
+# ------------------------------------------------------------------ the FFN, stage by stage and end to end
+def _run_ffn(dec, name, x, idx, wt, t, k, h):
+    cc = dec.cc
+    px, pi, pw, py = cc.to_device(x), cc.to_device(idx), cc.to_device(wt), cc.alloc(t * h * 4)
+    dec.moe_ffn(name, px, pi, pw, t, k, py)
+    y = cc.d2h(py, (t, h), np.float32)
+    ns = t * k
+    spec = dec.experts_spec(name)
+    act, blk = dec.moe_scratch(3, np.uint16)
+    c2, _ = dec.moe_scratch(4, np.uint16)
+    for p in (px, pi, pw, py):
+        cc.free(p)
+    return y, act.reshape(ns, spec["n_ff"]), c2.reshape(ns, h), blk
+
+
+def _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, what, threads=8):
+    t, k = idx.shape
+    full = orc.moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, threads=threads)
+    # stage 1: act against the oracle's act.  The device's gate/up sums differ from the lane order by f32 rounding
+    # (about 1e-6 absolute here), so a few round to the neighbouring f16 before the activation, and a sum that
+    # cancelled to almost nothing moves by many of its own tiny f16 steps.  Tolerance: the device value must lie
+    # inside the envelope of silu(g')*u' over g', u' within ONE f16 step of the oracle's gate/up — the step taken at
+    # a magnitude clamped from below at rms/128, the rule of tests/parity.py — widened by 1.5 f16 steps of the
+    # result (final rounding, exp implementation); and nearly all elements must be identical.
+    g0 = full["c13"][:, :n_ff].view(np.float16).astype(np.float64)
+    u0 = full["c13"][:, n_ff:].view(np.float16).astype(np.float64)
+    rms = float(np.sqrt(np.mean(np.concatenate([g0.ravel(), u0.ravel()]) ** 2)))
+    dg = parity.f16_ulp(np.maximum(np.abs(g0), rms / parity.CLAMP_DIV))
+    du = parity.f16_ulp(np.maximum(np.abs(u0), rms / parity.CLAMP_DIV))
+    lo = np.full(g0.shape, np.inf)
+    hi = np.full(g0.shape, -np.inf)
+    for gs in (-1.0, 0.0, 1.0):
+        for us in (-1.0, 0.0, 1.0):
+            g1, u1 = g0 + gs * dg, u0 + us * du
+            v = g1 / (1.0 + np.exp(-g1)) * u1
+            lo, hi = np.minimum(lo, v), np.maximum(hi, v)
+    a = _f16(act).astype(np.float64)
+    pad = 1.5 * parity.f16_ulp(np.maximum(np.abs(lo), np.abs(hi)))
+    bad = (a < lo - pad) | (a > hi + pad)
+    assert not bad.any(), (what, "act outside the one-step envelope", int(bad.sum()))
+    same = float(np.mean(act == full["act"]))
+    assert same > 0.97, (what, "act identical fraction", same)
+    # stage 2: c2 from the device's own act, against the oracle run on that same act
+    st2 = orc.moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, threads=threads, act_in=act)
+    m2 = parity.assert_close(_f16(c2), _f16(st2["c2"]), what + " c2")
+    # stage 3: the slot-order f32 sum of the device's c2 is exact arithmetic on f16 inputs -> bit for bit
+    y3 = orc.moe_topk_sum_f16(c2, t, h, k)
+    assert np.array_equal(y.view(np.uint32), y3.view(np.uint32)), what + " sum"
+    # end to end against the oracle's independent run
+    m = parity.compare(y, full["y"])
+    assert m["rel_l2"] <= parity.REL_L2_TOL, (what, m)
+    return same, m2, m
+
+
+@pytest.mark.parametrize("group,bf", [(32, False), (32, True), (128, False), (128, True)])
+@pytest.mark.parametrize("t", [1, 3, 4, 9, 16, 40, 70, 200])
+def test_moe_ffn_small(dec, orc, small_experts, group, bf, t):
+    say("moe_ffn small", group, bf, t)
+    name, q13, s13, q2, s2 = small_experts[(group, bf)]
+    E, h, n_ff, k = SMALL["E"], SMALL["h"], SMALL["n_ff"], SMALL["k"]
+    x = gen.normal_f16(1000 + t, (t, h))
+    idx, wt = ops.moe_topk(gen.router_logits(t, E, seed=t), k)
+    y, act, c2, blk = _run_ffn(dec, name, x, idx, wt, t, k, h)
+    _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, "small g%d bf%d t%d blk%d" % (group, bf, t, blk))
+
+
+@pytest.mark.parametrize("block,waves", [(4, 1), (4, 2), (16, 1), (16, 4), (32, 4), (48, 8), (64, 4)])
+def test_moe_ffn_launch_shapes_agree(dec, orc, small_experts, block, waves):
+    """Every segment size and wave count computes the same FFN (t small enough for the 4-slot segments)."""
+    say("moe shapes", block, waves)
+    name, q13, s13, q2, s2 = small_experts[(32, False)]
+    E, h, n_ff, k = SMALL["E"], SMALL["h"], SMALL["n_ff"], SMALL["k"]
+    t = 4 if block == 4 else 13 if block == 16 else 90
+    x = gen.normal_f16(77, (t, h))
+    idx, wt = ops.moe_topk(gen.router_logits(t, E, seed=3), k)
+    dec.set_moe_shape(block, waves)
+    try:
+        y, act, c2, blk = _run_ffn(dec, name, x, idx, wt, t, k, h)
+    finally:
+        dec.set_moe_shape(0, 0)
+    assert blk == block
+    _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, 32, False, "shape blk%d w%d" % (block, waves))
+
+
+def test_moe_ffn_unused_experts_and_hot_expert(dec, orc, small_experts):
+    """Routing that leaves experts empty and sends every token to one expert (runs longer than one segment)."""
+    name, q13, s13, q2, s2 = small_experts[(32, False)]
+    E, h, n_ff, k = SMALL["E"], SMALL["h"], SMALL["n_ff"], SMALL["k"]
+    t = 100
+    x = gen.normal_f16(5, (t, h))
+    idx = np.empty((t, k), np.int32)
+    idx[:, 0] = 6
+    idx[:, 1] = np.arange(t) % 2  # experts 2..5, 7 never chosen
+    wt = np.full((t, k), 0.5, np.float32)
+    y, act, c2, blk = _run_ffn(dec, name, x, idx, wt, t, k, h)
+    _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, 32, False, "hot expert")
+
+
+# ------------------------------------------------------------------ the 35B-A3B layer shape: 128 experts, top-8
+@pytest.fixture(scope="module")
+def full_experts(dec):
+    E, h, n_ff, g = 128, 2048, 768, 32
+    q13, s13, q2, s2 = gen.make_experts(E, h, n_ff, g)
+    dec.upload_experts("a3b", q13, s13, q2, s2, E, h, n_ff, g, False)
+    return "a3b", q13, s13, q2, s2
+
+
+@pytest.mark.parametrize("t", [1, 4, 512])
+def test_moe_ffn_full_shape(dec, orc, full_experts, t):
+    say("moe_ffn full", t)
+    name, q13, s13, q2, s2 = full_experts
+    E, h, n_ff, k = 128, 2048, 768, 8
+    x = gen.normal_f16(4242 + t, (t, h))
+    lg = gen.router_logits(t, E)
+    cc = dec.cc
+    pl, pi, pw = cc.to_device(lg), cc.alloc(t * k * 4), cc.alloc(t * k * 4)
+    dec.moe_route(pl, t, E, k, pi, pw)
+    idx, wt = cc.d2h(pi, (t, k), np.int32), cc.d2h(pw, (t, k), np.float32)
+    for p in (pl, pi, pw):
+        cc.free(p)
+    assert np.array_equal(idx, ops.moe_topk(lg, k)[0])
+    y, act, c2, blk = _run_ffn(dec, name, x, idx, wt, t, k, h)
+    same, m2, m = _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, 32, False, "a3b t%d" % t, threads=16)
+    say("  blk", blk, "act identical", same, "c2", m2["rel_l2"], m2["max_ulp"], "y rel_l2", m["rel_l2"])
+
+
+def test_moe_errors(dec, small_experts):
+    name = small_experts[(32, False)][0]
+    with pytest.raises(ops.W4a16Error):
+        dec.moe_ffn("nope", 1, 1, 1, 1, 2, 1)
+    with pytest.raises(ops.W4a16Error):
+        dec.moe_ffn(name, 0, 1, 1, 1, 2, 1)
+    with pytest.raises(ops.W4a16Error):
+        dec.moe_ffn(name, 1, 1, 1, 1, 99, 1)
+    with pytest.raises(ops.W4a16Error):
+        dec.upload_experts("bad", np.zeros(4, np.uint32), np.zeros(4, np.uint16), np.zeros(4, np.uint32),
+                           np.zeros(4, np.uint16), 2, 256, 128, 32, False)
+    with pytest.raises(ops.W4a16Error):
+        dec.set_moe_shape(5, 0)
