@@ -220,6 +220,41 @@ int w4a16_bench_moe(w4a16_ctx* ctx, const char* const* names, size_t n_names, ui
                     uint64_t wt_dev, size_t t, size_t top_k, uint64_t y_dev, size_t warmup, size_t reps,
                     float* ms_events, double* ms_wall);
 
+/* ------------------------------------------------------------------------------------------------------------
+ * Layer chain: the linears of a dense decoder layer run back to back with the elementwise glue between them
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* Register a linear whose operands are generated on the device from the SplitMix64 streams of the reference's
+ * parity gate (crates/server/src/probes/w4a16/gates.rs:182-196): q word i = low 32 bits of output i of stream
+ * seed_q; scale i = f16(lo + (hi - lo) * u_i), u_i = (output i of stream seed_s >> 40) / 2^24.  Same result as
+ * uploading those operands from the host; exists so that tens of GB of synthetic layers need no host generation. */
+int w4a16_upload_lin_synth(w4a16_ctx* ctx, const char* name, size_t n, size_t k, size_t group, uint64_t seed_q,
+                           uint64_t seed_s, float lo, float hi);
+
+/* RMS rescale of t rows to unit mean square, emitting f16 (the part of norm_resid, assets/norm.cu:4-48, that a chain
+ * of linears needs: no residual, no weight): out[r][c] = f16(v[r*ld + c] * inv_r), inv_r = f32(1/sqrt(ms_r + 1e-6)),
+ * c < ncols <= ld.  The sum of squares is taken in f64 in a fixed order (256 strided partials, pairwise fold), so a
+ * CPU restatement is bit-identical. */
+int w4a16_rms_rescale_f16(w4a16_ctx* ctx, uint64_t v_f32_dev, size_t ld, size_t ncols, size_t t, uint64_t out_f16_dev);
+/* ew (assets/ew.cu:9-32): out[r][c] = f16(silu(gu[r][c]) * gu[r][n_ff + c]) for gu f32 [t][2*n_ff], f32 arithmetic. */
+int w4a16_silu_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_ff, size_t t, uint64_t out_f16_dev);
+
+/* chain_device_body (w4a16_dec/chains.rs:195-304) reduced to its linears: for layer l = layer0 .. layer0+n_layers-1,
+ * with the linears registered as "<prefix>.<l>.attn_qkv", ".attn_output", ".ffn_gate_up", ".ffn_down":
+ *     a = rms_f16(qkv(x)[:, :hidden])      (stands in for the token mixer)
+ *     b = rms_f16(attn_output(a))
+ *     c = silu_mul_f16(ffn_gate_up(b))     (gate = columns 0..n_ff, up = n_ff..2 n_ff)
+ *     x = rms_f16(ffn_down(c))
+ * x_dev / y_dev: f16 [t][hidden], hidden = k of attn_qkv.  Every linear goes through w4a16_lin_forward (f32 output).
+ * No host synchronisation. */
+int w4a16_chain_forward(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers, uint64_t x_dev, size_t t,
+                        uint64_t y_dev);
+/* Timed chain passes (decode_bench, w4a16_dec/probe.rs:1123-1289): `warmup` untimed then `reps` timed passes over
+ * layers 0..n_layers-1.  use_graph != 0 captures one pass into a HIP graph and times graph launches
+ * (forward_graph, w4a16_dec/graphs.rs). */
+int w4a16_bench_chain(w4a16_ctx* ctx, const char* prefix, size_t n_layers, uint64_t x_dev, size_t t, uint64_t y_dev,
+                      size_t warmup, size_t reps, int use_graph, float* ms_events, double* ms_wall);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,164 @@
+// Layer chain of libw4a16hip.so: device-generated synthetic linears, the elementwise glue, and the decoder-layer
+// sequence of linears.  Stands in for chain_device_body (w4a16_dec/chains.rs:195-304), norm_resid_dev / ew_dev_fused
+// (the glue launches around it) and decode_bench (w4a16_dec/probe.rs:1123-1289).
+#include <algorithm>
+#include <chrono>
+#include <cmath>
+#include <cstring>
+
+#include "w4a16_internal.h"
+
+static inline unsigned ceil_div(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+
+extern "C" int w4a16_upload_lin_synth(w4a16_ctx* ctx, const char* name, size_t n, size_t k, size_t group,
+                                      uint64_t seed_q, uint64_t seed_s, float lo, float hi) {
+    if (!ctx || !name) return w4_fail(W4A16_ERR_ARG, "upload_lin_synth: null argument");
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    if (group != 128 && group != 32)
+        return w4_fail(W4A16_ERR_UNSUPPORTED, "gptq4: unsupported combination group=%zu scale_bf16=0", group);
+    if (n == 0 || k == 0 || k % group != 0 || n > 0x7fffffffu || k > 0x7fffffffu)
+        return w4_fail(W4A16_ERR_SHAPE, "upload_lin_synth %s: n%zu k%zu g%zu contract", name, n, k, group);
+    if (!(lo > 0.0f) || !(hi >= lo) || !std::isfinite(hi) || hi > 65504.0f)
+        return w4_fail(W4A16_ERR_ARG, "upload_lin_synth %s: scale range [%g, %g) must be positive and finite in f16", name,
+                       (double)lo, (double)hi);
+    W4Lin L;
+    L.n = n;
+    L.k = k;
+    L.group = group;
+    L.scale_bf16 = 0;
+    L.scales_regular = true;
+    unsigned long long words = (unsigned long long)n * (k / 8), scales = (unsigned long long)n * (k / group);
+    int rc = w4a16_alloc(ctx, words * 4, &L.q_raw);
+    if (!rc) rc = w4a16_alloc(ctx, scales * 2, &L.s_raw);
+    if (!rc) {
+        unsigned long long sq = seed_q, ss = seed_s;
+        float span = hi - lo;
+        void* pq[] = {&L.q_raw, &words, &sq};
+        rc = w4_launch(ctx, "w4a16_synth_q", std::min<unsigned>(ceil_div(words, 256), 65536), 1, 256, 0, pq);
+        void* ps[] = {&L.s_raw, &scales, &ss, &lo, &span};
+        if (!rc) rc = w4_launch(ctx, "w4a16_synth_s", std::min<unsigned>(ceil_div(scales, 256), 65536), 1, 256, 0, ps);
+    }
+    if (rc) {
+        const std::string keep = w4_err_save();
+        (void)w4a16_free(ctx, L.q_raw);
+        (void)w4a16_free(ctx, L.s_raw);
+        w4_err_restore(keep);
+        return rc;
+    }
+    return w4_register_lin(ctx, name, L);
+}
+
+extern "C" int w4a16_rms_rescale_f16(w4a16_ctx* ctx, uint64_t v_f32_dev, size_t ld, size_t ncols, size_t t,
+                                     uint64_t out_f16_dev) {
+    if (!ctx || !v_f32_dev || !out_f16_dev) return w4_fail(W4A16_ERR_ARG, "rms_rescale: null argument");
+    if (t == 0 || ncols == 0 || ncols > ld || ld > 0x7fffffffu || t > 0x7fffffffu)
+        return w4_fail(W4A16_ERR_SHAPE, "rms_rescale: t=%zu ncols=%zu ld=%zu", t, ncols, ld);
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    int ldi = (int)ld, nc = (int)ncols;
+    void* p[] = {&v_f32_dev, &ldi, &nc, &out_f16_dev};
+    return w4_launch(ctx, "w4a16_rms_rescale_f16", (unsigned)t, 1, 256, 0, p);
+}
+
+extern "C" int w4a16_silu_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_ff, size_t t, uint64_t out_f16_dev) {
+    if (!ctx || !gu_f32_dev || !out_f16_dev) return w4_fail(W4A16_ERR_ARG, "silu_mul: null argument");
+    if (t == 0 || n_ff == 0 || n_ff > 0x3fffffffu || t > 0x7fffffffu)
+        return w4_fail(W4A16_ERR_SHAPE, "silu_mul: t=%zu n_ff=%zu", t, n_ff);
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    int nf = (int)n_ff, ti = (int)t;
+    void* p[] = {&gu_f32_dev, &nf, &ti, &out_f16_dev};
+    return w4_launch(ctx, "w4a16_silu_mul_f16", std::min<unsigned>(ceil_div(t * n_ff, 256), 4096), 1, 256, 0, p);
+}
+
+extern "C" int w4a16_chain_forward(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers, uint64_t x_dev,
+                                   size_t t, uint64_t y_dev) {
+    if (!ctx || !prefix || !x_dev || !y_dev) return w4_fail(W4A16_ERR_ARG, "chain_forward: null argument");
+    if (n_layers == 0 || t == 0) return w4_fail(W4A16_ERR_SHAPE, "chain_forward: n_layers=%zu t=%zu", n_layers, t);
+    W4ChainScratch& S = ctx->chain;
+    uint64_t cur = x_dev;
+    for (size_t l = layer0; l < layer0 + n_layers; l++) {
+        char nm[4][160];
+        const char* role[4] = {"attn_qkv", "attn_output", "ffn_gate_up", "ffn_down"};
+        W4Lin* L[4];
+        for (int i = 0; i < 4; i++) {
+            snprintf(nm[i], sizeof nm[i], "%s.%zu.%s", prefix, l, role[i]);
+            W4_TRY(w4_find_lin(ctx, nm[i], &L[i]));
+        }
+        const size_t hidden = L[0]->k, n_ff = L[3]->k;
+        if (L[0]->n < hidden || L[1]->k != hidden || L[1]->n != hidden || L[2]->k != hidden || L[2]->n != 2 * n_ff ||
+            L[3]->n != hidden)
+            return w4_fail(W4A16_ERR_SHAPE, "chain_forward %s.%zu: linears do not chain (hidden %zu, n_ff %zu)", prefix, l,
+                           hidden, n_ff);
+        const size_t widest = std::max(std::max(L[0]->n, L[2]->n), hidden);
+        W4_TRY(w4_ensure(ctx, &S.y32, &S.y32_cap, t * widest * 4));
+        W4_TRY(w4_ensure(ctx, &S.h16a, &S.h16a_cap, t * hidden * 2));
+        W4_TRY(w4_ensure(ctx, &S.h16b, &S.h16b_cap, t * n_ff * 2));
+        const bool last = l + 1 == layer0 + n_layers;
+        uint64_t out = y_dev;
+        if (!last) {
+            const int pp = (int)(l & 1);
+            W4_TRY(w4_ensure(ctx, &S.ping[pp], &S.ping_cap[pp], t * hidden * 2));
+            out = S.ping[pp];
+        }
+        W4_TRY(w4a16_lin_forward(ctx, nm[0], cur, S.y32, t, 0, W4A16_PATH_AUTO));
+        W4_TRY(w4a16_rms_rescale_f16(ctx, S.y32, L[0]->n, hidden, t, S.h16a));
+        W4_TRY(w4a16_lin_forward(ctx, nm[1], S.h16a, S.y32, t, 0, W4A16_PATH_AUTO));
+        W4_TRY(w4a16_rms_rescale_f16(ctx, S.y32, hidden, hidden, t, S.h16a));
+        W4_TRY(w4a16_lin_forward(ctx, nm[2], S.h16a, S.y32, t, 0, W4A16_PATH_AUTO));
+        W4_TRY(w4a16_silu_mul_f16(ctx, S.y32, n_ff, t, S.h16b));
+        W4_TRY(w4a16_lin_forward(ctx, nm[3], S.h16b, S.y32, t, 0, W4A16_PATH_AUTO));
+        W4_TRY(w4a16_rms_rescale_f16(ctx, S.y32, hidden, hidden, t, out));
+        cur = out;
+    }
+    return 0;
+}
+
+extern "C" int w4a16_bench_chain(w4a16_ctx* ctx, const char* prefix, size_t n_layers, uint64_t x_dev, size_t t,
+                                 uint64_t y_dev, size_t warmup, size_t reps, int use_graph, float* ms_events,
+                                 double* ms_wall) {
+    if (!ctx || !prefix || reps == 0) return w4_fail(W4A16_ERR_ARG, "bench_chain: null argument");
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    // one untimed pass always runs first: it sizes the scratch, which must not happen while capturing
+    for (size_t i = 0; i < std::max<size_t>(warmup, 1); i++)
+        W4_TRY(w4a16_chain_forward(ctx, prefix, 0, n_layers, x_dev, t, y_dev));
+    W4_TRY(w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"));
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int rc = 0;
+    if (use_graph) {
+        rc = w4_hip(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+        if (!rc) {
+            int frc = w4a16_chain_forward(ctx, prefix, 0, n_layers, x_dev, t, y_dev);
+            const std::string keep = w4_err_save();
+            rc = w4_hip(hipStreamEndCapture(ctx->stream, &graph), "hipStreamEndCapture");
+            if (frc) {
+                w4_err_restore(keep);
+                rc = frc;
+            }
+        }
+        if (!rc) rc = w4_hip(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
+        if (!rc) rc = w4_hip(hipGraphLaunch(exec, ctx->stream), "hipGraphLaunch");  // one untimed replay
+        if (!rc) rc = w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    }
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (!rc) rc = w4_hip(hipEventCreate(&e0), "hipEventCreate");
+    if (!rc) rc = w4_hip(hipEventCreate(&e1), "hipEventCreate");
+    auto w0 = std::chrono::steady_clock::now();
+    if (!rc) rc = w4_hip(hipEventRecord(e0, ctx->stream), "hipEventRecord");
+    for (size_t i = 0; i < reps && !rc; i++)
+        rc = use_graph ? w4_hip(hipGraphLaunch(exec, ctx->stream), "hipGraphLaunch")
+                       : w4a16_chain_forward(ctx, prefix, 0, n_layers, x_dev, t, y_dev);
+    if (!rc) rc = w4_hip(hipEventRecord(e1, ctx->stream), "hipEventRecord");
+    if (!rc) rc = w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    auto w1 = std::chrono::steady_clock::now();
+    float ms = 0.f;
+    if (!rc) rc = w4_hip(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+    if (ms_events) *ms_events = ms;
+    if (ms_wall) *ms_wall = std::chrono::duration<double, std::milli>(w1 - w0).count();
+    const std::string keep = w4_err_save();
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    if (rc) w4_err_restore(keep);
+    return rc;
+}

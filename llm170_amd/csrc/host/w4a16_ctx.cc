@@ -62,6 +62,8 @@ static const char* const kDecodeSyms[] = {
 static const char* const kPrefillSyms[] = {"w4a16_prefill_g128_f16", "w4a16_prefill_g128_bf16", "w4a16_prefill_g32_f16",
                                            "w4a16_prefill_g32_bf16", nullptr};
 static const char* const kUtilSyms[] = {"w4a16_fill0_u32", "w4a16_copy_u4", nullptr};
+static const char* const kGlueSyms[] = {"w4a16_rms_rescale_f16", "w4a16_silu_mul_f16", "w4a16_synth_q", "w4a16_synth_s",
+                                        nullptr};
 #define W4_MOE_FAMILY(P)                                                                                      \
     P "_dec_glu_x1", P "_dec_glu_x4", P "_dec_lin_x1", P "_dec_lin_x4", P "_mm_glu_t1", P "_mm_glu_t2",       \
         P "_mm_glu_t3", P "_mm_glu_t4", P "_mm_lin_t1", P "_mm_lin_t2", P "_mm_lin_t3", P "_mm_lin_t4"
@@ -84,6 +86,7 @@ static const W4Asset kAssets[] = {
     {"decode", kDecodeSyms},
     {"prefill", kPrefillSyms},
     {"moe", kMoeSyms},
+    {"glue", kGlueSyms},
     {"util", kUtilSyms},
 };
 static const size_t kAssetCount = sizeof kAssets / sizeof kAssets[0];

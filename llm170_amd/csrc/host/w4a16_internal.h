@@ -41,6 +41,12 @@ struct W4MoeScratch {
     size_t block = 0;
 };
 
+// Scratch of the layer chain, grown on demand (reference: dchain / dx16 / dy buffers, w4a16_dec/buffers.rs).
+struct W4ChainScratch {
+    uint64_t y32 = 0, h16a = 0, h16b = 0, ping[2] = {0, 0};
+    size_t y32_cap = 0, h16a_cap = 0, h16b_cap = 0, ping_cap[2] = {0, 0};
+};
+
 struct w4a16_event {
     hipEvent_t ev;
 };
@@ -56,6 +62,7 @@ struct w4a16_ctx {
     std::map<std::string, W4Lin> lins;
     std::map<std::string, W4Experts> experts;
     W4MoeScratch moe;
+    W4ChainScratch chain;
     int moe_block = 0, moe_waves = 0;  // 0 = automatic
     int decode_rows_per_wave = 0, decode_waves_per_block = 0;  // 0 = automatic
     int cu_count = 0;
@@ -68,6 +75,10 @@ std::string w4_err_save();
 void w4_err_restore(const std::string& msg);
 int w4_launch(w4a16_ctx* ctx, const char* symbol, unsigned gx, unsigned gy, unsigned block, unsigned shmem,
               void** params);
+
+int w4_register_lin(w4a16_ctx* ctx, const char* name, W4Lin& L);
+int w4_find_lin(w4a16_ctx* ctx, const char* name, W4Lin** out);
+int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes);
 
 #define W4_TRY(expr)          \
     do {                      \

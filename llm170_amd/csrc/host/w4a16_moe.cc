@@ -185,7 +185,7 @@ extern "C" int w4a16_moe_align(w4a16_ctx* ctx, uint64_t idx_dev, size_t ns, size
 }
 
 // ------------------------------------------------------------------------------------------------ FFN
-static int ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes) {
+int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes) {
     if (bytes <= *cap) return 0;
     if (*buf) W4_TRY(w4a16_sync(ctx));  // earlier launches may still read the old buffer
     (void)w4a16_free(ctx, *buf);
@@ -261,12 +261,12 @@ extern "C" int w4a16_moe_ffn(w4a16_ctx* ctx, const char* name, uint64_t x_dev, u
     S.expert_len = (ns / block + E->n_exp + 1) * 4;
     S.act_len = ns * E->n_ff * 2;
     S.c2_len = ns * E->h * 2;
-    W4_TRY(ensure(ctx, &S.sorted, &S.sorted_cap, S.sorted_len));
-    W4_TRY(ensure(ctx, &S.expert_ids, &S.expert_cap, S.expert_len));
+    W4_TRY(w4_ensure(ctx, &S.sorted, &S.sorted_cap, S.sorted_len));
+    W4_TRY(w4_ensure(ctx, &S.expert_ids, &S.expert_cap, S.expert_len));
     size_t np_cap = S.num_post ? 8 : 0;
-    W4_TRY(ensure(ctx, &S.num_post, &np_cap, 8));
-    W4_TRY(ensure(ctx, &S.act, &S.act_cap, S.act_len));
-    W4_TRY(ensure(ctx, &S.c2, &S.c2_cap, S.c2_len));
+    W4_TRY(w4_ensure(ctx, &S.num_post, &np_cap, 8));
+    W4_TRY(w4_ensure(ctx, &S.act, &S.act_cap, S.act_len));
+    W4_TRY(w4_ensure(ctx, &S.c2, &S.c2_cap, S.c2_len));
     W4_TRY(w4a16_moe_align(ctx, idx_dev, ns, E->n_exp, block, S.sorted, S.expert_ids, S.num_post));
     // gate|up with the SiLU*up epilogue: slot j reads token j / top_k
     W4_TRY(launch_moe_gemm(ctx, *E, true, x_dev, t, top_k, S.act, 1, 0, ns, block, max_segs));

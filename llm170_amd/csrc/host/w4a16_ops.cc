@@ -169,14 +169,27 @@ extern "C" int w4a16_upload_lin(w4a16_ctx* ctx, const char* name, const void* q,
     if (!rc) rc = w4a16_alloc(ctx, slen_bytes, &L.s_raw);
     if (!rc) rc = w4a16_h2d(ctx, L.q_raw, q, qlen_bytes);
     if (!rc) rc = w4a16_h2d(ctx, L.s_raw, s, slen_bytes);
-    if (!rc && k % 128 == 0) {
-        L.row_blocks = (n + 15) / 16;
-        const size_t kt_n = k / 128, kg_n = k / group;
+    if (rc) {
+        const std::string keep = w4_err_save();
+        free_lin(ctx, L);
+        w4_err_restore(keep);
+        return rc;
+    }
+    return w4_register_lin(ctx, name, L);
+}
+
+// Second half of a registration: build the tiled copy from the as-given operands already on the device and enter
+// the linear under its name.  Frees L's buffers on failure.
+int w4_register_lin(w4a16_ctx* ctx, const char* name, W4Lin& L) {
+    int rc = 0;
+    if (L.k % 128 == 0) {
+        L.row_blocks = (L.n + 15) / 16;
+        const size_t kt_n = L.k / 128, kg_n = L.k / L.group;
         const size_t qt_bytes = L.row_blocks * kt_n * 1024, st_bytes = L.row_blocks * kg_n * 16 * 2;
         rc = w4a16_alloc(ctx, qt_bytes, &L.q_tiled);
         if (!rc) rc = w4a16_alloc(ctx, st_bytes, &L.s_tiled);
         if (!rc) {
-            int ni = (int)n, ki = (int)k, rbi = (int)L.row_blocks, kgi = (int)kg_n;
+            int ni = (int)L.n, ki = (int)L.k, rbi = (int)L.row_blocks, kgi = (int)kg_n;
             void* pq[] = {&L.q_raw, &L.q_tiled, &ni, &ki, &rbi};
             rc = w4_launch(ctx, "w4a16_tile_q", ceil_div(qt_bytes / 4, 256), 1, 256, 0, pq);
             void* ps[] = {&L.s_raw, &L.s_tiled, &ni, &kgi, &rbi};
@@ -196,7 +209,7 @@ extern "C" int w4a16_upload_lin(w4a16_ctx* ctx, const char* name, const void* q,
     return 0;
 }
 
-static int find_lin(w4a16_ctx* ctx, const char* name, W4Lin** out) {
+int w4_find_lin(w4a16_ctx* ctx, const char* name, W4Lin** out) {
     if (!ctx || !name) return w4_fail(W4A16_ERR_ARG, "lin: null argument");
     auto it = ctx->lins.find(name);
     if (it == ctx->lins.end()) return w4_fail(W4A16_ERR_NOT_FOUND, "lin %s: not registered", name);
@@ -206,7 +219,7 @@ static int find_lin(w4a16_ctx* ctx, const char* name, W4Lin** out) {
 
 extern "C" int w4a16_lin_drop_raw(w4a16_ctx* ctx, const char* name) {
     W4Lin* L = nullptr;
-    W4_TRY(find_lin(ctx, name, &L));
+    W4_TRY(w4_find_lin(ctx, name, &L));
     if (!L->q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "lin %s: no tiled copy, the operands as given must stay", name);
     W4_TRY(w4a16_free(ctx, L->q_raw));
     W4_TRY(w4a16_free(ctx, L->s_raw));
@@ -217,7 +230,7 @@ extern "C" int w4a16_lin_drop_raw(w4a16_ctx* ctx, const char* name) {
 extern "C" int w4a16_lin_info(w4a16_ctx* ctx, const char* name, size_t* n, size_t* k, size_t* group, int* scale_bf16,
                               int* has_tiled, int* has_raw) {
     W4Lin* L = nullptr;
-    W4_TRY(find_lin(ctx, name, &L));
+    W4_TRY(w4_find_lin(ctx, name, &L));
     if (n) *n = L->n;
     if (k) *k = L->k;
     if (group) *group = L->group;
@@ -231,7 +244,7 @@ extern "C" int w4a16_lin_info(w4a16_ctx* ctx, const char* name, size_t* n, size_
 extern "C" int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16,
                                  int path) {
     W4Lin* L = nullptr;
-    W4_TRY(find_lin(ctx, name, &L));
+    W4_TRY(w4_find_lin(ctx, name, &L));
     if (!x_dev || !y_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward %s: null operand or t=0", name);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     if (path == W4A16_PATH_AUTO) {
@@ -261,7 +274,7 @@ extern "C" int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_de
 extern "C" int w4a16_lin_forward_host(w4a16_ctx* ctx, const char* name, const uint16_t* x_f16, void* y, size_t t,
                                       int out_f16, int path) {
     W4Lin* L = nullptr;
-    W4_TRY(find_lin(ctx, name, &L));
+    W4_TRY(w4_find_lin(ctx, name, &L));
     if (!x_f16 || !y || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_host %s: null operand or t=0", name);
     const size_t xb = t * L->k * 2, yb = t * L->n * (out_f16 ? 2 : 4);
     uint64_t dx = 0, dy = 0;
@@ -279,7 +292,7 @@ extern "C" int w4a16_lin_forward_host(w4a16_ctx* ctx, const char* name, const ui
 
 extern "C" int w4a16_dequant_dump(w4a16_ctx* ctx, const char* name, int from_tiled, uint64_t out_f32_dev) {
     W4Lin* L = nullptr;
-    W4_TRY(find_lin(ctx, name, &L));
+    W4_TRY(w4_find_lin(ctx, name, &L));
     if (!out_f32_dev) return w4_fail(W4A16_ERR_ARG, "dequant_dump %s: null output", name);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     int ni = (int)L->n, ki = (int)L->k, gi = (int)L->group, rbi = (int)L->row_blocks;
@@ -297,7 +310,7 @@ extern "C" int w4a16_dequant_dump(w4a16_ctx* ctx, const char* name, int from_til
 
 extern "C" int w4a16_lin_untile(w4a16_ctx* ctx, const char* name, uint64_t q_out_dev, uint64_t s_out_dev) {
     W4Lin* L = nullptr;
-    W4_TRY(find_lin(ctx, name, &L));
+    W4_TRY(w4_find_lin(ctx, name, &L));
     if (!q_out_dev || !s_out_dev) return w4_fail(W4A16_ERR_ARG, "lin_untile %s: null output", name);
     if (!L->q_tiled) return w4_fail(W4A16_ERR_NOT_FOUND, "lin %s: no tiled copy", name);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
@@ -324,10 +337,10 @@ extern "C" int w4a16_bench_forward(w4a16_ctx* ctx, const char* const* names, siz
                                    float* ms_events, double* ms_wall) {
     if (!ctx || !names || n_names == 0 || reps == 0) return w4_fail(W4A16_ERR_ARG, "bench_forward: null argument");
     W4Lin* first = nullptr;
-    W4_TRY(find_lin(ctx, names[0], &first));
+    W4_TRY(w4_find_lin(ctx, names[0], &first));
     for (size_t i = 1; i < n_names; i++) {
         W4Lin* L = nullptr;
-        W4_TRY(find_lin(ctx, names[i], &L));
+        W4_TRY(w4_find_lin(ctx, names[i], &L));
         if (L->n != first->n || L->k != first->k || L->group != first->group)
             return w4_fail(W4A16_ERR_SHAPE, "bench_forward: %s and %s differ in shape", names[0], names[i]);
     }

@@ -282,6 +282,47 @@ class W4a16Dec:
                                               warmup, reps, C.byref(ms), C.byref(wall)))
         return ms.value, wall.value
 
+    # ---- layer chain
+    CHAIN_ROLES = ("attn_qkv", "attn_output", "ffn_gate_up", "ffn_down")
+
+    def upload_lin_synth(self, name, n, k, group, seed_q, seed_s, lo=0.002, hi=0.02):
+        """A linear generated on the device from the SplitMix64 streams gen.weights_q(seed_q, n, k) and
+        gen.scales_f16(seed_s, n, k, group, lo, hi)."""
+        ffi.check(self.cc.lib.w4a16_upload_lin_synth(self.cc.h, name.encode(), n, k, group, seed_q, seed_s, lo, hi))
+
+    def upload_chain_synth(self, prefix, n_layers, hidden, n_qkv, n_ff, group=128, seed=None):
+        """Register n_layers synthetic decoder layers "<prefix>.<l>.<role>" with independent weights; returns the
+        (seed_q, seed_s) pairs used, keyed by linear name."""
+        from . import gen
+        seed = gen.GATE_SEED if seed is None else seed
+        shapes = {"attn_qkv": (n_qkv, hidden), "attn_output": (hidden, hidden), "ffn_gate_up": (2 * n_ff, hidden),
+                  "ffn_down": (hidden, n_ff)}
+        seeds = {}
+        for l in range(n_layers):
+            for r, role in enumerate(self.CHAIN_ROLES):
+                n, k = shapes[role]
+                sq, ss = gen.shape_seed(n, k, seed, 100 + 8 * l + 2 * r), gen.shape_seed(n, k, seed, 101 + 8 * l + 2 * r)
+                name = "%s.%d.%s" % (prefix, l, role)
+                self.upload_lin_synth(name, n, k, group, sq, ss)
+                seeds[name] = (sq, ss)
+        return seeds
+
+    def rms_rescale_f16(self, v_dev, ld, ncols, t, out_dev):
+        ffi.check(self.cc.lib.w4a16_rms_rescale_f16(self.cc.h, v_dev, ld, ncols, t, out_dev))
+
+    def silu_mul_f16(self, gu_dev, n_ff, t, out_dev):
+        ffi.check(self.cc.lib.w4a16_silu_mul_f16(self.cc.h, gu_dev, n_ff, t, out_dev))
+
+    def chain_forward(self, prefix, layer0, n_layers, x_dev, t, y_dev):
+        """chain_device_body (w4a16_dec/chains.rs:195-304) reduced to its linears and glue."""
+        ffi.check(self.cc.lib.w4a16_chain_forward(self.cc.h, prefix.encode(), layer0, n_layers, x_dev, t, y_dev))
+
+    def bench_chain(self, prefix, n_layers, x_dev, t, y_dev, reps, warmup=1, use_graph=False):
+        ms, wall = C.c_float(), C.c_double()
+        ffi.check(self.cc.lib.w4a16_bench_chain(self.cc.h, prefix.encode(), n_layers, x_dev, t, y_dev, warmup, reps,
+                                                int(use_graph), C.byref(ms), C.byref(wall)))
+        return ms.value, wall.value
+
 
 def moe_topk(logits, top_k):
     """moe_topk (w4a16_dec/mod.rs:168-185) on the host: logits f32 [t][n_exp] -> (idx int32 [t][top_k], w f32)."""

@@ -25,6 +25,9 @@
  *                           large |g| (silu -> g, -> 0)
  *   orc_moe_topk_sum_f16 .. numpy float32 sequential sum; exactly-summable inputs
  *   orc_moe_align ......... numpy stable argsort by expert + padding arithmetic; tiny hand-worked case
+ *   orc_rms_rescale_f16 ... float64 v / sqrt(mean(v^2) + 1e-6) within one f16 step, >= 99.9 % identical; constant rows;
+ *                           invariance of the output under scaling the row by a power of two
+ *   orc_silu_mul_f16_rows . float64 evaluation within one f16 step; layout (gate | up) by a crafted row
  * No function here is "parity unpinned".
  */
 #include <math.h>
@@ -394,4 +397,35 @@ size_t orc_moe_align(const int32_t* idx, size_t ns, size_t n_exp, size_t block, 
 /* Array form of orc_f32_to_f16 (same routine, element by element). */
 void orc_f32_to_f16_array(const float* v, size_t n, uint16_t* out) {
     for (size_t i = 0; i < n; i++) out[i] = orc_f32_to_f16(v[i]);
+}
+
+/* ---- RMS rescale emitting f16: the normalisation of norm_resid (crates/backend-gpu/src/rawcuda/assets/norm.cu:4-48)
+ * without residual and weight.  out[r][c] = f16(v[r*ld + c] * inv), inv = f32(1 / sqrt(ss / ncols + 1e-6)).
+ * Order of the sum of squares (the contract the device kernel shares): 256 partials, partial i adds the exact f64
+ * squares of columns i, i+256, ... in order; partials folded pairwise at strides 128, 64, ..., 1. ---- */
+void orc_rms_rescale_f16(const float* v, size_t ld, size_t ncols, size_t t, uint16_t* out) {
+    for (size_t r = 0; r < t; r++) {
+        const float* row = v + r * ld;
+        double red[256];
+        for (size_t i = 0; i < 256; i++) {
+            double ss = 0.0;
+            for (size_t c = i; c < ncols; c += 256) {
+                const double d = (double)row[c];
+                ss = ss + d * d;
+            }
+            red[i] = ss;
+        }
+        for (size_t st = 128; st > 0; st >>= 1)
+            for (size_t i = 0; i < st; i++) red[i] = red[i] + red[i + st];
+        const float inv = (float)(1.0 / sqrt(red[0] / (double)ncols + 1e-6));
+        for (size_t c = 0; c < ncols; c++) out[r * ncols + c] = orc_f32_to_f16(row[c] * inv);
+    }
+}
+
+/* ---- ew (assets/ew.cu:9-32) on rows gu f32 [t][2*n_ff] = (gate | up): out[r][c] = f16((g / (1 + exp(-g))) * u) in
+ * f32 arithmetic. ---- */
+void orc_silu_mul_f16_rows(const float* gu, size_t n_ff, size_t t, uint16_t* out) {
+    for (size_t r = 0; r < t; r++)
+        for (size_t c = 0; c < n_ff; c++)
+            out[r * n_ff + c] = orc_silu_mul_f16(gu[r * 2 * n_ff + c], gu[r * 2 * n_ff + n_ff + c]);
 }

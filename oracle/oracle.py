@@ -54,6 +54,8 @@ def lib():
         L.orc_moe_topk.argtypes, L.orc_moe_topk.restype = [f32p, sz, sz, u32p, f32p], None
         L.orc_silu_mul_f16.argtypes, L.orc_silu_mul_f16.restype = [C.c_float, C.c_float], C.c_uint16
         L.orc_f32_to_f16_array.argtypes, L.orc_f32_to_f16_array.restype = [f32p, sz, u16p], None
+        L.orc_rms_rescale_f16.argtypes, L.orc_rms_rescale_f16.restype = [f32p, sz, sz, sz, u16p], None
+        L.orc_silu_mul_f16_rows.argtypes, L.orc_silu_mul_f16_rows.restype = [f32p, sz, sz, u16p], None
         i32p = C.POINTER(C.c_int32)
         L.orc_moe_act_silu_f16.argtypes, L.orc_moe_act_silu_f16.restype = [u16p, sz, sz, u16p], None
         L.orc_moe_topk_sum_f16.argtypes, L.orc_moe_topk_sum_f16.restype = [u16p, sz, sz, sz, f32p], None
@@ -262,3 +264,39 @@ def moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, scale_bf16=False, thre
         c2[slots] = f32_to_f16_array(y2).reshape(len(slots), h)
     y = moe_topk_sum_f16(c2, t, h, top_k)
     return {"c13": c13, "act": act, "c2": c2, "y": y}
+
+
+def rms_rescale_f16(v, ncols):
+    """v f32 [t][ld] -> f16 bits [t][ncols] over the first ncols columns of every row."""
+    v = _c(v, np.float32)
+    t, ld = v.shape
+    out = np.empty((t, ncols), np.uint16)
+    lib().orc_rms_rescale_f16(_p(v, C.c_float), ld, ncols, t, _p(out, C.c_uint16))
+    return out
+
+
+def silu_mul_f16_rows(gu):
+    gu = _c(gu, np.float32)
+    t, two = gu.shape
+    out = np.empty((t, two // 2), np.uint16)
+    lib().orc_silu_mul_f16_rows(_p(gu, C.c_float), two // 2, t, _p(out, C.c_uint16))
+    return out
+
+
+def chain_layer(x, lins, group=128, threads=1):
+    """One decoder layer of linears with its glue (the build's statement of chain_device_body, chains.rs:195-304):
+    lins = [(q, s, n, k)] for attn_qkv, attn_output, ffn_gate_up, ffn_down; x f16 bits [t][hidden].
+    Returns the stage outputs {qkv, a, o, b, gu, c, d, x}."""
+    x = _c(x, np.uint16)
+    t, hidden = x.shape
+    (q0, s0, n0, k0), (q1, s1, n1, k1), (q2, s2, n2, k2), (q3, s3, n3, k3) = lins
+    st = {}
+    st["qkv"] = gemm_lane(x, t, q0, s0, n0, k0, group, False, threads)
+    st["a"] = rms_rescale_f16(st["qkv"], hidden)
+    st["o"] = gemm_lane(st["a"], t, q1, s1, n1, k1, group, False, threads)
+    st["b"] = rms_rescale_f16(st["o"], hidden)
+    st["gu"] = gemm_lane(st["b"], t, q2, s2, n2, k2, group, False, threads)
+    st["c"] = silu_mul_f16_rows(st["gu"])
+    st["d"] = gemm_lane(st["c"], t, q3, s3, n3, k3, group, False, threads)
+    st["x"] = rms_rescale_f16(st["d"], hidden)
+    return st

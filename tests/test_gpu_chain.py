@@ -1,0 +1,188 @@
+"""GPU parity tests of the layer chain (linears of a dense decoder layer run back to back with their glue) through
+the C ABI against the CPU oracle."""
+import numpy as np
+import pytest
+
+from llm170_amd import gen, ops
+from tests import parity
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def dec():
+    d = ops.W4a16Dec()
+    yield d
+    d.cc.close()
+
+
+def _f16(bits):
+    return np.asarray(bits, np.uint16).view(np.float16).astype(np.float32)
+
+
+# ------------------------------------------------------------------ device generator == host generator
+@pytest.mark.parametrize("n,k,group", [(48, 256, 128), (7168, 5120, 128), (100, 768, 32)])
+def test_synth_linear_equals_host_generator(dec, n, k, group):
+    sq, ss = gen.shape_seed(n, k, tensor=7), gen.shape_seed(n, k, tensor=8)
+    dec.upload_lin_synth("syn", n, k, group, sq, ss)
+    q, s = dec.untile("syn")
+    assert np.array_equal(q, gen.weights_q(sq, n, k))
+    assert np.array_equal(s, gen.scales_f16(ss, n, k, group))
+
+
+def test_synth_errors(dec):
+    with pytest.raises(ops.W4a16Error):
+        dec.upload_lin_synth("bad", 16, 256, 128, 1, 2, lo=0.0, hi=0.02)
+    with pytest.raises(ops.W4a16Error):
+        dec.upload_lin_synth("bad", 16, 200, 128, 1, 2)
+
+
+# ------------------------------------------------------------------ glue kernels
+@pytest.mark.parametrize("t,ld,ncols", [(1, 5120, 5120), (4, 7168, 5120), (16, 300, 257), (3, 64, 1)])
+def test_rms_rescale_bit_exact(dec, orc, t, ld, ncols):
+    rng = np.random.default_rng(t * 1000 + ld)
+    v = (rng.standard_normal((t, ld)) * rng.uniform(0.01, 300, (t, 1))).astype(np.float32)
+    cc = dec.cc
+    pv, po = cc.to_device(v), cc.alloc(t * ncols * 2)
+    dec.rms_rescale_f16(pv, ld, ncols, t, po)
+    got = cc.d2h(po, (t, ncols), np.uint16)
+    cc.free(pv)
+    cc.free(po)
+    assert np.array_equal(got, orc.rms_rescale_f16(v, ncols))
+
+
+@pytest.mark.parametrize("t,n_ff", [(1, 17408), (4, 17408), (5, 33)])
+def test_silu_mul_close(dec, orc, t, n_ff):
+    rng = np.random.default_rng(t + n_ff)
+    gu = (rng.standard_normal((t, 2 * n_ff)) * 6).astype(np.float32)
+    cc = dec.cc
+    pg, po = cc.to_device(gu), cc.alloc(t * n_ff * 2)
+    dec.silu_mul_f16(pg, n_ff, t, po)
+    got = cc.d2h(po, (t, n_ff), np.uint16)
+    cc.free(pg)
+    cc.free(po)
+    want = orc.silu_mul_f16_rows(gu)
+    # exp is evaluated by different libraries: results may differ in the last f32 bit before the f16 rounding
+    a, b = _f16(got).astype(np.float64), _f16(want).astype(np.float64)
+    assert np.all(np.abs(a - b) <= parity.f16_ulp(b))
+    assert np.mean(got == want) > 0.995
+
+
+# ------------------------------------------------------------------ the chain
+def _host_lins(seeds, prefix, layer, shapes, group):
+    out = []
+    for role in ops.W4a16Dec.CHAIN_ROLES:
+        n, k = shapes[role]
+        sq, ss = seeds["%s.%d.%s" % (prefix, layer, role)]
+        out.append((gen.weights_q(sq, n, k), gen.scales_f16(ss, n, k, group), n, k))
+    return out
+
+
+def _chain_stagewise(dec, orc, prefix, seeds, shapes, group, layers, t, x, threads):
+    """Run the layers one stage at a time through the C ABI; every GEMM is checked against the lane oracle on the
+    device's own input of that stage, the RMS glue bit for bit, the activation glue to one f16 step."""
+    cc = dec.cc
+    hidden, n_ff = shapes["attn_output"][0], shapes["ffn_down"][1]
+    cur = x
+    for l in range(layers):
+        lins = _host_lins(seeds, prefix, l, shapes, group)
+        names = ["%s.%d.%s" % (prefix, l, r) for r in ops.W4a16Dec.CHAIN_ROLES]
+
+        def gemm(i, xin):
+            got = dec.gemv_host(names[i], xin, t=t)
+            q, s, n, k = lins[i]
+            want = orc.gemm_lane(xin, t, q, s, n, k, group, False, threads)
+            parity.assert_close(got, want, "layer %d %s" % (l, names[i]))
+            return got
+
+        def rms(v, ncols):
+            pv, po = cc.to_device(v), cc.alloc(t * ncols * 2)
+            dec.rms_rescale_f16(pv, v.shape[1], ncols, t, po)
+            got = cc.d2h(po, (t, ncols), np.uint16)
+            cc.free(pv)
+            cc.free(po)
+            assert np.array_equal(got, orc.rms_rescale_f16(v, ncols)), "layer %d rms" % l
+            return got
+
+        a = rms(gemm(0, cur), hidden)
+        b = rms(gemm(1, a), hidden)
+        gu = gemm(2, b)
+        pg, po = cc.to_device(gu), cc.alloc(t * n_ff * 2)
+        dec.silu_mul_f16(pg, n_ff, t, po)
+        c = cc.d2h(po, (t, n_ff), np.uint16)
+        cc.free(pg)
+        cc.free(po)
+        cw = orc.silu_mul_f16_rows(gu)
+        assert np.all(np.abs(_f16(c).astype(np.float64) - _f16(cw)) <= parity.f16_ulp(_f16(cw))), "layer %d act" % l
+        cur = rms(gemm(3, c), hidden)
+    return cur
+
+
+def _chain_oracle(orc, prefix, seeds, shapes, group, layers, x, threads):
+    cur = x
+    for l in range(layers):
+        cur = orc.chain_layer(cur, _host_lins(seeds, prefix, l, shapes, group), group, threads)["x"]
+    return cur
+
+
+@pytest.mark.parametrize("t", [1, 4, 16])
+def test_chain_small_many_layers(dec, orc, t):
+    """24 small layers: stage-wise parity, the one-call chain equals the staged run bit for bit, and the end-to-end
+    result stays close to the oracle's independent run."""
+    say("chain small", t)
+    hidden, n_qkv, n_ff, group, layers = 256, 384, 512, 128, 24
+    shapes = {"attn_qkv": (n_qkv, hidden), "attn_output": (hidden, hidden), "ffn_gate_up": (2 * n_ff, hidden),
+              "ffn_down": (hidden, n_ff)}
+    seeds = dec.upload_chain_synth("small", layers, hidden, n_qkv, n_ff, group)
+    x = gen.normal_f16(31 + t, (t, hidden))
+    staged = _chain_stagewise(dec, orc, "small", seeds, shapes, group, layers, t, x, 4)
+    cc = dec.cc
+    px, py = cc.to_device(x), cc.alloc(t * hidden * 2)
+    dec.chain_forward("small", 0, layers, px, t, py)
+    got = cc.d2h(py, (t, hidden), np.uint16)
+    assert np.array_equal(got, staged)
+    # two half chains compose to the whole
+    dec.chain_forward("small", 0, 10, px, t, py)
+    dec.chain_forward("small", 10, layers - 10, py, t, py)
+    assert np.array_equal(cc.d2h(py, (t, hidden), np.uint16), staged)
+    want = _chain_oracle(orc, "small", seeds, shapes, group, layers, x, 4)
+    m = parity.compare(_f16(got), _f16(want))
+    say("  end to end rel_l2", m["rel_l2"], "identical", float(np.mean(got == want)))
+    assert m["rel_l2"] < 2e-2  # rounding flips of f16 intermediates accumulate over 96 linears
+    ms, _ = dec.bench_chain("small", layers, px, t, py, reps=3, warmup=1, use_graph=True)
+    assert np.array_equal(cc.d2h(py, (t, hidden), np.uint16), staged)  # graph replays give the same bits
+    cc.free(px)
+    cc.free(py)
+
+
+def test_chain_27b_layer_shapes(dec, orc):
+    """Two layers at the 27B-dense shapes (QKV 5120x7168, O 5120x5120, gate+up 5120x34816, down 17408x5120), M = 4."""
+    hidden, n_qkv, n_ff, group, layers, t = 5120, 7168, 17408, 128, 2, 4
+    shapes = {"attn_qkv": (n_qkv, hidden), "attn_output": (hidden, hidden), "ffn_gate_up": (2 * n_ff, hidden),
+              "ffn_down": (hidden, n_ff)}
+    seeds = dec.upload_chain_synth("d27", layers, hidden, n_qkv, n_ff, group)
+    x = gen.normal_f16(4, (t, hidden))
+    say("chain 27b staged")
+    staged = _chain_stagewise(dec, orc, "d27", seeds, shapes, group, layers, t, x, 16)
+    cc = dec.cc
+    px, py = cc.to_device(x), cc.alloc(t * hidden * 2)
+    dec.chain_forward("d27", 0, layers, px, t, py)
+    got = cc.d2h(py, (t, hidden), np.uint16)
+    cc.free(px)
+    cc.free(py)
+    assert np.array_equal(got, staged)
+
+
+def test_chain_errors(dec):
+    with pytest.raises(ops.W4a16Error):
+        dec.chain_forward("nochain", 0, 1, 1, 1, 1)
+    dec.upload_lin_synth("brk.0.attn_qkv", 64, 128, 128, 1, 2)
+    dec.upload_lin_synth("brk.0.attn_output", 128, 128, 128, 1, 2)
+    dec.upload_lin_synth("brk.0.ffn_gate_up", 256, 128, 128, 1, 2)
+    dec.upload_lin_synth("brk.0.ffn_down", 128, 128, 128, 1, 2)
+    with pytest.raises(ops.W4a16Error):  # qkv narrower than hidden
+        dec.chain_forward("brk", 0, 1, 1, 1, 1)
