@@ -34,14 +34,15 @@ def make_copies(dec, gen, n, k, g, copies, prefix):
     names = []
     first = None
     for c in range(copies):
-        q = gen.weights_q(gen.shape_seed(n, k, tensor=1) + 977 * c, n, k)
-        s = gen.scales_f16(gen.shape_seed(n, k, tensor=2) + 977 * c, n, k, g)
+        sq, ss = gen.shape_seed(n, k, tensor=1) + 977 * c, gen.shape_seed(n, k, tensor=2) + 977 * c
         name = "%s.%d" % (prefix, c)
-        dec.upload_lin_g(name, q, s, n, k, g, False)
+        if c == 0:  # the copy the oracle checks is generated on the host; the others, same streams, on the device
+            first = (gen.weights_q(sq, n, k), gen.scales_f16(ss, n, k, g))
+            dec.upload_lin_g(name, first[0], first[1], n, k, g, False)
+        else:
+            dec.upload_lin_synth(name, n, k, g, sq, ss)
         dec.drop_raw(name)
         names.append(name)
-        if c == 0:
-            first = (q, s)
     return names, first
 
 
@@ -61,6 +62,74 @@ def measured_traffic(kernel):
 def time_forward(dec, names, xd, yd, t, steps, warmup, path, out_f16=True):
     ms, wall = dec.bench_forward(names, xd, yd, t, steps, warmup=warmup, out_f16=out_f16, path=path)
     return ms / steps, wall / steps
+
+
+def bench_moe(dec, gen, ops, args):
+    """MoE expert FFN of the 35B-A3B layer shape: 128 experts, top-8, hidden 2048, n_ff 768, group 32; routing from
+    seeded N(0,1) router logits (ragged per-expert row counts).  Bytes = distinct experts hit x (weights + scales of
+    both projections) + activations in and out of every stage."""
+    cc = dec.cc
+    E, h, n_ff, g, k = 128, 2048, 768, 32, 8
+    q13, s13, q2, s2 = gen.make_experts(E, h, n_ff, g)
+    names = []
+    for c in range(3):  # 3 x 340 MB of experts rotated: beyond L2 + last-level cache
+        dec.upload_experts("experts.%d" % c, q13, s13, q2, s2, E, h, n_ff, g, False)
+        names.append("experts.%d" % c)
+    per_expert = (2 * n_ff * h // 2 + 2 * n_ff * (h // g) * 2) + (h * n_ff // 2 + h * (n_ff // g) * 2)
+    out = []
+    for t in (1, 4, 512):
+        x = gen.normal_f16(1 + t, (t, h))
+        lg = cc.to_device(gen.router_logits(t, E))
+        px, pi, pw, py = cc.to_device(x), cc.alloc(t * k * 4), cc.alloc(t * k * 4), cc.alloc(t * h * 4)
+        dec.moe_route(lg, t, E, k, pi, pw)
+        hit = int(np.unique(cc.d2h(pi, (t * k,), np.int32)).size)
+        ns = t * k
+        nbytes = hit * per_expert + t * h * 2 + 2 * ns * n_ff * 2 + 2 * ns * h * 2 + t * h * 4
+        flops = 2.0 * ns * (2 * n_ff * h + h * n_ff)
+        reps = max(10, args.steps // (2 if t <= 4 else 8))
+        ms, _ = dec.bench_moe(names, px, pi, pw, t, k, py, reps, warmup=5)
+        us = ms * 1e3 / reps
+        out.append({"T": t, "experts_hit": hit, "us_per_ffn": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                    "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4), "TFLOPs": round(flops / us / 1e6, 1),
+                    "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4)})
+        for p_ in (lg, px, pi, pw, py):
+            cc.free(p_)
+    return out
+
+
+def bench_chain(dec, gen, ops, args):
+    """64 dense decoder layers of linears at M = 4 (QKV 5120->7168, O 5120->5120, gate+up 5120->34816, down
+    17408->5120, group 128) with the RMS-rescale / SiLU*up glue, independent device-generated weights (10.9 GB)."""
+    cc = dec.cc
+    layers, hidden, n_qkv, n_ff, g, t = 64, 5120, 7168, 17408, 128, 4
+    dec.upload_chain_synth("c4", layers, hidden, n_qkv, n_ff, g)
+    shapes = {"attn_qkv": (n_qkv, hidden), "attn_output": (hidden, hidden), "ffn_gate_up": (2 * n_ff, hidden),
+              "ffn_down": (hidden, n_ff)}
+    for l in range(layers):
+        for role in ops.W4a16Dec.CHAIN_ROLES:
+            dec.drop_raw("c4.%d.%s" % (l, role))
+    px, py = cc.to_device(gen.normal_f16(404, (t, hidden))), cc.alloc(t * hidden * 2)
+    reps = max(3, args.steps // 80)
+    ms_eager, _ = dec.bench_chain("c4", layers, px, t, py, reps, warmup=1, use_graph=False)
+    ms_graph, _ = dec.bench_chain("c4", layers, px, t, py, reps, warmup=1, use_graph=True)
+    total = sum(algorithmic_bytes(t, kk, nn, g) for (nn, kk) in shapes.values()) * layers
+    best = min(ms_eager, ms_graph) / reps
+    per_gemm = []
+    xw, yw = cc.alloc(t * n_ff * 2), cc.alloc(t * 2 * n_ff * 4)
+    cc.memset0(xw, t * n_ff * 2)
+    for role in ops.W4a16Dec.CHAIN_ROLES:
+        nn, kk = shapes[role]
+        names = ["c4.%d.%s" % (l, role) for l in range(layers)]
+        ms, _ = dec.bench_forward(names, xw, yw, t, 256, warmup=64, out_f16=False)
+        b = algorithmic_bytes(t, kk, nn, g) + 2 * t * nn  # f32 output
+        per_gemm.append({"linear": role, "K": kk, "N": nn, "us": round(ms / 256 * 1e3, 2),
+                         "GBps": round(b / (ms / 256 * 1e-3) / 1e9, 1)})
+    for p_ in (px, py, xw, yw):
+        cc.free(p_)
+    return {"layers": layers, "M": t, "ms_per_pass_eager": round(ms_eager / reps, 4),
+            "ms_per_pass_graph": round(ms_graph / reps, 4), "us_per_token": round(best * 1e3 / t, 2),
+            "GBps_end_to_end": round(total / (best * 1e-3) / 1e9, 1),
+            "hbm_frac_end_to_end": round(total / (best * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "per_gemm": per_gemm}
 
 
 def main():
@@ -180,6 +249,10 @@ def main():
                 ptable.append({"shape": shape, "M": mm, "ms": round(ms_m, 4), "TFLOPs": round(tf, 1),
                                "mfma_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4)})
         extra["prefill_table"] = ptable
+        for p_ in (xp2, yp2, xp1, x2d):
+            cc.free(p_)
+        extra["moe_table"] = bench_moe(dec, gen, ops, args)
+        extra["chain"] = bench_chain(dec, gen, ops, args)
 
     line = {
         "metric": "W4A16 GEMM: decode GB/s (M=1) & prefill TFLOP/s (M=4096) vs MI355X peak",

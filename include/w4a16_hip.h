@@ -233,7 +233,7 @@ int w4a16_upload_lin_synth(w4a16_ctx* ctx, const char* name, size_t n, size_t k,
 
 /* RMS rescale of t rows to unit mean square, emitting f16 (the part of norm_resid, assets/norm.cu:4-48, that a chain
  * of linears needs: no residual, no weight): out[r][c] = f16(v[r*ld + c] * inv_r), inv_r = f32(1/sqrt(ms_r + 1e-6)),
- * c < ncols <= ld.  The sum of squares is taken in f64 in a fixed order (256 strided partials, pairwise fold), so a
+ * c < ncols <= ld.  The sum of squares is taken in f64 in a fixed order (1024 strided partials, pairwise fold), so a
  * CPU restatement is bit-identical. */
 int w4a16_rms_rescale_f16(w4a16_ctx* ctx, uint64_t v_f32_dev, size_t ld, size_t ncols, size_t t, uint64_t out_f16_dev);
 /* ew (assets/ew.cu:9-32): out[r][c] = f16(silu(gu[r][c]) * gu[r][n_ff + c]) for gu f32 [t][2*n_ff], f32 arithmetic. */

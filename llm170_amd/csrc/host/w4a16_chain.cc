@@ -56,7 +56,7 @@ extern "C" int w4a16_rms_rescale_f16(w4a16_ctx* ctx, uint64_t v_f32_dev, size_t 
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     int ldi = (int)ld, nc = (int)ncols;
     void* p[] = {&v_f32_dev, &ldi, &nc, &out_f16_dev};
-    return w4_launch(ctx, "w4a16_rms_rescale_f16", (unsigned)t, 1, 256, 0, p);
+    return w4_launch(ctx, "w4a16_rms_rescale_f16", (unsigned)t, 1, 1024, 0, p);
 }
 
 extern "C" int w4a16_silu_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_ff, size_t t, uint64_t out_f16_dev) {
@@ -66,7 +66,7 @@ extern "C" int w4a16_silu_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     int nf = (int)n_ff, ti = (int)t;
     void* p[] = {&gu_f32_dev, &nf, &ti, &out_f16_dev};
-    return w4_launch(ctx, "w4a16_silu_mul_f16", std::min<unsigned>(ceil_div(t * n_ff, 256), 4096), 1, 256, 0, p);
+    return w4_launch(ctx, "w4a16_silu_mul_f16", std::min<unsigned>(ceil_div(t * n_ff / (n_ff % 4 == 0 ? 4 : 1), 256), 4096), 1, 256, 0, p);
 }
 
 extern "C" int w4a16_chain_forward(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers, uint64_t x_dev,

@@ -11,33 +11,64 @@ __device__ __forceinline__ _Float16 glue_round_f16(float v) {
 }
 
 // out[r][c] = f16(v[r][c] * inv),  inv = f32(1 / sqrt(mean_c(v[r][c]^2) + 1e-6)).
-// The sum of squares has a fixed order so that a CPU restatement is bit-identical: thread i adds the (exact) f64
-// squares of columns i, i+256, ... in order; the 256 partials are folded pairwise at strides 128, 64, ..., 1.
-// One workgroup of 256 threads per row; v rows are ld floats apart (a column slice of a wider matrix is allowed).
-extern "C" __global__ __launch_bounds__(256) void w4a16_rms_rescale_f16(const float* __restrict__ v, int ld, int ncols,
-                                                                       uint16_t* __restrict__ out) {
-    __shared__ double red[256];
+// The sum of squares has a fixed order so that a CPU restatement is bit-identical: partial i (i < 1024) adds the
+// (exact) f64 squares of columns i, i+1024, ... in order; the 1024 partials are folded pairwise at strides 512, 256,
+// ..., 1.  One workgroup of 1024 threads per row; every thread has its few loads in flight at once.  v rows are ld
+// floats apart (a column slice of a wider matrix is allowed).
+#define RMS_LANES 1024
+#define RMS_UNROLL 8
+extern "C" __global__ __launch_bounds__(RMS_LANES) void w4a16_rms_rescale_f16(const float* __restrict__ v, int ld,
+                                                                             int ncols, uint16_t* __restrict__ out) {
+    __shared__ double red[RMS_LANES];
     const int tid = threadIdx.x;
     const float* row = v + (size_t)blockIdx.x * ld;
     double ss = 0.0;
-    for (int c = tid; c < ncols; c += 256) {
-        const double d = (double)row[c];
-        ss = ss + d * d;
+    for (int c0 = tid; c0 < ncols; c0 += RMS_LANES * RMS_UNROLL) {
+        float x[RMS_UNROLL];
+#pragma unroll
+        for (int j = 0; j < RMS_UNROLL; j++) {
+            const int c = c0 + j * RMS_LANES;
+            x[j] = c < ncols ? row[c] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < RMS_UNROLL; j++) {
+            const double d = (double)x[j];
+            ss = ss + d * d;  // a zero past the row end adds +0.0 and changes nothing
+        }
     }
     red[tid] = ss;
     __syncthreads();
-    for (int st = 128; st > 0; st >>= 1) {
+    for (int st = RMS_LANES / 2; st >= 64; st >>= 1) {
         if (tid < st) red[tid] = red[tid] + red[tid + st];
         __syncthreads();
     }
-    const float inv = (float)(1.0 / sqrt(red[0] / (double)ncols + 1e-6));
+    // the last 64 partials are folded inside wave 0 with the same pairing (strides 32, 16, ..., 1)
+    double r = red[tid & 63];
+#pragma unroll
+    for (int st = 32; st > 0; st >>= 1) r = r + __shfl_down(r, st);
+    r = __shfl(r, 0);
+    const float inv = (float)(1.0 / sqrt(r / (double)ncols + 1e-6));
     _Float16* o = reinterpret_cast<_Float16*>(out) + (size_t)blockIdx.x * ncols;
-    for (int c = tid; c < ncols; c += 256) o[c] = glue_round_f16(row[c] * inv);
+    for (int c = tid; c < ncols; c += RMS_LANES) o[c] = glue_round_f16(row[c] * inv);
 }
 
 // out[r][c] = f16((g / (1 + exp(-g))) * u),  g = gu[r][c], u = gu[r][n_ff + c], all in f32 (assets/ew.cu:19-30).
+// Four columns per thread when n_ff % 4 == 0.
 extern "C" __global__ __launch_bounds__(256) void w4a16_silu_mul_f16(const float* __restrict__ gu, int n_ff, int t,
                                                                     uint16_t* __restrict__ out) {
+    if ((n_ff & 3) == 0) {
+        const size_t total = (size_t)t * n_ff / 4;
+        for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+            const size_t r = (i * 4) / n_ff, c = (i * 4) % n_ff;
+            const f4_t g = *reinterpret_cast<const f4_t*>(gu + r * 2 * n_ff + c);
+            const f4_t u = *reinterpret_cast<const f4_t*>(gu + r * 2 * n_ff + n_ff + c);
+            h4_t o;
+#pragma unroll
+            for (int j = 0; j < 4; j++) o[j] = glue_round_f16((g[j] / (1.0f + expf(-g[j]))) * u[j]);
+            *reinterpret_cast<h4_t*>(reinterpret_cast<_Float16*>(out) + i * 4) = o;
+        }
+        return;
+    }
     const size_t total = (size_t)t * n_ff;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t r = i / n_ff, c = i % n_ff;

@@ -401,21 +401,21 @@ void orc_f32_to_f16_array(const float* v, size_t n, uint16_t* out) {
 
 /* ---- RMS rescale emitting f16: the normalisation of norm_resid (crates/backend-gpu/src/rawcuda/assets/norm.cu:4-48)
  * without residual and weight.  out[r][c] = f16(v[r*ld + c] * inv), inv = f32(1 / sqrt(ss / ncols + 1e-6)).
- * Order of the sum of squares (the contract the device kernel shares): 256 partials, partial i adds the exact f64
- * squares of columns i, i+256, ... in order; partials folded pairwise at strides 128, 64, ..., 1. ---- */
+ * Order of the sum of squares (the contract the device kernel shares): 1024 partials, partial i adds the exact f64
+ * squares of columns i, i+1024, ... in order; partials folded pairwise at strides 512, 256, ..., 1. ---- */
 void orc_rms_rescale_f16(const float* v, size_t ld, size_t ncols, size_t t, uint16_t* out) {
     for (size_t r = 0; r < t; r++) {
         const float* row = v + r * ld;
-        double red[256];
-        for (size_t i = 0; i < 256; i++) {
+        double red[1024];
+        for (size_t i = 0; i < 1024; i++) {
             double ss = 0.0;
-            for (size_t c = i; c < ncols; c += 256) {
+            for (size_t c = i; c < ncols; c += 1024) {
                 const double d = (double)row[c];
                 ss = ss + d * d;
             }
             red[i] = ss;
         }
-        for (size_t st = 128; st > 0; st >>= 1)
+        for (size_t st = 512; st > 0; st >>= 1)
             for (size_t i = 0; i < st; i++) red[i] = red[i] + red[i + st];
         const float inv = (float)(1.0 / sqrt(red[0] / (double)ncols + 1e-6));
         for (size_t c = 0; c < ncols; c++) out[r * ncols + c] = orc_f32_to_f16(row[c] * inv);
