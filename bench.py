@@ -206,8 +206,8 @@ def main():
     xp = gen.normal_f16(gen.shape_seed(n, k, tensor=4), (mp, k))
     xpd = cc.to_device(xp)
     ypd = cc.alloc(mp * n * 2)
-    psteps = max(5, args.steps // 20)
-    pf_ms, _ = time_forward(dec, names, xpd, ypd, mp, psteps, 3, ops.PATH_PREFILL)
+    psteps = max(10, args.steps // 8)
+    pf_ms, _ = time_forward(dec, names, xpd, ypd, mp, psteps, 10, ops.PATH_PREFILL)
     pf_flops = 2.0 * mp * n * k
     pf_tf = pf_flops / (pf_ms * 1e-3) / 1e12
     # parity of the prefill result: a seeded sample of outputs against the CPU oracle
@@ -244,7 +244,7 @@ def main():
         for (nm, kk, nn, xdev, shape) in ((names, k, n, xp1, "gate_up K5120 N34816 g128"),
                                           (names2, k2, n2, xp2, "down K17408 N5120 g128")):
             for mm in (512, 1024, 4096):
-                ms_m, _ = time_forward(dec, nm, xdev, yp2, mm, psteps, 3, ops.PATH_PREFILL)
+                ms_m, _ = time_forward(dec, nm, xdev, yp2, mm, psteps, 5, ops.PATH_PREFILL)
                 tf = 2.0 * mm * nn * kk / (ms_m * 1e-3) / 1e12
                 ptable.append({"shape": shape, "M": mm, "ms": round(ms_m, 4), "TFLOPs": round(tf, 1),
                                "mfma_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4)})

@@ -559,36 +559,57 @@ extern "C" __global__ __launch_bounds__(512) void w4a16_moe_align(const int* __r
         all += wsum[w];
         allhit += whit[w];
     }
-    if (tid == 0) {
-        num_post[0] = (int)all;
-        num_post[1] = (int)allhit;
-    }
-    unsigned pos = base + incl - local;
+    // global stores come last: a workgroup barrier waits for every outstanding store, so none may be pending at one
+    const unsigned pos0 = base + incl - local;
+    {
+        unsigned pos = pos0;
 #pragma unroll
-    for (int h = 0; h < 2; h++) {
-        const int e = 2 * tid + h;
-        if (e < n_exp) {
-            poff[e] = pos;
-            const unsigned c = tot[e];
-            for (unsigned p = c; p < padded[h]; p++) sorted_ids[pos + p] = ns;
-            for (unsigned b = 0; b < padded[h] / block; b++) expert_ids[pos / block + b] = e;
+        for (int h = 0; h < 2; h++) {
+            const int e = 2 * tid + h;
+            if (e < n_exp) poff[e] = pos;
             pos += padded[h];
         }
     }
     __syncthreads();
-    // placement in slot order: every wave walks its range 64 slots at a time; rank among equal experts in the step
+    // placement in slot order: every wave walks its range 64 slots at a time; rank among equal experts in the step.
+    // cnt[wave][*] is private to the wave and LDS operations of one wave execute in order, so the loop needs no
+    // workgroup barrier; the wave-scope fences keep the compiler from reordering the LDS accesses.
     for (int s = 0; s < steps; s++) {
         const int e = expert_of(s);
         unsigned rank = 0, same = 0;
+#pragma unroll
         for (int i = 0; i < 64; i++) {
-            const int ei = __shfl(e, i);
+            const int ei = __builtin_amdgcn_readlane(e, i);  // lane i's expert in a scalar register
             same += ei == e;
             rank += (ei == e) && (i < lane);
         }
-        if (e >= 0) sorted_ids[poff[e] + cnt[wave][e] + rank] = j0 + s * 64 + lane;
-        __syncthreads();
-        if (e >= 0 && rank + 1 == same) cnt[wave][e] += same;
-        __syncthreads();
+        unsigned before = 0;
+        if (e >= 0) before = cnt[wave][e];
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (e >= 0) {
+            sorted_ids[poff[e] + before + rank] = j0 + s * 64 + lane;
+            if (rank + 1 == same) cnt[wave][e] = before + same;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (tid == 0) {
+        num_post[0] = (int)all;
+        num_post[1] = (int)allhit;
+    }
+    {
+        unsigned pos = pos0;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int e = 2 * tid + h;
+            if (e < n_exp) {
+                const unsigned c = tot[e];
+                for (unsigned p = c; p < padded[h]; p++) sorted_ids[pos + p] = ns;
+                for (unsigned b = 0; b < padded[h] / block; b++) expert_ids[pos / block + b] = e;
+            }
+            pos += padded[h];
+        }
     }
 }
 
