@@ -39,16 +39,17 @@ static int launch_lane(w4a16_ctx* ctx, uint64_t q, uint64_t s, uint64_t x, uint6
     return w4_launch(ctx, sym, ceil_div(n, 4), ceil_div(t, 8), 256, 0, params);
 }
 
-// Launch shape of the row-block decode kernel.  Measured on MI355X at the 27B layer shapes: two row blocks per
-// wave and four waves per block (in-block split-K by 4) is best or within 2 % of best for t <= 8 and for narrow
-// outputs; for 9..16 token rows on wide outputs four row blocks per wave halve the x operand traffic.
+// Launch shape of the row-block decode kernel.  Measured on MI355X at the 27B layer shapes (gate+up 5120x34816, down
+// 17408x5120, QKV 5120x7168, O 5120x5120): two row blocks per wave with eight waves per block (in-block split-K by 8)
+// is best or within 1 % of best for t <= 8 on every shape; for 9..16 token rows on wide outputs four row blocks per
+// wave halve the x operand traffic.
 static int pick_decode_shape(const w4a16_ctx* ctx, const W4Lin& L, size_t t, int* rb_out, int* waves_out) {
     const bool wide16 = t > 8 && L.row_blocks >= 1024;
     int rb = ctx->decode_rows_per_wave ? ctx->decode_rows_per_wave / 16 : (wide16 ? 4 : 2);
     if (rb != 1 && rb != 2 && rb != 4) return w4_fail(W4A16_ERR_ARG, "decode: rows_per_wave must be 16, 32 or 64");
     while (rb > 1 && L.row_blocks < (size_t)rb) rb >>= 1;
     const int kt_n = (int)(L.k / 128);
-    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : (wide16 ? 2 : 4);
+    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : (wide16 ? 2 : t > 8 ? 4 : 8);
     waves = std::max(1, std::min(std::min(waves, 8), kt_n));
     *rb_out = rb;
     *waves_out = waves;
@@ -69,7 +70,10 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of};
-    unsigned shmem = waves > 1 ? (unsigned)(waves * rb * 64 * 16) : 0;
+    // LDS: the split-K partial tiles [waves][rb][1 KiB], then two scale slots per wave; a slot holds the scales of
+    // one ring round (rb x depth x groups-per-tile x 32 bytes, ring never deeper than 8 tiles) rounded up to 512
+    const unsigned slot = ((unsigned)(rb * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
+    const unsigned shmem = (unsigned)(waves * rb * 1024) + (unsigned)waves * 2u * slot;
     return w4_launch(ctx, sym, ceil_div(L.row_blocks, (size_t)rb), 1, (unsigned)(waves * 64), shmem, params);
 }
 

@@ -14,16 +14,20 @@
 //   * weights enter the MFMA as exact integers; the per-group scale multiplies the f32 group sum, so no weight is
 //     ever rounded to f16 (error vs the f32 lane contract is summation order only);
 //   * each wave keeps DEPTH k-tiles of loads in flight (register ring, software pipelined);
+//   * scales: a per-row-block scale load per k tile is a vector-memory instruction that moves 32 distinct bytes; with
+//     the x load they cost more address-unit time than the weight stream itself (measured: without them the same
+//     load structure runs 13 % faster).  So ONE 8-byte-per-lane load per ring round fetches the scales of all RB row
+//     blocks x DEPTH k tiles of the next round into a wave-private LDS slot (double buffered, no barrier: LDS
+//     operations of one wave execute in order) and each MFMA group reads its four scales back with ds_read_b64;
 //   * split-K lives inside the workgroup: the W waves of a block take consecutive k-tile slices of the same RB row
 //     blocks and wave 0 folds the partial tiles through LDS in fixed order (deterministic, no atomics, no second
 //     launch).  The host picks RB and W.
 #include "w4a16_common.hpp"
 
 // One pipeline stage = the loads of one k tile: RB weight tiles, their scales, and XL loads of x.
-template <int G, int RB, int XL>
+template <int RB, int XL>
 struct DecodeStage {
     u4_t q[RB];
-    u2_t s[RB][W4_TILE_K / G];
     u4_t x[XL];
 };
 
@@ -41,8 +45,11 @@ template <int G, bool SBF, int RB, int DEPTH, int XL>
 __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                             const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
                                             int k, int n, int t, int out_f16) {
-    extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K
+    extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K, then [W][2][AUXB] scale slots
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
+    constexpr int AUXB = RB * DEPTH * GPT * 32;      // bytes of scales one ring round needs: [rb][tile][group][16 rows]
+    constexpr int AUXN = (AUXB + 511) / 512;         // 8-byte-per-lane loads that fetch them
+    constexpr int SLOT = AUXN * 512;                 // LDS bytes of one slot: every lane of every load has a place
     constexpr int C = 4 / XL;           // 32-k chunks (MFMAs) served by one x load
     constexpr int TPL = 16 / C;         // token columns served by one x load
     const int lane = threadIdx.x & 63, W = blockDim.x >> 6;
@@ -55,42 +62,61 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     const int m = lane & 15, g = lane >> 4;
 
     // Every load is a raw buffer load: an out-of-range offset returns zeros and costs no memory traffic, which
-    // predicates tiles past kt1 and token columns >= t without a branch.
-    const __amdgpu_buffer_rsrc_t qr = w4_make_rsrc(qt, (unsigned)row_blocks * (unsigned)kt_n * 1024u);
-    const __amdgpu_buffer_rsrc_t sr = w4_make_rsrc(st, (unsigned)row_blocks * (unsigned)kg_n * 32u);
-    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)t * (unsigned)k * 2u);
+    // predicates token columns >= t without a branch.
     // x load l of a tile: lane (m, g) fetches, for token m % TPL, the 8 halves of chunk l*C + m / TPL at k offset g*8
     const int xtok = m % TPL, xchunk = m / TPL;
     const unsigned xoff = xtok < t ? ((unsigned)xtok * (unsigned)k + (unsigned)(xchunk * 32 + g * 8)) * 2u : W4_OOB;
+    const unsigned q_bytes = (unsigned)row_blocks * (unsigned)kt_n * 1024u, s_bytes = (unsigned)row_blocks * (unsigned)kg_n * 32u,
+                   x_bytes = (unsigned)t * (unsigned)k * 2u;
     f4_t acc[RB];
-    unsigned qoff[RB], soff[RB];
+    unsigned qoff[RB];
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
         acc[rb] = (f4_t){0.f, 0.f, 0.f, 0.f};
         const unsigned nb = (unsigned)min(nb0 + rb, row_blocks - 1);  // a tail block re-reads the last row block
         qoff[rb] = nb * (unsigned)kt_n * 1024u + (unsigned)lane * 16u;
-        soff[rb] = nb * (unsigned)kg_n * 32u + (unsigned)g * 8u;
     }
+    // scale fetch: byte o = lane*8 + a*512 of the round's slot belongs to row block o / (DEPTH*GPT*32); the rest of o
+    // is the offset inside that row block's run of DEPTH tiles, contiguous in the tiled scale array as well
+    char* const aux_lds = reinterpret_cast<char*>(red) + W * RB * 1024 + wave * (2 * SLOT);
+    unsigned aoff[AUXN];
+#pragma unroll
+    for (int a = 0; a < AUXN; a++) {
+        const int o = lane * 8 + a * 512;
+        const int rb = o / (DEPTH * GPT * 32), rem = o % (DEPTH * GPT * 32);
+        const unsigned nb = (unsigned)min(nb0 + rb, row_blocks - 1);
+        aoff[a] = o < AUXB ? nb * (unsigned)kg_n * 32u + (unsigned)rem : W4_OOB;
+    }
+    u2_t aux[AUXN];
+    auto load_aux = [&](int kt) {  // scales of tiles kt .. kt+DEPTH-1 (a run past the wave's slice is never used)
+        const __amdgpu_buffer_rsrc_t sr_ = w4_make_rsrc(st, kt < kt1 ? s_bytes : 0u);
+#pragma unroll
+        for (int a = 0; a < AUXN; a++) aux[a] = __builtin_amdgcn_raw_buffer_load_b64(sr_, aoff[a], kt * (GPT * 32), 0);
+    };
+    auto store_aux = [&](int buf) {  // all lanes store (lanes past AUXB hold zeros): no divergence, nothing for the
+                                     // compiler to sink the loads into
+#pragma unroll
+        for (int a = 0; a < AUXN; a++) *reinterpret_cast<u2_t*>(aux_lds + buf * SLOT + lane * 8 + a * 512) = aux[a];
+    };
 
-    DecodeStage<G, RB, XL> stage[DEPTH];
-    auto load = [&](DecodeStage<G, RB, XL>& s_, int kt) {
+    // Per-tile addressing costs no vector ALU work: the lane part of every offset is loop invariant, the k-tile part
+    // travels in the scalar offset operand, and a tile past the wave's range is switched off by a zero-length
+    // descriptor (the wave-uniform select is scalar work).
+    DecodeStage<RB, XL> stage[DEPTH];
+    auto load = [&](DecodeStage<RB, XL>& s_, int kt) {
         const bool live = kt < kt1;
+        const __amdgpu_buffer_rsrc_t qr_ = w4_make_rsrc(qt, live ? q_bytes : 0u);
+        const __amdgpu_buffer_rsrc_t xr_ = w4_make_rsrc(x, live ? x_bytes : 0u);
 #pragma unroll
         for (int rb = 0; rb < RB; rb++)
-            s_.q[rb] = __builtin_amdgcn_raw_buffer_load_b128(qr, live ? qoff[rb] + (unsigned)kt * 1024u : W4_OOB, 0,
-                                                             2 /* nt: read-once stream */);
-#pragma unroll
-        for (int rb = 0; rb < RB; rb++)
-#pragma unroll
-            for (int gi = 0; gi < GPT; gi++)
-                s_.s[rb][gi] = __builtin_amdgcn_raw_buffer_load_b64(
-                    sr, live ? soff[rb] + (unsigned)(kt * GPT + gi) * 32u : W4_OOB, 0, 0);
+            s_.q[rb] = __builtin_amdgcn_raw_buffer_load_b128(qr_, qoff[rb], kt * 1024, 2 /* nt: read-once stream */);
 #pragma unroll
         for (int l = 0; l < XL; l++)
-            s_.x[l] = __builtin_amdgcn_raw_buffer_load_b128(
-                xr, live ? xoff + (unsigned)(kt * W4_TILE_K + l * C * 32) * 2u : W4_OOB, 0, 0);
+            s_.x[l] = __builtin_amdgcn_raw_buffer_load_b128(xr_, xoff + (unsigned)(l * C * 32) * 2u, kt * (W4_TILE_K * 2), 0);
     };
-    auto compute = [&](const DecodeStage<G, RB, XL>& s_) {
+    // sc = this lane's view of the round's scale slot: rows 4g..4g+3 of (row block rb, tile d, group gi) are the 8
+    // bytes at sc + ((rb*DEPTH + d)*GPT + gi)*32
+    auto compute = [&](const DecodeStage<RB, XL>& s_, const char* sc, int d) {
         // B operand of MFMA w = chunk w of x for token column m: held by lane (m + (w % C) * TPL) of load w / C
         u4_t xb[4];
 #pragma unroll
@@ -110,19 +136,20 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                 for (int w = 0; w < 4; w++)
                     part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
                                                                   __builtin_bit_cast(h8_t, xb[w]), part, 0, 0, 0);
+                const u2_t sv = *reinterpret_cast<const u2_t*>(sc + (rb * DEPTH + d) * GPT * 32);
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    acc[rb][i] += w4_scale_fast<SBF>((s_.s[rb][0][i >> 1] >> (16 * (i & 1))) & 0xFFFFu) * part[i];
+                    acc[rb][i] += w4_scale_fast<SBF>((sv[i >> 1] >> (16 * (i & 1))) & 0xFFFFu) * part[i];
             } else {
 #pragma unroll
                 for (int w = 0; w < 4; w++) {
                     f4_t part = {0.f, 0.f, 0.f, 0.f};
                     part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
                                                                   __builtin_bit_cast(h8_t, xb[w]), part, 0, 0, 0);
+                    const u2_t sv = *reinterpret_cast<const u2_t*>(sc + ((rb * DEPTH + d) * GPT + w % GPT) * 32);
 #pragma unroll
                     for (int i = 0; i < 4; i++)
-                        acc[rb][i] +=
-                            w4_scale_fast<SBF>((s_.s[rb][w % GPT][i >> 1] >> (16 * (i & 1))) & 0xFFFFu) * part[i];
+                        acc[rb][i] += w4_scale_fast<SBF>((sv[i >> 1] >> (16 * (i & 1))) & 0xFFFFu) * part[i];
                 }
             }
         }
@@ -134,18 +161,30 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     // is finished by the unrolled tail.  The scheduling barriers keep each stage's loads together.
     const int tiles = kt1 - kt0;
     const int rounds = tiles / DEPTH;
+    const char* const sc0 = aux_lds + g * 8;
     for (int r = -1; r < rounds; r++) {
+        // scales of round r+1 travel with this round's ring loads and are parked in LDS slot (r+1)&1 once this
+        // round's computes (which read slot r&1) are issued; they are older than every ring load issued below, so
+        // waiting for them leaves the whole ring in flight
+        load_aux(kt0 + (r + 1) * DEPTH);
+        __builtin_amdgcn_sched_barrier(0);
+        const char* sc = sc0 + (r & 1) * SLOT;
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
-            if (r >= 0) compute(stage[d]);
+            if (r >= 0) compute(stage[d], sc, d);
             __builtin_amdgcn_sched_barrier(0);
             load(stage[d], kt0 + (r + 1) * DEPTH + d);
             __builtin_amdgcn_sched_barrier(0);
         }
+        store_aux((r + 1) & 1);
+        __builtin_amdgcn_sched_barrier(0);
     }
+    {
+        const char* sc = sc0 + (rounds & 1) * SLOT;
 #pragma unroll
-    for (int d = 0; d < DEPTH - 1; d++)
-        if (rounds * DEPTH + d < tiles) compute(stage[d]);
+        for (int d = 0; d < DEPTH - 1; d++)
+            if (rounds * DEPTH + d < tiles) compute(stage[d], sc, d);
+    }
 
     if (W > 1) {
         if (wave != 0) {
@@ -187,28 +226,48 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     }
 }
 
-// ring depth: as many stages as ~96 VGPRs of load buffers allow
-#define DECODE_DEPTH(G, RB, XL) \
-    ((96 / (4 * RB + 2 * RB * (W4_TILE_K / G) + 4 * XL)) < 2 ? 2 : (96 / (4 * RB + 2 * RB * (W4_TILE_K / G) + 4 * XL)) > 8 ? 8 : (96 / (4 * RB + 2 * RB * (W4_TILE_K / G) + 4 * XL)))
+// Two register regimes, chosen per instantiation.  Measured on MI355X: what the streaming rate needs is many resident
+// waves with a short ring each, not a deep ring in few waves — with <= 80 VGPRs six waves per SIMD are resident, the
+// whole grid of the 27B layer shapes is on the chip at once, every wave gets its share of HBM and all finish together
+// (a deep-ring build at three waves per SIMD ran the grid in two uneven generations: 4.6 -> 5.0 TB/s at M = 1).
+//   HI: ring sized for 24 VGPRs of load buffers, amdgpu_waves_per_eu(6,6)   — variants that fit 80 VGPRs unspilled
+//   MID: the same ring at five waves per SIMD (<= 102 VGPRs)
+//   LO: ring sized for 64 VGPRs, occupancy left to the compiler             — the wide variants (4 row blocks, 4 x
+//       loads) and group size 32
+#define DECODE_STAGE_REGS(G, RB, XL) (4 * RB + 4 * XL)
+#define DECODE_DEPTH(BUDGET, G, RB, XL) \
+    ((BUDGET / DECODE_STAGE_REGS(G, RB, XL)) < 2 ? 2 : (BUDGET / DECODE_STAGE_REGS(G, RB, XL)) > 8 ? 8 : (BUDGET / DECODE_STAGE_REGS(G, RB, XL)))
 
-#define DECODE_KERNEL_X(NAME, G, SBF, RB, XL)                                                                        \
-    extern "C" __global__ __launch_bounds__(512) void NAME##_x##XL(const u4_t* qt, const uint16_t* st,               \
-                                                                   const uint16_t* x, void* y, int row_blocks,       \
-                                                                   int k, int n, int t, int out_f16) {               \
-        decode_body<G, SBF, RB, DECODE_DEPTH(G, RB, XL), XL>(qt, st, x, y, row_blocks, k, n, t, out_f16);            \
+#define DECODE_KERNEL_X(NAME, G, SBF, RB, XL, BUDGET, ATTR)                                                          \
+    extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
+                                                                        const uint16_t* x, void* y, int row_blocks,  \
+                                                                        int k, int n, int t, int out_f16) {          \
+        decode_body<G, SBF, RB, DECODE_DEPTH(BUDGET, G, RB, XL), XL>(qt, st, x, y, row_blocks, k, n, t, out_f16);    \
     }
-#define DECODE_KERNEL(NAME, G, SBF, RB) \
-    DECODE_KERNEL_X(NAME, G, SBF, RB, 1) DECODE_KERNEL_X(NAME, G, SBF, RB, 2) DECODE_KERNEL_X(NAME, G, SBF, RB, 4)
+#define DECODE_HI __attribute__((amdgpu_waves_per_eu(6, 6)))
+#define DECODE_MID __attribute__((amdgpu_waves_per_eu(5, 5)))
+#define DECODE_LO
+// rb1 at group 128: all three x widths fit the HI regime
+#define DECODE_KERNEL_RB1(NAME, G, SBF)                                                       \
+    DECODE_KERNEL_X(NAME, G, SBF, 1, 1, 24, DECODE_HI) DECODE_KERNEL_X(NAME, G, SBF, 1, 2, 24, DECODE_HI) \
+    DECODE_KERNEL_X(NAME, G, SBF, 1, 4, 24, DECODE_HI)
+// rb2 at group 128: x1 fits HI, x2 MID
+#define DECODE_KERNEL_RB2_G128(NAME, SBF)                                                         \
+    DECODE_KERNEL_X(NAME, 128, SBF, 2, 1, 24, DECODE_HI) DECODE_KERNEL_X(NAME, 128, SBF, 2, 2, 24, DECODE_MID) \
+    DECODE_KERNEL_X(NAME, 128, SBF, 2, 4, 64, DECODE_LO)
+#define DECODE_KERNEL_LO3(NAME, G, SBF, RB)                                                   \
+    DECODE_KERNEL_X(NAME, G, SBF, RB, 1, 64, DECODE_LO) DECODE_KERNEL_X(NAME, G, SBF, RB, 2, 64, DECODE_LO) \
+    DECODE_KERNEL_X(NAME, G, SBF, RB, 4, 64, DECODE_LO)
 
-DECODE_KERNEL(w4a16_decode_g128_f16_rb1, 128, false, 1)
-DECODE_KERNEL(w4a16_decode_g128_f16_rb2, 128, false, 2)
-DECODE_KERNEL(w4a16_decode_g128_f16_rb4, 128, false, 4)
-DECODE_KERNEL(w4a16_decode_g32_f16_rb1, 32, false, 1)
-DECODE_KERNEL(w4a16_decode_g32_f16_rb2, 32, false, 2)
-DECODE_KERNEL(w4a16_decode_g32_f16_rb4, 32, false, 4)
-DECODE_KERNEL(w4a16_decode_g128_bf16_rb1, 128, true, 1)
-DECODE_KERNEL(w4a16_decode_g128_bf16_rb2, 128, true, 2)
-DECODE_KERNEL(w4a16_decode_g128_bf16_rb4, 128, true, 4)
-DECODE_KERNEL(w4a16_decode_g32_bf16_rb1, 32, true, 1)
-DECODE_KERNEL(w4a16_decode_g32_bf16_rb2, 32, true, 2)
-DECODE_KERNEL(w4a16_decode_g32_bf16_rb4, 32, true, 4)
+DECODE_KERNEL_RB1(w4a16_decode_g128_f16_rb1, 128, false)
+DECODE_KERNEL_RB2_G128(w4a16_decode_g128_f16_rb2, false)
+DECODE_KERNEL_LO3(w4a16_decode_g128_f16_rb4, 128, false, 4)
+DECODE_KERNEL_LO3(w4a16_decode_g32_f16_rb1, 32, false, 1)
+DECODE_KERNEL_LO3(w4a16_decode_g32_f16_rb2, 32, false, 2)
+DECODE_KERNEL_LO3(w4a16_decode_g32_f16_rb4, 32, false, 4)
+DECODE_KERNEL_RB1(w4a16_decode_g128_bf16_rb1, 128, true)
+DECODE_KERNEL_RB2_G128(w4a16_decode_g128_bf16_rb2, true)
+DECODE_KERNEL_LO3(w4a16_decode_g128_bf16_rb4, 128, true, 4)
+DECODE_KERNEL_LO3(w4a16_decode_g32_bf16_rb1, 32, true, 1)
+DECODE_KERNEL_LO3(w4a16_decode_g32_bf16_rb2, 32, true, 2)
+DECODE_KERNEL_LO3(w4a16_decode_g32_bf16_rb4, 32, true, 4)
