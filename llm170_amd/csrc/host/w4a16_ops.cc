@@ -93,7 +93,7 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of};
-    return w4_launch(ctx, sym, (unsigned)grid, 1, 256, 2 * 128 * 72 * 2, params);
+    return w4_launch(ctx, sym, (unsigned)grid, 1, 256, 2 * 128 * 64 * 2, params);
 }
 
 // t > 16 without the prefill kernel (irregular scales): the decode kernel over chunks of 16 rows.

@@ -4,8 +4,9 @@
 //   * workgroup = 4 waves along n, block tile 128 (m) x 256 (n), wave tile 128 x 64 = 4 x 2 MFMA tiles of 32 x 32 with
 //     f32 accumulators in arch VGPRs (128 registers); two workgroups per CU, so one block's barriers and LDS writes
 //     overlap the other's MFMAs;
-//   * x (the A operand) is staged through LDS in k slabs of 64, double buffered, rows padded to 72 halves so the
-//     ds_read_b128 fragment reads are bank-conflict free; rows >= t come from out-of-range buffer loads (zeros);
+//   * x (the A operand) is staged through LDS in k slabs of 64, double buffered, by LDS DMA (buffer_load ... lds:
+//     no staging registers, no ds_write); rows are unpadded and their 16-byte chunks swizzled by row so the
+//     ds_read_b128 fragment reads are bank-conflict free; rows >= t come from out-of-range loads (zeros);
 //   * the weights (B operand) never touch LDS: the tiled layout of w4a16_common.hpp already is the MFMA B layout —
 //     lane (n = l % 32, khalf = l / 32) reads 16 B of tile lane g = 2h + khalf, r = n % 16 of its row block, dword w of
 //     which is the k16 block (w, h) of the k tile — so each wave fetches its 64 x 128 weights with four coalesced
@@ -24,7 +25,8 @@
 #define PF_BM (128 * PF_WM)
 #define PF_BN 256
 #define PF_KS 64          // k per LDS stage
-#define PF_LDA 72         // halves per staged x row (64 + 8 padding)
+#define PF_LDA 64         // halves per staged x row (unpadded; chunks swizzled)
+#define PF_STAGE_BYTES (PF_BM * PF_LDA * 2)
 #define PF_THREADS (256 * PF_WM)
 #define PF_SUPER 8        // super-tile edge: 8 x 8 block tiles run together on one XCD
 
@@ -56,25 +58,25 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     const __amdgpu_buffer_rsrc_t qr = w4_make_rsrc(qt, (unsigned)row_blocks * (unsigned)kt_n * 1024u);
     const __amdgpu_buffer_rsrc_t sr = w4_make_rsrc(st, (unsigned)row_blocks * (unsigned)kg_n * 32u);
 
-    // ---- x staging: PF_BM rows x 64 k per stage = PF_BM * 8 chunks of 16 B, 4 per thread
+    // ---- x staging by LDS DMA (buffer_load ... lds: global -> LDS without passing through registers).  A stage is
+    // PF_BM rows x 64 k = PF_BM * 8 chunks of 16 B, 4 per thread; one instruction of a wave fills 1 KiB of LDS, lane i
+    // at byte 16*i, so rows are 128 B apart without padding.  To keep the fragment reads conflict free the chunks of a
+    // row are stored swizzled: chunk position p of row r holds k chunk p ^ (r & 7) — the lane that fills position p
+    // simply fetches that k chunk.  Rows >= t fetch out of range: zeros.
+    typedef __attribute__((address_space(3))) char lds_char_t;
+    lds_char_t* const lds_base = (lds_char_t*)lds;
     unsigned xa_off[4];
-    int xa_lds[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const int c = tid + i * PF_THREADS, row = c >> 3, col = (c & 7) * 8;
-        xa_off[i] = (m0 + row < t) ? ((unsigned)(m0 + row) * (unsigned)k + (unsigned)col) * 2u : W4_OOB;
-        xa_lds[i] = row * PF_LDA + col;
+        const int c = tid + i * PF_THREADS, row = c >> 3, kc = (c & 7) ^ (row & 7);
+        xa_off[i] = (m0 + row < t) ? ((unsigned)(m0 + row) * (unsigned)k + (unsigned)kc * 8u) * 2u : W4_OOB;
     }
-    u4_t xa[4];
-    auto load_a = [&](int s) {
+    auto load_a = [&](int s, int buf) {
 #pragma unroll
         for (int i = 0; i < 4; i++)
-            xa[i] = __builtin_amdgcn_raw_buffer_load_b128(xr, xa_off[i] + (unsigned)s * (PF_KS * 2u), 0, 0);  // an out-of-range row stays out of range
-    };
-    auto store_a = [&](int buf) {
-        _Float16* base = lds + buf * (PF_BM * PF_LDA);
-#pragma unroll
-        for (int i = 0; i < 4; i++) *reinterpret_cast<u4_t*>(base + xa_lds[i]) = xa[i];
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                xr, (__attribute__((address_space(3))) void*)(lds_base + buf * PF_STAGE_BYTES + (i * PF_THREADS + wave * 64) * 16),
+                16, xa_off[i], s * (PF_KS * 2), 0, 0);
     };
 
     // ---- weights: lane (nl = l % 32, khalf = l / 32); per n sub-tile ni and half h one dwordx4 per k tile
@@ -115,49 +117,71 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     const int a_row = wm * 128 + nl;  // + mi * 32
     const int stages = k / PF_KS;
 
-    load_a(0);
+    load_a(0, 0);
     load_b(bq, sc, 0);
-    store_a(0);
-    __syncthreads();
+    __syncthreads();  // the compiler waits for the LDS DMA (vmcnt) ahead of the barrier
 
     for (int kt = 0; kt < kt_n; kt++) {
 #pragma unroll
         for (int half = 0; half < 2; half++) {
             const int s = kt * 2 + half;
-            if (s + 1 < stages) load_a(s + 1);
+            // stage s+1 goes into the buffer that stage s-1 was read from: every wave is past the barrier that ended it
+            if (s + 1 < stages) load_a(s + 1, (s + 1) & 1);
             if (half == 0 && kt + 1 < kt_n) load_b(bqn, scn, kt + 1);
-            const _Float16* abuf = lds + (s & 1) * (PF_BM * PF_LDA) + a_row * PF_LDA + khalf * 8;
+            const _Float16* abuf = lds + (s & 1) * (PF_BM * PF_LDA) + a_row * PF_LDA;
 #pragma unroll
             for (int kbl = 0; kbl < 4; kbl++) {
                 const int kb = half * 4 + kbl, w = kb >> 1, h = kb & 1;
-                // group boundary: re-express the accumulators in the new group's scale.  The multiply of each
-                // accumulator tile sits right before that tile's first MFMA of the group, so the VALU work of one tile
-                // overlaps the matrix-core time of the previous one.
-                const bool boundary = (G == 128 && kb == 0) || (G == 32 && h == 0);
+                // Group boundary: re-express the accumulators in the next group's scale.
+                //   group 128: the multiply is done at the END of a k tile, tile by tile right after each tile's last
+                //   MFMA of the group, with the scale of the next k tile (already loaded), so the VALU work of tile j
+                //   runs in the shadow of the MFMAs of tiles j+1.. instead of stalling the next stage's first MFMAs;
+                //   group 32: at the first k16 of each 32-k group, before the tile's first MFMA.
+                const bool boundary32 = G == 32 && h == 0;
                 float ratio[2] = {1.f, 1.f};
-                if (boundary) {
+                if (boundary32) {
 #pragma unroll
                     for (int ni = 0; ni < 2; ni++) {
-                        const float s_cur = w4_scale_fast<SBF>(sc[ni][G == 128 ? 0 : w]);
+                        const float s_cur = w4_scale_fast<SBF>(sc[ni][w]);
                         ratio[ni] = unit[ni] / s_cur;
                         unit[ni] = s_cur;
                     }
                 }
+                if (G == 128 && kb == 0 && kt == 0) {  // the very first group: unit = its scale, accumulators are zero
+#pragma unroll
+                    for (int ni = 0; ni < 2; ni++) unit[ni] = w4_scale_fast<SBF>(sc[ni][0]);
+                }
                 h8_t a[4];
 #pragma unroll
                 for (int mi = 0; mi < 4; mi++)
-                    a[mi] = *reinterpret_cast<const h8_t*>(abuf + mi * 32 * PF_LDA + kbl * 16);
+                    a[mi] = *reinterpret_cast<const h8_t*>(abuf + mi * 32 * PF_LDA + (((kbl * 2 + khalf) ^ (nl & 7)) * 8));
+                const bool last128 = G == 128 && kb == 7;  // branch free: the last k tile multiplies by 1
+                float next_ratio[2] = {1.f, 1.f};
+                if (last128) {
+                    const bool more = kt + 1 < kt_n;
+#pragma unroll
+                    for (int ni = 0; ni < 2; ni++) {
+                        const float s_next = more ? w4_scale_fast<SBF>(scn[ni][0]) : unit[ni];
+                        next_ratio[ni] = unit[ni] / s_next;
+                        unit[ni] = s_next;
+                    }
+                }
 #pragma unroll
                 for (int ni = 0; ni < 2; ni++) {
                     const h8_t b = w4_deq8(bq[ni][h][w]);
 #pragma unroll
                     for (int mi = 0; mi < 4; mi++) {
-                        if (boundary) acc[mi][ni] *= ratio[ni];
+                        if (boundary32) acc[mi][ni] *= ratio[ni];
                         acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b, acc[mi][ni], 0, 0, 0);
                     }
                 }
+                if (last128) {
+#pragma unroll
+                    for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+                        for (int mi = 0; mi < 4; mi++) acc[mi][ni] *= next_ratio[ni];
+                }
             }
-            if (s + 1 < stages) store_a((s + 1) & 1);
             __syncthreads();
         }
 #pragma unroll
