@@ -41,15 +41,17 @@ static int launch_lane(w4a16_ctx* ctx, uint64_t q, uint64_t s, uint64_t x, uint6
 
 // Launch shape of the row-block decode kernel.  Measured on MI355X at the 27B layer shapes (gate+up 5120x34816, down
 // 17408x5120, QKV 5120x7168, O 5120x5120): two row blocks per wave with eight waves per block (in-block split-K by 8)
-// is best or within 1 % of best for t <= 8 on every shape; for 9..16 token rows on wide outputs four row blocks per
-// wave halve the x operand traffic.
+// is best or within 1 % of best for 2 <= t <= 8 on every shape and for t = 1 on the narrow outputs; a single token on
+// a wide output runs best with one row block per wave and four waves (5.5 against 5.3 TB/s on gate+up); for 9..16
+// token rows on wide outputs four row blocks per wave halve the x operand traffic.
 static int pick_decode_shape(const w4a16_ctx* ctx, const W4Lin& L, size_t t, int* rb_out, int* waves_out) {
-    const bool wide16 = t > 8 && L.row_blocks >= 1024;
-    int rb = ctx->decode_rows_per_wave ? ctx->decode_rows_per_wave / 16 : (wide16 ? 4 : 2);
+    const bool wide = L.row_blocks >= 1024;
+    const bool wide16 = t > 8 && wide, wide1 = t == 1 && wide;
+    int rb = ctx->decode_rows_per_wave ? ctx->decode_rows_per_wave / 16 : (wide16 ? 4 : wide1 ? 1 : 2);
     if (rb != 1 && rb != 2 && rb != 4) return w4_fail(W4A16_ERR_ARG, "decode: rows_per_wave must be 16, 32 or 64");
     while (rb > 1 && L.row_blocks < (size_t)rb) rb >>= 1;
     const int kt_n = (int)(L.k / 128);
-    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : (wide16 ? 2 : t > 8 ? 4 : 8);
+    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : (wide16 ? 2 : (t > 8 || wide1) ? 4 : 8);
     waves = std::max(1, std::min(std::min(waves, 8), kt_n));
     *rb_out = rb;
     *waves_out = waves;
