@@ -205,14 +205,18 @@ int w4a16_moe_align(w4a16_ctx* ctx, uint64_t idx_dev, size_t ns, size_t n_exp, s
  *               -> c2[slot] = f16(wt[slot] * (W2[expert] * act[slot]))
  *               -> y[token] = sum over the token's slots of c2, in slot order, f32.
  *   x_dev f16 [t][h]; idx_dev int32 [t*top_k]; wt_dev f32 [t*top_k]; y_dev f32 [t][h].
- * Scratch (sorted ids, act, c2) is owned by the context and grown on demand. */
+ * Scratch (sorted ids, act, c2) is owned by the context and grown on demand.
+ * For t <= 4 and top_k <= 8 the call runs in direct mode: no alignment, the gate|up GEMM takes one segment per slot and
+ * one more launch does the down projections of a token's experts, the weight multiply, the f16 rounding of c2 and
+ * the slot-order sum (same values, c2 never reaches memory). */
 int w4a16_moe_ffn(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t idx_dev, uint64_t wt_dev, size_t t,
                   size_t top_k, uint64_t y_dev);
 /* Scratch of the last w4a16_moe_ffn call, for stage-by-stage checks (the reference exposes the same buffers to
  * its moe_selfcheck, w4a16_dec/probe.rs:153): which = 0 sorted ids (int32), 1 expert ids (int32), 2 num_post
- * (int32 [2]), 3 act (f16 [ns][n_ff]), 4 c2 (f16 [ns][h]).  Also reports the segment size used. */
+ * (int32 [2]), 3 act (f16 [ns][n_ff]), 4 c2 (f16 [ns][h]).  Also reports the segment size used (1 = direct mode, where only
+ * act exists). */
 int w4a16_moe_scratch(w4a16_ctx* ctx, int which, uint64_t* dptr, size_t* bytes, size_t* block);
-/* Launch-shape override for the MoE GEMMs (0 = automatic): block = slots per segment (4, 16, 32, 48, 64);
+/* Launch-shape override for the MoE GEMMs (0 = automatic): block = slots per segment (4, 16, 32, 48, 64; 1 = direct mode);
  * waves = waves per workgroup (k split for segments of <= 16 slots, output-row units otherwise). */
 int w4a16_set_moe_shape(w4a16_ctx* ctx, int block, int waves);
 /* Timed back-to-back w4a16_moe_ffn calls (as w4a16_bench_forward); call i uses experts names[i % n_names]. */

@@ -39,6 +39,8 @@ struct W4MoeScratch {
     size_t sorted_cap = 0, expert_cap = 0, act_cap = 0, c2_cap = 0;       // bytes
     size_t sorted_len = 0, expert_len = 0, act_len = 0, c2_len = 0;       // bytes used by the last call
     size_t block = 0;
+    uint64_t iota = 0, always = 0;  // direct mode: identity segment table and a "padded total" no slot index reaches
+    size_t iota_cap = 0;            // entries
 };
 
 // Scratch of the layer chain, grown on demand (reference: dchain / dx16 / dy buffers, w4a16_dec/buffers.rs).

@@ -199,8 +199,9 @@ int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes) {
 // Segment size (slots of one expert per workgroup).  t <= 4: an expert is chosen by at most 4 tokens -> 4;
 // t <= 16 -> 16; beyond, the smallest of 16/32/48/64 that the mean run fills to under 90 %
 // (the reference's rule over its block sizes, kernels/marlin_moe.rs:309-315).
-static size_t pick_block(const w4a16_ctx* ctx, size_t t, size_t ns, size_t n_exp) {
+static size_t pick_block(const w4a16_ctx* ctx, size_t t, size_t ns, size_t n_exp, size_t top_k) {
     if (ctx->moe_block) return (size_t)ctx->moe_block;
+    if (t <= 4 && top_k <= 8) return 1;  // direct mode: no alignment, two launches (see w4a16_moe_ffn)
     if (t <= 4) return 4;
     if (t <= 16) return 16;
     for (size_t b : {16, 32, 48, 64})
@@ -210,7 +211,8 @@ static size_t pick_block(const w4a16_ctx* ctx, size_t t, size_t ns, size_t n_exp
 
 // One grouped GEMM: y[slot] = W[expert(slot)] * x[slot / x_div] over the aligned segments.
 static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_t x, size_t x_rows, size_t x_div,
-                           uint64_t y, int y_f16, uint64_t topw, size_t ns, size_t block, size_t max_segs) {
+                           uint64_t y, int y_f16, uint64_t topw, size_t ns, size_t block, size_t max_segs,
+                           uint64_t sorted, uint64_t eids, uint64_t npost) {
     const size_t n = glu ? 2 * E.n_ff : E.h, k = glu ? E.h : E.n_ff;
     const size_t row_blocks = (n + 15) / 16, kt_n = k / 128;
     const size_t units = glu ? row_blocks / 2 : (row_blocks + 1) / 2;
@@ -219,9 +221,8 @@ static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_
     uint64_t qa = glu ? E.q13 : E.q2, sa = glu ? E.s13 : E.s2;
     unsigned long long qs = glu ? E.q13_stride : E.q2_stride, ss = glu ? E.s13_stride : E.s2_stride;
     int xr = (int)x_rows, xd = (int)x_div, yf = y_f16, blk = (int)block, nsi = (int)ns, rbi = (int)row_blocks,
-        ki = (int)k, ni = (int)n;
-    uint64_t sorted = ctx->moe.sorted, eids = ctx->moe.expert_ids, npost = ctx->moe.num_post;
-    void* p[] = {&qa, &sa, &qs, &ss, &x, &xr, &xd, &y, &yf, &topw, &sorted, &eids, &npost, &blk, &nsi, &rbi, &ki, &ni};
+        ki = (int)k, ni = (int)n, nei = (int)E.n_exp;
+    void* p[] = {&qa, &sa, &qs, &ss, &x, &xr, &xd, &y, &yf, &topw, &sorted, &eids, &npost, &blk, &nsi, &rbi, &ki, &ni, &nei};
     char sym[80];
     const char* fam = E.scale_bf16 ? "bf16" : "f16";
     if (block <= 16) {
@@ -241,6 +242,47 @@ static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_
     return w4_launch(ctx, sym, (unsigned)(max_segs * groups), 1, (unsigned)(waves * 64), shmem, p);
 }
 
+// Direct mode for decode steps: no alignment pass.  The gate|up GEMM runs one segment per slot — the segment table is
+// the identity, the expert table is idx itself, the "padded total" a constant no slot index reaches — and
+// w4a16_moe_*_down_sum folds the down projection of a token's experts, the routing-weight multiply, the f16 rounding
+// of c2 and the slot-order sum into one launch of top_k waves per block.  Experts chosen by several tokens are
+// streamed once per token, which is cheaper than the two extra launches for a handful of tokens.
+static int moe_ffn_direct(w4a16_ctx* ctx, const char* name, const W4Experts& E, uint64_t x_dev, uint64_t idx_dev,
+                          uint64_t wt_dev, size_t t, size_t top_k, uint64_t y_dev) {
+    if (top_k > 8) return w4_fail(W4A16_ERR_UNSUPPORTED, "moe_ffn %s: direct mode needs top_k <= 8 (got %zu)", name, top_k);
+    const size_t ns = t * top_k;
+    W4MoeScratch& S = ctx->moe;
+    S.block = 1;
+    S.sorted_len = S.expert_len = S.c2_len = 0;
+    S.act_len = ns * E.n_ff * 2;
+    W4_TRY(w4_ensure(ctx, &S.act, &S.act_cap, S.act_len));
+    if (S.iota_cap < ns) {
+        const size_t cap = std::max<size_t>(ns, 256);
+        std::vector<int32_t> host(cap);
+        for (size_t i = 0; i < cap; i++) host[i] = (int32_t)i;
+        size_t bytes_cap = S.iota_cap * 4;
+        W4_TRY(w4_ensure(ctx, &S.iota, &bytes_cap, cap * 4));
+        W4_TRY(w4a16_h2d(ctx, S.iota, host.data(), cap * 4));
+        S.iota_cap = cap;
+    }
+    if (!S.always) {
+        const int32_t big[2] = {0x7fffffff, 0};
+        W4_TRY(w4a16_alloc(ctx, 8, &S.always));
+        W4_TRY(w4a16_h2d(ctx, S.always, big, 8));
+    }
+    // gate|up with the SiLU*up epilogue, one slot per segment
+    W4_TRY(launch_moe_gemm(ctx, E, true, x_dev, t, top_k, S.act, 1, 0, ns, 1, ns, S.iota, idx_dev, S.always));
+    // down + routing weight + f16 rounding + slot-order sum
+    const size_t row_blocks = (E.h + 15) / 16, units = (row_blocks + 1) / 2;
+    uint64_t qa = E.q2, sa = E.s2;
+    unsigned long long qs = E.q2_stride, ss = E.s2_stride;
+    int tk = (int)top_k, nsi = (int)ns, rbi = (int)row_blocks, ki = (int)E.n_ff, ni = (int)E.h, nei = (int)E.n_exp;
+    void* p[] = {&qa, &sa, &qs, &ss, &S.act, &idx_dev, &wt_dev, &y_dev, &tk, &nsi, &rbi, &ki, &ni, &nei};
+    char sym[80];
+    snprintf(sym, sizeof sym, "w4a16_moe_g%zu_%s_down_sum", E.group, E.scale_bf16 ? "bf16" : "f16");
+    return w4_launch(ctx, sym, (unsigned)(t * units), 1, (unsigned)(top_k * 64), (unsigned)(top_k * 2 * 64 * 16), p);
+}
+
 extern "C" int w4a16_moe_ffn(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t idx_dev, uint64_t wt_dev,
                              size_t t, size_t top_k, uint64_t y_dev) {
     W4Experts* E = nullptr;
@@ -250,9 +292,10 @@ extern "C" int w4a16_moe_ffn(w4a16_ctx* ctx, const char* name, uint64_t x_dev, u
         return w4_fail(W4A16_ERR_SHAPE, "moe_ffn %s: t=%zu top_k=%zu experts=%zu", name, t, top_k, E->n_exp);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     const size_t ns = t * top_k;
-    const size_t block = pick_block(ctx, t, ns, E->n_exp);
-    if (block != 4 && block != 16 && block != 32 && block != 48 && block != 64)
-        return w4_fail(W4A16_ERR_ARG, "moe_ffn %s: segment size %zu not in {4,16,32,48,64}", name, block);
+    const size_t block = pick_block(ctx, t, ns, E->n_exp, top_k);
+    if (block != 1 && block != 4 && block != 16 && block != 32 && block != 48 && block != 64)
+        return w4_fail(W4A16_ERR_ARG, "moe_ffn %s: segment size %zu not in {1,4,16,32,48,64}", name, block);
+    if (block == 1) return moe_ffn_direct(ctx, name, *E, x_dev, idx_dev, wt_dev, t, top_k, y_dev);
     // every expert's run is padded to a multiple of block: at most ns/block full segments plus one partial per expert
     const size_t max_segs = std::min(ns, ns / block + E->n_exp);
     W4MoeScratch& S = ctx->moe;
@@ -269,9 +312,11 @@ extern "C" int w4a16_moe_ffn(w4a16_ctx* ctx, const char* name, uint64_t x_dev, u
     W4_TRY(w4_ensure(ctx, &S.c2, &S.c2_cap, S.c2_len));
     W4_TRY(w4a16_moe_align(ctx, idx_dev, ns, E->n_exp, block, S.sorted, S.expert_ids, S.num_post));
     // gate|up with the SiLU*up epilogue: slot j reads token j / top_k
-    W4_TRY(launch_moe_gemm(ctx, *E, true, x_dev, t, top_k, S.act, 1, 0, ns, block, max_segs));
+    W4_TRY(launch_moe_gemm(ctx, *E, true, x_dev, t, top_k, S.act, 1, 0, ns, block, max_segs, S.sorted, S.expert_ids,
+                           S.num_post));
     // down, multiplied by the routing weight: slot j reads act row j
-    W4_TRY(launch_moe_gemm(ctx, *E, false, S.act, ns, 1, S.c2, 1, wt_dev, ns, block, max_segs));
+    W4_TRY(launch_moe_gemm(ctx, *E, false, S.act, ns, 1, S.c2, 1, wt_dev, ns, block, max_segs, S.sorted, S.expert_ids,
+                           S.num_post));
     int ti = (int)t, hi = (int)E->h, ki = (int)top_k;
     void* p[] = {&S.c2, &y_dev, &ti, &hi, &ki};
     return w4_launch(ctx, "w4a16_moe_topk_sum_f16", std::min<unsigned>(ceil_div(t * E->h / (E->h % 8 == 0 ? 8 : 1), 256), 4096), 1, 256, 0, p);
@@ -295,8 +340,9 @@ extern "C" int w4a16_moe_scratch(w4a16_ctx* ctx, int which, uint64_t* dptr, size
 
 extern "C" int w4a16_set_moe_shape(w4a16_ctx* ctx, int block, int waves) {
     if (!ctx) return w4_fail(W4A16_ERR_ARG, "set_moe_shape: null context");
-    if ((block != 0 && block != 4 && block != 16 && block != 32 && block != 48 && block != 64) || waves < 0 || waves > 8)
-        return w4_fail(W4A16_ERR_ARG, "set_moe_shape: block in {0,4,16,32,48,64}, waves in 0..8");
+    if ((block != 0 && block != 1 && block != 4 && block != 16 && block != 32 && block != 48 && block != 64) || waves < 0 ||
+        waves > 8)
+        return w4_fail(W4A16_ERR_ARG, "set_moe_shape: block in {0,1,4,16,32,48,64}, waves in 0..8");
     ctx->moe_block = block;
     ctx->moe_waves = waves;
     return 0;

@@ -14,6 +14,9 @@
 //       - moe_mm (segments of 16..64 slots, prefill chunks): the waves of a block take different output rows of the
 //         same segment and share the gathered x rows through LDS (double buffered, one k tile per stage), so x is
 //         fetched once per block instead of once per wave.
+//   * decode steps of at most four tokens skip the alignment: the gate|up GEMM runs one segment per slot (segment table
+//     = identity, expert table = idx itself) and moe_down_sum does the down projection of a token's experts, the
+//     routing-weight multiply, the f16 rounding and the slot-order sum in one launch — two launches per FFN;
 //   * GLU epilogue: a wave owns gate row block u and up row block u + n_ff/16, rounds both sums to f16 (the reference
 //     materialises them as f16, moe.cu:1649-1660) and writes silu(g)*u as f16 — the intermediate never reaches
 //     memory.  LIN epilogue: optional multiply by the slot's routing weight, f16 or f32 rows scattered by slot id.
@@ -107,14 +110,15 @@ __device__ __forceinline__ void moe_store(f4_t a0, f4_t a1, int slot, int q, int
 //          tiles and [row_blocks][k/G][16] scales.  x: f16 [x_rows][k]; slot j reads row j / x_div.
 //   y: GLU -> f16 [ns][n/2]; LIN -> f16 or f32 [ns][n].  topw: null or f32 [ns] (LIN only).
 //   sorted_ids[seg*blk + i]: slot id or the sentinel ns; expert_ids[seg]; num_post[0] = padded slot total.
+//   A segment whose expert id is outside 0..n_exp-1 is skipped (its slots stay unwritten).
 #define MOE_PARAMS                                                                                                  \
     const char *__restrict__ qa, const char *__restrict__ sa, unsigned long long q_stride,                          \
         unsigned long long s_stride, const uint16_t *__restrict__ x, int x_rows, int x_div, void *__restrict__ y,   \
         int y_f16, const float *__restrict__ topw, const int *__restrict__ sorted_ids,                              \
         const int *__restrict__ expert_ids, const int *__restrict__ num_post, int blk, int ns, int row_blocks, int k, \
-        int n
+        int n, int n_exp
 #define MOE_ARGS \
-    qa, sa, q_stride, s_stride, x, x_rows, x_div, y, y_f16, topw, sorted_ids, expert_ids, num_post, blk, ns, row_blocks, k, n
+    qa, sa, q_stride, s_stride, x, x_rows, x_div, y, y_f16, topw, sorted_ids, expert_ids, num_post, blk, ns, row_blocks, k, n, n_exp
 
 // ---------------------------------------------------------------------------------------------------- moe_dec
 template <int RB, int XL>
@@ -136,6 +140,7 @@ __device__ __forceinline__ void moe_dec_body(MOE_PARAMS) {
     const int seg = blockIdx.x / units, u = blockIdx.x % units;
     if (seg * blk >= num_post[0]) return;
     const int e = __builtin_amdgcn_readfirstlane(expert_ids[seg]);
+    if ((unsigned)e >= (unsigned)n_exp) return;  // uniform for the block
     const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
     const int kt0 = (kt_n * wave) / W, kt1 = (kt_n * (wave + 1)) / W;
     const int m = lane & 15, g = lane >> 4;
@@ -243,6 +248,144 @@ __device__ __forceinline__ void moe_dec_body(MOE_PARAMS) {
     moe_store<GLU>(acc[0], acc[1], slot, g, u, rbA, rbB, haveB, y, y_f16, wgt, n);
 }
 
+// ---------------------------------------------------------------------------------------------------- moe_down_sum
+// Decode steps (a handful of tokens): the down projection of all of a token's experts and the slot-order sum in one
+// launch.  One block = (token, unit of two row blocks); wave w < top_k owns slot token*top_k + w: it streams that
+// expert's rows over the whole k range with the slot's activation row as x, multiplies by the routing weight and
+// rounds to f16 exactly as the staged path materialises c2; wave 0 then adds the waves' values in slot order in f32
+// (the same order as the separate sum kernel) and writes y f32 [t][n].  No alignment pass is needed: the expert of
+// a slot is read straight from idx.
+template <int G, bool SBF, int DEPTH>
+__device__ __forceinline__ void moe_down_sum_body(const char* __restrict__ qa, const char* __restrict__ sa,
+                                                  unsigned long long q_stride, unsigned long long s_stride,
+                                                  const uint16_t* __restrict__ act, const int* __restrict__ idx,
+                                                  const float* __restrict__ topw, float* __restrict__ y, int top_k,
+                                                  int ns, int row_blocks, int k, int n, int n_exp) {
+    extern __shared__ f4_t red[];  // [top_k][2][64]
+    constexpr int GPT = W4_TILE_K / G;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int units = (row_blocks + 1) >> 1;
+    const int token = blockIdx.x / units, u = blockIdx.x % units;
+    const int slot = token * top_k + wave;
+    const int e_raw = __builtin_amdgcn_readfirstlane(idx[slot]);
+    const bool valid = (unsigned)e_raw < (unsigned)n_exp;  // an out-of-range expert id contributes zero
+    const int e = valid ? e_raw : 0;
+    const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
+    const int m = lane & 15, g = lane >> 4;
+    const int rbA = 2 * u, rbB = min(2 * u + 1, row_blocks - 1);
+    const bool haveB = 2 * u + 1 < row_blocks;
+
+    const __amdgpu_buffer_rsrc_t qr = w4_make_rsrc(qa + (unsigned long long)e * q_stride,
+                                                   valid ? (unsigned)row_blocks * (unsigned)kt_n * 1024u : 0u);
+    const __amdgpu_buffer_rsrc_t sr = w4_make_rsrc(sa + (unsigned long long)e * s_stride,
+                                                   valid ? (unsigned)row_blocks * (unsigned)kg_n * 32u : 0u);
+    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(act, (unsigned)ns * (unsigned)k * 2u);
+    // one x load per k tile: lane m = 4c fetches chunk c of the slot's row; DPP row shifts bring chunk c to column 0
+    const unsigned xoff = (m & 3) == 0 ? ((unsigned)slot * (unsigned)k + (unsigned)((m >> 2) * 32 + g * 8)) * 2u : W4_OOB;
+    const unsigned qoff[2] = {(unsigned)rbA * (unsigned)kt_n * 1024u + (unsigned)lane * 16u,
+                              (unsigned)rbB * (unsigned)kt_n * 1024u + (unsigned)lane * 16u};
+    const unsigned sg = G == 32 ? (unsigned)(lane & 3) * 32u : 0u;
+    const unsigned soff[2] = {(unsigned)rbA * (unsigned)kg_n * 32u + sg + (unsigned)g * 8u,
+                              (unsigned)rbB * (unsigned)kg_n * 32u + sg + (unsigned)g * 8u};
+    f4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+
+    MoeDecStage<2, 1> stage[DEPTH];
+    auto load = [&](MoeDecStage<2, 1>& s_, int kt) {
+        const bool live = kt < kt_n;
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+            s_.q[rb] = __builtin_amdgcn_raw_buffer_load_b128(qr, live ? qoff[rb] + (unsigned)kt * 1024u : W4_OOB, 0, 2);
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+            s_.s[rb] = __builtin_amdgcn_raw_buffer_load_b64(sr, live ? soff[rb] + (unsigned)kt * (GPT * 32u) : W4_OOB, 0, 0);
+        s_.x[0] = __builtin_amdgcn_raw_buffer_load_b128(xr, live ? xoff + (unsigned)(kt * W4_TILE_K) * 2u : W4_OOB, 0, 0);
+    };
+    auto compute = [&](const MoeDecStage<2, 1>& s_) {
+        u4_t xb[4];
+        xb[0] = s_.x[0];
+        xb[1] = moe_row_shl<4>(s_.x[0]);
+        xb[2] = moe_row_shl<8>(s_.x[0]);
+        xb[3] = moe_row_shl<12>(s_.x[0]);
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++) {
+            const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+            if (G == 128) {
+                f4_t part = zero;
+#pragma unroll
+                for (int w = 0; w < 4; w++)
+                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
+                                                                  __builtin_bit_cast(h8_t, xb[w]), part, 0, 0, 0);
+                acc[rb] += moe_scale4<G, SBF, 0>(s_.s[rb]) * part;
+            } else {
+                f4_t p0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][0]), __builtin_bit_cast(h8_t, xb[0]), zero, 0, 0, 0);
+                f4_t p1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][1]), __builtin_bit_cast(h8_t, xb[1]), zero, 0, 0, 0);
+                f4_t p2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][2]), __builtin_bit_cast(h8_t, xb[2]), zero, 0, 0, 0);
+                f4_t p3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][3]), __builtin_bit_cast(h8_t, xb[3]), zero, 0, 0, 0);
+                acc[rb] += moe_scale4<G, SBF, 0>(s_.s[rb]) * p0;
+                acc[rb] += moe_scale4<G, SBF, 1>(s_.s[rb]) * p1;
+                acc[rb] += moe_scale4<G, SBF, 2>(s_.s[rb]) * p2;
+                acc[rb] += moe_scale4<G, SBF, 3>(s_.s[rb]) * p3;
+            }
+        }
+    };
+    const int rounds = kt_n / DEPTH;
+    for (int r = -1; r < rounds; r++) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            if (r >= 0) compute(stage[d]);
+            __builtin_amdgcn_sched_barrier(0);
+            load(stage[d], (r + 1) * DEPTH + d);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < DEPTH - 1; d++)
+        if (rounds * DEPTH + d < kt_n) compute(stage[d]);
+
+    // c2 of this slot: routing weight, one rounding to f16 (the value the staged path stores), back to f32
+    const float wgt = topw[slot];
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[rb][i] = moe_round_f16(acc[rb][i] * wgt);
+    red[(wave * 2 + 0) * 64 + lane] = acc[0];
+    red[(wave * 2 + 1) * 64 + lane] = acc[1];
+    __syncthreads();
+    if (wave != 0 || m != 0) return;
+    f4_t sum[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    for (int w = 0; w < top_k; w++) {
+        sum[0] += red[(w * 2 + 0) * 64 + lane];
+        sum[1] += red[(w * 2 + 1) * 64 + lane];
+    }
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) {
+        if (rb == 1 && !haveB) break;
+        const int row = (rb == 0 ? rbA : rbB) * 16 + 4 * g;
+        float* yo = y + (size_t)token * n + row;
+        if (row + 3 < n) {
+            *reinterpret_cast<f4_t*>(yo) = sum[rb];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (row + i < n) yo[i] = sum[rb][i];
+        }
+    }
+}
+
+#define MOE_DOWN_SUM_KERNEL(NAME, G, SBF)                                                                         \
+    extern "C" __global__ __launch_bounds__(512) void NAME(                                                       \
+        const char* qa, const char* sa, unsigned long long q_stride, unsigned long long s_stride,                 \
+        const uint16_t* act, const int* idx, const float* topw, float* y, int top_k, int ns, int row_blocks, int k, \
+        int n, int n_exp) {                                                                                       \
+        moe_down_sum_body<G, SBF, 3>(qa, sa, q_stride, s_stride, act, idx, topw, y, top_k, ns, row_blocks, k, n,  \
+                                     n_exp);                                                                      \
+    }
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g32_f16_down_sum, 32, false)
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g32_bf16_down_sum, 32, true)
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g128_f16_down_sum, 128, false)
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g128_bf16_down_sum, 128, true)
+
 // ---------------------------------------------------------------------------------------------------- moe_mm
 template <int RB>
 struct MoeMmStage {
@@ -266,6 +409,7 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     const bool active = u_raw < units;  // a surplus wave repeats the last unit and stores nothing
     const int u = min(u_raw, units - 1);
     const int e = __builtin_amdgcn_readfirstlane(expert_ids[seg]);
+    if ((unsigned)e >= (unsigned)n_exp) return;  // uniform for the block, before any barrier
     const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
     const int c = lane & 15, q = lane >> 4;
     const int rbA = GLU ? u : 2 * u, rbB = GLU ? u + units : min(2 * u + 1, row_blocks - 1);

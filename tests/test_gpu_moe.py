@@ -116,10 +116,10 @@ def _run_ffn(dec, name, x, idx, wt, t, k, h):
     ns = t * k
     spec = dec.experts_spec(name)
     act, blk = dec.moe_scratch(3, np.uint16)
-    c2, _ = dec.moe_scratch(4, np.uint16)
+    c2 = None if blk == 1 else dec.moe_scratch(4, np.uint16)[0].reshape(ns, h)  # direct mode keeps c2 in registers
     for p in (px, pi, pw, py):
         cc.free(p)
-    return y, act.reshape(ns, spec["n_ff"]), c2.reshape(ns, h), blk
+    return y, act.reshape(ns, spec["n_ff"]), c2, blk
 
 
 def _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, what, threads=8):
@@ -151,10 +151,21 @@ def _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf
     assert same > 0.97, (what, "act identical fraction", same)
     # stage 2: c2 from the device's own act, against the oracle run on that same act
     st2 = orc.moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, threads=threads, act_in=act)
-    m2 = parity.assert_close(_f16(c2), _f16(st2["c2"]), what + " c2")
-    # stage 3: the slot-order f32 sum of the device's c2 is exact arithmetic on f16 inputs -> bit for bit
-    y3 = orc.moe_topk_sum_f16(c2, t, h, k)
-    assert np.array_equal(y.view(np.uint32), y3.view(np.uint32)), what + " sum"
+    if c2 is not None:
+        m2 = parity.assert_close(_f16(c2), _f16(st2["c2"]), what + " c2")
+        # stage 3: the slot-order f32 sum of the device's c2 is exact arithmetic on f16 inputs -> bit for bit
+        y3 = orc.moe_topk_sum_f16(c2, t, h, k)
+        assert np.array_equal(y.view(np.uint32), y3.view(np.uint32)), what + " sum"
+    else:
+        # direct mode: down projection, weight, f16 rounding and sum are one launch; y against the oracle's y from the
+        # device's own act.  Each of the k terms may round to the neighbouring f16 (the f32 sums differ in their last
+        # bits), which moves y by one f16 step of that term; the f32 additions themselves are exact here.
+        c2r = _f16(st2["c2"]).astype(np.float64).reshape(t, k, h)
+        bound = parity.f16_ulp(c2r).sum(axis=1) + 1e-7
+        dy = np.abs(y.astype(np.float64) - st2["y"].astype(np.float64))
+        assert np.all(dy <= bound), (what, "y from act", float((dy / bound).max()))
+        assert np.mean(y == st2["y"]) > 0.97, (what, "y identical fraction", float(np.mean(y == st2["y"])))
+        m2 = parity.compare(y, st2["y"])
     # end to end against the oracle's independent run
     m = parity.compare(y, full["y"])
     assert m["rel_l2"] <= parity.REL_L2_TOL, (what, m)
@@ -173,13 +184,13 @@ def test_moe_ffn_small(dec, orc, small_experts, group, bf, t):
     _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, "small g%d bf%d t%d blk%d" % (group, bf, t, blk))
 
 
-@pytest.mark.parametrize("block,waves", [(4, 1), (4, 2), (16, 1), (16, 4), (32, 4), (48, 8), (64, 4)])
+@pytest.mark.parametrize("block,waves", [(1, 0), (1, 2), (4, 1), (4, 2), (16, 1), (16, 4), (32, 4), (48, 8), (64, 4)])
 def test_moe_ffn_launch_shapes_agree(dec, orc, small_experts, block, waves):
     """Every segment size and wave count computes the same FFN (t small enough for the 4-slot segments)."""
     say("moe shapes", block, waves)
     name, q13, s13, q2, s2 = small_experts[(32, False)]
     E, h, n_ff, k = SMALL["E"], SMALL["h"], SMALL["n_ff"], SMALL["k"]
-    t = 4 if block == 4 else 13 if block == 16 else 90
+    t = 4 if block <= 4 else 13 if block == 16 else 90
     x = gen.normal_f16(77, (t, h))
     idx, wt = ops.moe_topk(gen.router_logits(t, E, seed=3), k)
     dec.set_moe_shape(block, waves)
@@ -246,3 +257,35 @@ def test_moe_errors(dec, small_experts):
                            np.zeros(4, np.uint16), 2, 256, 128, 32, False)
     with pytest.raises(ops.W4a16Error):
         dec.set_moe_shape(5, 0)
+
+
+def test_moe_direct_and_aligned_modes_agree(dec, orc, small_experts):
+    """t <= 4 runs without the alignment pass by default; forcing the aligned path gives the same act bit for bit and
+    a y that differs at most by f16 rounding flips of single c2 terms."""
+    name, q13, s13, q2, s2 = small_experts[(32, False)]
+    E, h, n_ff, k = SMALL["E"], SMALL["h"], SMALL["n_ff"], SMALL["k"]
+    for t in (1, 2, 4):
+        x = gen.normal_f16(500 + t, (t, h))
+        idx, wt = ops.moe_topk(gen.router_logits(t, E, seed=40 + t), k)
+        y_d, act_d, c2_d, blk_d = _run_ffn(dec, name, x, idx, wt, t, k, h)
+        assert blk_d == 1 and c2_d is None
+        dec.set_moe_shape(4, 0)
+        try:
+            y_a, act_a, c2_a, blk_a = _run_ffn(dec, name, x, idx, wt, t, k, h)
+        finally:
+            dec.set_moe_shape(0, 0)
+        assert blk_a == 4 and np.array_equal(act_d, act_a)
+        parity.assert_close(y_d, y_a, "direct vs aligned t%d" % t)
+
+
+def test_moe_direct_mode_out_of_range_expert_contributes_zero(dec, orc, small_experts):
+    name, q13, s13, q2, s2 = small_experts[(32, False)]
+    E, h, n_ff, k = SMALL["E"], SMALL["h"], SMALL["n_ff"], SMALL["k"]
+    x = gen.normal_f16(77, (2, h))
+    idx = np.array([[1, 99], [3, 2]], np.int32)  # expert 99 does not exist
+    wt = np.full((2, k), 0.5, np.float32)
+    y, act, c2, blk = _run_ffn(dec, name, x, idx, wt, 2, k, h)
+    ok_idx = np.array([[1, 1], [3, 2]], np.int32)
+    ok_wt = np.array([[0.5, 0.0], [0.5, 0.5]], np.float32)
+    ref = orc.moe_ffn(x, ok_idx, ok_wt, q13, s13, q2, s2, h, n_ff, 32, False)
+    assert parity.compare(y, ref["y"])["rel_l2"] < 1e-3
