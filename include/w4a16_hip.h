@@ -153,6 +153,11 @@ int w4a16_lin_untile(w4a16_ctx* ctx, const char* name, uint64_t q_out_dev, uint6
  * sk_ksp, w4a16_dec/kernels/decode.rs:3-16). */
 int w4a16_set_decode_shape(w4a16_ctx* ctx, int rows_per_wave, int waves_per_block);
 
+/* Split-K override for the prefill kernel: 0 = automatic (split when the tile grid alone would leave most of the chip
+ * idle — narrow outputs at moderate t; the reference's prefill path makes the same choice inside its vendored GEMM),
+ * -1 = never, n >= 1 = exactly n k slices (clamped so a slice has at least 4 k tiles). */
+int w4a16_set_prefill_ksplit(w4a16_ctx* ctx, int ksplit);
+
 /* run_bench_gemv / run_bench_gemm (crates/server/src/probes/w4a16/gpu/bench.rs:366-433): `warmup` untimed then
  * `reps` timed back-to-back lin_forward launches on the launch stream, one synchronisation at the end.  Launch i
  * uses linear names[i % n_names] — rotating over copies whose total size exceeds the last-level caches gives the

@@ -87,15 +87,44 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     if (t * L.k * 2 >= 0x80000000ull || L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
         return w4_fail(W4A16_ERR_SHAPE, "prefill: x or the tiled weights reach 2 GiB, beyond the buffer-descriptor range");
     // block tile 128 (m) x 256 (n); 8 x 8 super-tiles dealt round-robin to the 8 XCDs (kernels/prefill.hip)
+    // Super-tile shape: up to 8 x 8, narrowed along n on small grids until there are at least two super-tiles per XCD.
     const size_t tiles_m = (t + 127) / 128, tiles_n = (L.n + 255) / 256;
-    const size_t supers = ((tiles_m + 7) / 8) * ((tiles_n + 7) / 8);
-    const size_t grid = ((supers + 7) / 8) * 64 * 8;
+    const size_t sup_m = std::min<size_t>(8, tiles_m), sm_n = (tiles_m + sup_m - 1) / sup_m;
+    const size_t sup_n = std::max<size_t>(1, std::min<size_t>(8, tiles_n * sm_n / 16));
+    const size_t supers = sm_n * ((tiles_n + sup_n - 1) / sup_n);
+    const size_t grid = ((supers + 7) / 8) * (sup_m * sup_n) * 8;
+    // Split-K when the tile grid alone leaves much of the chip idle (two workgroups fit a CU: 512 slots): k slices are
+    // doubled until the launch has at least 512 workgroups (measured best at the 27B down projection: 8 slices at
+    // t = 512, 4 at t = 1024), each slice at least 4 k tiles.  Partials are f32 in a context-owned workspace, added in
+    // slice order by a second launch (deterministic).
+    const size_t tiles = tiles_m * tiles_n, kt_n = L.k / 128;
+    size_t nks = 1;
+    if (ctx->prefill_ksplit > 0) {
+        nks = (size_t)ctx->prefill_ksplit;
+    } else if (ctx->prefill_ksplit == 0 && L.n % 4 == 0) {
+        while (tiles * nks < 512 && nks < 8) nks *= 2;
+    }
+    nks = std::max<size_t>(1, std::min(nks, kt_n / 4));
     char sym[64];
     snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s", L.group, L.scale_bf16 ? "bf16" : "f16");
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
-    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of};
-    return w4_launch(ctx, sym, (unsigned)grid, 1, 256, 2 * 128 * 64 * 2, params);
+    int spm = (int)sup_m, spn = (int)sup_n;
+    if (nks == 1) {
+        void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &spm, &spn};
+        return w4_launch(ctx, sym, (unsigned)grid, 1, 256, 2 * 128 * 64 * 2, params);
+    }
+    if (L.n % 4 != 0) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: split-K needs n %% 4 == 0");
+    const size_t count = t * L.n;
+    W4_TRY(w4_ensure(ctx, &ctx->prefill_ws, &ctx->prefill_ws_cap, count * 4 * nks));
+    uint64_t ws = ctx->prefill_ws;
+    int zero = 0;
+    void* params[] = {&qt, &st, &x, &ws, &row_blocks, &ki, &ni, &ti, &zero, &spm, &spn};
+    W4_TRY(w4_launch(ctx, sym, (unsigned)grid, (unsigned)nks, 256, 2 * 128 * 64 * 2, params));
+    int nksi = (int)nks;
+    size_t cnt = count;
+    void* rp[] = {&ws, &y, &nksi, &cnt, &of};
+    return w4_launch(ctx, "w4a16_prefill_splitk_sum", std::min<unsigned>(ceil_div(count / 4, 256), 4096), 1, 256, 0, rp);
 }
 
 // t > 16 without the prefill kernel (irregular scales): the decode kernel over chunks of 16 rows.
@@ -325,6 +354,13 @@ extern "C" int w4a16_lin_untile(w4a16_ctx* ctx, const char* name, uint64_t q_out
     W4_TRY(w4_launch(ctx, "w4a16_untile_q", ceil_div(L->n * (L->k / 8), 256), 1, 256, 0, pq));
     void* ps[] = {&L->s_tiled, &s_out_dev, &ni, &kgi};
     return w4_launch(ctx, "w4a16_untile_s", ceil_div(L->n * (L->k / L->group), 256), 1, 256, 0, ps);
+}
+
+extern "C" int w4a16_set_prefill_ksplit(w4a16_ctx* ctx, int ksplit) {
+    if (!ctx) return w4_fail(W4A16_ERR_ARG, "set_prefill_ksplit: null context");
+    if (ksplit < -1 || ksplit > 16) return w4_fail(W4A16_ERR_ARG, "set_prefill_ksplit: -1 (never), 0 (automatic) or 1..16");
+    ctx->prefill_ksplit = ksplit;
+    return 0;
 }
 
 extern "C" int w4a16_set_decode_shape(w4a16_ctx* ctx, int rows_per_wave, int waves_per_block) {

@@ -15,8 +15,9 @@
 //     holds sum / s_g; at each group boundary it is multiplied by s_prev / s_cur and the new group's integer products
 //     are added by the MFMA itself; the epilogue multiplies by the last scale.  No weight is rounded to f16 and no
 //     second accumulator set is needed.  (Linears with a zero or non-finite scale are not routed here.)
-//   * workgroups are numbered so that the ~64 blocks resident on one XCD form an 8 x 8 super-tile: each x slab and
-//     each weight panel is fetched into that L2 once per eight uses.
+//   * workgroups are numbered so that the blocks resident on one XCD form a super-tile (8 x 8 block tiles on large
+//     grids: each x slab and each weight panel is fetched into that L2 once per eight uses; smaller on small grids so
+//     that all eight XCDs get work).
 #include "w4a16_common.hpp"
 
 #ifndef PF_WM
@@ -28,12 +29,11 @@
 #define PF_LDA 64         // halves per staged x row (unpadded; chunks swizzled)
 #define PF_STAGE_BYTES (PF_BM * PF_LDA * 2)
 #define PF_THREADS (256 * PF_WM)
-#define PF_SUPER 8        // super-tile edge: 8 x 8 block tiles run together on one XCD
 
 template <int G, bool SBF>
 __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                              const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
-                                             int k, int n, int t, int out_f16) {
+                                             int k, int n, int t, int out_f16, int sup_m, int sup_n) {
     extern __shared__ _Float16 lds[];  // 2 stages x [PF_BM][PF_LDA]
     constexpr int GPT = W4_TILE_K / G;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -42,15 +42,16 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
 
     // XCD-aware tile numbering.  Block b runs on XCD b % 8 and is the (b / 8)-th block of that XCD; consecutive
-    // blocks of an XCD walk one super-tile of PF_SUPER x PF_SUPER block tiles (m fastest), so the ~64 blocks resident
-    // on an XCD at a time share 8 x slabs and 8 weight panels through its L2.  Super-tiles are dealt round-robin
-    // to the XCDs.
+    // blocks of an XCD walk one super-tile of sup_m x sup_n block tiles (m fastest), so the blocks resident on an XCD
+    // at a time share x slabs and weight panels through its L2.  Super-tiles are dealt round-robin to the XCDs.  The
+    // host picks the super-tile shape: 8 x 8 on large grids, smaller on small ones so that every XCD gets work.
     const int tiles_m = (t + PF_BM - 1) / PF_BM, tiles_n = (n + PF_BN - 1) / PF_BN;
-    const int sm_n = (tiles_m + PF_SUPER - 1) / PF_SUPER, sn_n = (tiles_n + PF_SUPER - 1) / PF_SUPER;
+    const int sm_n = (tiles_m + sup_m - 1) / sup_m, sn_n = (tiles_n + sup_n - 1) / sup_n;
+    const int per = sup_m * sup_n;
     const int j = blockIdx.x >> 3;
-    const int super = (blockIdx.x & 7) + 8 * (j / (PF_SUPER * PF_SUPER)), within = j % (PF_SUPER * PF_SUPER);
+    const int super = (blockIdx.x & 7) + 8 * (j / per), within = j % per;
     if (super >= sm_n * sn_n) return;  // uniform for the whole block
-    const int tm = (super % sm_n) * PF_SUPER + within % PF_SUPER, tn = (super / sm_n) * PF_SUPER + within / PF_SUPER;
+    const int tm = (super % sm_n) * sup_m + within % sup_m, tn = (super / sm_n) * sup_n + within / sup_m;
     if (tm >= tiles_m || tn >= tiles_n) return;
     const int m0 = tm * PF_BM, n0 = tn * PF_BN;
 
@@ -115,19 +116,22 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     float unit[2] = {1.f, 1.f};  // scale the accumulator of sub-tile ni is currently expressed in
 
     const int a_row = wm * 128 + nl;  // + mi * 32
-    const int stages = k / PF_KS;
+    // split-K over gridDim.y (narrow outputs at moderate t, where the tile grid alone cannot fill the chip): this
+    // block covers k tiles [kt_lo, kt_hi) and writes an f32 partial; a second launch adds the partials in order
+    const int kt_lo = (kt_n * (int)blockIdx.y) / (int)gridDim.y, kt_hi = (kt_n * ((int)blockIdx.y + 1)) / (int)gridDim.y;
+    const int stages = 2 * kt_hi;
 
-    load_a(0, 0);
-    load_b(bq, sc, 0);
+    load_a(2 * kt_lo, 0);
+    load_b(bq, sc, kt_lo);
     __syncthreads();  // the compiler waits for the LDS DMA (vmcnt) ahead of the barrier
 
-    for (int kt = 0; kt < kt_n; kt++) {
+    for (int kt = kt_lo; kt < kt_hi; kt++) {
 #pragma unroll
         for (int half = 0; half < 2; half++) {
             const int s = kt * 2 + half;
             // stage s+1 goes into the buffer that stage s-1 was read from: every wave is past the barrier that ended it
             if (s + 1 < stages) load_a(s + 1, (s + 1) & 1);
-            if (half == 0 && kt + 1 < kt_n) load_b(bqn, scn, kt + 1);
+            if (half == 0 && kt + 1 < kt_hi) load_b(bqn, scn, kt + 1);
             const _Float16* abuf = lds + (s & 1) * (PF_BM * PF_LDA) + a_row * PF_LDA;
 #pragma unroll
             for (int kbl = 0; kbl < 4; kbl++) {
@@ -147,7 +151,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
                         unit[ni] = s_cur;
                     }
                 }
-                if (G == 128 && kb == 0 && kt == 0) {  // the very first group: unit = its scale, accumulators are zero
+                if (G == 128 && kb == 0 && kt == kt_lo) {  // the very first group: unit = its scale, accumulators are zero
 #pragma unroll
                     for (int ni = 0; ni < 2; ni++) unit[ni] = w4_scale_fast<SBF>(sc[ni][0]);
                 }
@@ -158,7 +162,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
                 const bool last128 = G == 128 && kb == 7;  // branch free: the last k tile multiplies by 1
                 float next_ratio[2] = {1.f, 1.f};
                 if (last128) {
-                    const bool more = kt + 1 < kt_n;
+                    const bool more = kt + 1 < kt_hi;
 #pragma unroll
                     for (int ni = 0; ni < 2; ni++) {
                         const float s_next = more ? w4_scale_fast<SBF>(scn[ni][0]) : unit[ni];
@@ -194,6 +198,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     }
 
     // ---- epilogue: y[m][n] = acc * unit; D register e of lane (nl, khalf) is row 8*(e/4) + 4*khalf + e%4, column nl
+    if (gridDim.y > 1) y = reinterpret_cast<float*>(y) + (size_t)blockIdx.y * (size_t)t * (size_t)n;  // partial (f32)
 #pragma unroll
     for (int ni = 0; ni < 2; ni++) {
         const int col = n0 + wn * 64 + ni * 32 + nl;
@@ -218,9 +223,26 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
 #define PREFILL_KERNEL(NAME, G, SBF)                                                                               \
     extern "C" __global__ __launch_bounds__(PF_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void NAME(const u4_t* qt, const uint16_t* st, \
                                                                   const uint16_t* x, void* y, int row_blocks,      \
-                                                                  int k, int n, int t, int out_f16) {              \
-        prefill_body<G, SBF>(qt, st, x, y, row_blocks, k, n, t, out_f16);                                          \
+                                                                  int k, int n, int t, int out_f16, int sup_m,     \
+                                                                  int sup_n) {                                     \
+        prefill_body<G, SBF>(qt, st, x, y, row_blocks, k, n, t, out_f16, sup_m, sup_n);                            \
     }
+
+// y[i] = sum over the nks partials of a split-K launch, added in split order in f32; f32 or f16 out.
+extern "C" __global__ __launch_bounds__(256) void w4a16_prefill_splitk_sum(const float* __restrict__ part, void* __restrict__ y,
+                                                                           int nks, size_t count, int out_f16) {
+    const size_t n4 = count / 4;  // count = t*n with n % 4 == 0 is guaranteed by the host
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) {
+        f4_t a = reinterpret_cast<const f4_t*>(part)[i];
+        for (int ks = 1; ks < nks; ks++) a += reinterpret_cast<const f4_t*>(part + (size_t)ks * count)[i];
+        if (out_f16) {
+            h4_t v = {(_Float16)a[0], (_Float16)a[1], (_Float16)a[2], (_Float16)a[3]};
+            reinterpret_cast<h4_t*>(y)[i] = v;
+        } else {
+            reinterpret_cast<f4_t*>(y)[i] = a;
+        }
+    }
+}
 
 PREFILL_KERNEL(w4a16_prefill_g128_f16, 128, false)
 PREFILL_KERNEL(w4a16_prefill_g128_bf16, 128, true)

@@ -219,6 +219,9 @@ class W4a16Dec:
     def set_decode_shape(self, rows_per_wave=0, waves_per_block=0):
         ffi.check(self.cc.lib.w4a16_set_decode_shape(self.cc.h, rows_per_wave, waves_per_block))
 
+    def set_prefill_ksplit(self, ksplit=0):
+        ffi.check(self.cc.lib.w4a16_set_prefill_ksplit(self.cc.h, ksplit))
+
     def bench_forward(self, names, x_dev, y_dev, t, reps, warmup=1, out_f16=False, path=PATH_AUTO):
         """run_bench_gemv / run_bench_gemm (probes/w4a16/gpu/bench.rs:366-433): returns (ms by events, ms wall) for
         `reps` back-to-back launches rotating over `names`."""

@@ -247,6 +247,33 @@ def test_prefill_full_shapes_against_device_twin_and_sampled_oracle(dec, orc, n,
     say("   ", {a: m[a] for a in ("rel_l2", "max_ulp", "max_ulp_strict", "strict_pass_frac", "clamped")})
 
 
+@pytest.mark.parametrize("n,k,group,t,ksplit", [(512, 4096, 128, 100, 2), (512, 4096, 128, 100, 3), (512, 4096, 128, 100, 8),
+                                                (300, 2048, 32, 48, 4), (5120, 17408, 128, 512, 0)])
+def test_prefill_split_k(dec, orc, n, k, group, t, ksplit):
+    """Split-K (forced, or chosen automatically for the narrow down projection at t = 512): partial sums in f32 added
+    in slice order; same contract against the lane oracle, and close to the unsplit result."""
+    say("prefill split-k", n, k, group, t, ksplit)
+    q, s, x = gen.make_linear(n, k, group, t, seed=33)
+    dec.upload_lin_g("pks", q, s, n, k, group, False)
+    dec.set_prefill_ksplit(-1)
+    try:
+        whole = _device_forward(dec, "pks", x, t, ops.PATH_PREFILL)
+        dec.set_prefill_ksplit(ksplit)
+        got = _device_forward(dec, "pks", x, t, ops.PATH_PREFILL)
+        got16 = _device_forward(dec, "pks", x, t, ops.PATH_PREFILL, out_f16=True)
+    finally:
+        dec.set_prefill_ksplit(0)
+    assert np.array_equal(got16, gen.f32_to_f16_bits(got))
+    if n * t <= 1 << 18:
+        want = orc.gemm_lane(x, t, q, s, n, k, group, threads=16)
+    else:
+        want = _device_forward(dec, "pks", x, t, ops.PATH_LANE)  # the bit-exact device twin of the oracle
+    parity.assert_close(got, want, "split-k %d" % ksplit)
+    parity.assert_close(got, whole, "split-k %d vs unsplit" % ksplit)
+    if ksplit != 0:
+        assert not np.array_equal(_bits(got), _bits(whole))  # a different summation order: the split really happened
+
+
 def test_prefill_refuses_irregular_scales_and_auto_falls_back(dec, orc):
     n, k, group, t = 64, 256, 128, 40
     q, s, x = gen.make_linear(n, k, group, t, seed=9)
