@@ -87,11 +87,19 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     if (t * L.k * 2 >= 0x80000000ull || L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
         return w4_fail(W4A16_ERR_SHAPE, "prefill: x or the tiled weights reach 2 GiB, beyond the buffer-descriptor range");
     // block tile 128 (m) x 256 (n); 8 x 8 super-tiles dealt round-robin to the 8 XCDs (kernels/prefill.hip)
-    // Super-tile shape: up to 8 x 8, narrowed along n on small grids until there are at least two super-tiles per XCD.
+    // Super-tile shape: up to 8 tiles along m; along n the width in {8, 4, 2, 1} that leaves the busiest XCD with the
+    // fewest tiles (super-tiles are dealt round-robin to the 8 XCDs), the wider one on ties for L2 reuse.
     const size_t tiles_m = (t + 127) / 128, tiles_n = (L.n + 255) / 256;
     const size_t sup_m = std::min<size_t>(8, tiles_m), sm_n = (tiles_m + sup_m - 1) / sup_m;
-    const size_t sup_n = std::max<size_t>(1, std::min<size_t>(8, tiles_n * sm_n / 16));
-    const size_t supers = sm_n * ((tiles_n + sup_n - 1) / sup_n);
+    size_t sup_n = 8, supers = 0, best_load = ~(size_t)0;
+    for (size_t cand : {8, 4, 2, 1}) {
+        const size_t sp = sm_n * ((tiles_n + cand - 1) / cand), load = ((sp + 7) / 8) * sup_m * cand;
+        if (load < best_load) {
+            best_load = load;
+            sup_n = cand;
+            supers = sp;
+        }
+    }
     const size_t grid = ((supers + 7) / 8) * (sup_m * sup_n) * 8;
     // Split-K when the tile grid alone leaves much of the chip idle (two workgroups fit a CU: 512 slots): k slices are
     // doubled until the launch has at least 512 workgroups (measured best at the 27B down projection: 8 slices at
