@@ -136,6 +136,13 @@ enum {
 int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16,
                       int path);
 
+/* The gate|up projection of a dense FFN with the elementwise kernel that follows it folded in
+ * (gemv_multi_dev of the gate/up group + ew_dev_fused, w4a16_dec/chains.rs:271-287, assets/ew.cu:9-32):
+ * y[r][c] = f16(silu(g) * u), g = (W x)[r][c], u = (W x)[r][n/2 + c], f32 arithmetic, for a linear whose rows 0..n/2 are
+ * the gate and n/2..n the up projection (n % 32 == 0).  t <= 16 (decode regime); y_f16_dev: f16 [t][n/2].  Same values
+ * as w4a16_lin_forward (decode path, same launch shape) followed by w4a16_silu_mul_f16. */
+int w4a16_lin_forward_glu(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_f16_dev, size_t t);
+
 /* gemv_host (w4a16_dec/mod.rs, host-operand convenience used by probes): lin_forward with host x / y. */
 int w4a16_lin_forward_host(w4a16_ctx* ctx, const char* name, const uint16_t* x_f16, void* y, size_t t, int out_f16,
                            int path);

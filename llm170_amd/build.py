@@ -20,8 +20,10 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 # packed FP32 instructions are disabled for all device code
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
                 "-packed-fp32-ops", "-ffp-contract=off", "--genco", "--no-gpu-bundle-output"]
-# the matrix-core kernels may fuse their (not bit-exact) f32 scale-accumulate; the lane twin must not
-FUSED_OK = {"decode", "prefill", "moe", "util"}
+# No code object is built with floating-point contraction: the lane twin must keep its un-fused multiply and add, and
+# a library routine (expf) must expand identically in every code object so that fused epilogues give the bits of the
+# separate kernels.  Kernels that want a fused multiply-add write __builtin_fmaf.
+FUSED_OK = set()
 
 
 def kernel_sources():

@@ -58,6 +58,10 @@ static const char* const kDecodeSyms[] = {
     "w4a16_decode_g32_bf16_rb1_x1", "w4a16_decode_g32_bf16_rb1_x2", "w4a16_decode_g32_bf16_rb1_x4",
     "w4a16_decode_g32_bf16_rb2_x1", "w4a16_decode_g32_bf16_rb2_x2", "w4a16_decode_g32_bf16_rb2_x4",
     "w4a16_decode_g32_bf16_rb4_x1", "w4a16_decode_g32_bf16_rb4_x2", "w4a16_decode_g32_bf16_rb4_x4",
+    "w4a16_decode_g128_f16_glu_x1", "w4a16_decode_g128_f16_glu_x2", "w4a16_decode_g128_f16_glu_x4",
+    "w4a16_decode_g128_bf16_glu_x1", "w4a16_decode_g128_bf16_glu_x2", "w4a16_decode_g128_bf16_glu_x4",
+    "w4a16_decode_g32_f16_glu_x1", "w4a16_decode_g32_f16_glu_x2", "w4a16_decode_g32_f16_glu_x4",
+    "w4a16_decode_g32_bf16_glu_x1", "w4a16_decode_g32_bf16_glu_x2", "w4a16_decode_g32_bf16_glu_x4",
     nullptr};
 static const char* const kPrefillSyms[] = {"w4a16_prefill_g128_f16", "w4a16_prefill_g128_bf16", "w4a16_prefill_g32_f16",
                                            "w4a16_prefill_g32_bf16", "w4a16_prefill_splitk_sum", nullptr};

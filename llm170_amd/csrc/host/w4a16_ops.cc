@@ -79,6 +79,27 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     return w4_launch(ctx, sym, ceil_div(L.row_blocks, (size_t)rb), 1, (unsigned)(waves * 64), shmem, params);
 }
 
+// Fused gate|up projection with the SiLU*up epilogue (decode regime): y f16 [t][n/2].
+static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t) {
+    if (t == 0 || t > 16) return w4_fail(W4A16_ERR_SHAPE, "decode glu: t=%zu outside 1..16", t);
+    if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode glu: linear has no tiled copy (needs k %% 128 == 0)");
+    if (L.n % 32 != 0) return w4_fail(W4A16_ERR_SHAPE, "decode glu: n=%zu must be a multiple of 32 (gate and up halves of whole row blocks)", L.n);
+    if (L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
+        return w4_fail(W4A16_ERR_SHAPE, "decode: tiled weights of 2 GiB or more exceed the buffer-descriptor range");
+    const int kt_n = (int)(L.k / 128);
+    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : (t > 8 ? 4 : 8);
+    waves = std::max(1, std::min(std::min(waves, 8), kt_n));
+    const int xl = t <= 4 ? 1 : t <= 8 ? 2 : 4;
+    char sym[64];
+    snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_glu_x%d", L.group, L.scale_bf16 ? "bf16" : "f16", xl);
+    uint64_t qt = L.q_tiled, st = L.s_tiled;
+    int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = 1;
+    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of};
+    const unsigned slot = ((unsigned)(2 * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
+    const unsigned shmem = (unsigned)(waves * 2 * 1024) + (unsigned)waves * 2u * slot;
+    return w4_launch(ctx, sym, (unsigned)(L.row_blocks / 2), 1, (unsigned)(waves * 64), shmem, params);
+}
+
 // Prefill GEMM (kernels/prefill.hip).
 static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16) {
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has no tiled copy (needs k %% 128 == 0)");
@@ -312,6 +333,14 @@ extern "C" int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_de
         default:
             return w4_fail(W4A16_ERR_ARG, "lin_forward %s: unknown path %d", name, path);
     }
+}
+
+extern "C" int w4a16_lin_forward_glu(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_f16_dev, size_t t) {
+    W4Lin* L = nullptr;
+    W4_TRY(w4_find_lin(ctx, name, &L));
+    if (!x_dev || !y_f16_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_glu %s: null operand or t=0", name);
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t);
 }
 
 extern "C" int w4a16_lin_forward_host(w4a16_ctx* ctx, const char* name, const uint16_t* x_f16, void* y, size_t t,

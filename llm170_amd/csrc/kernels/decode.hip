@@ -41,7 +41,10 @@ __device__ __forceinline__ u4_t w4_row_shl(u4_t v) {
 }
 
 // XL = vector loads of x per k tile: 1 serves t <= 4, 2 serves t <= 8, 4 serves t <= 16.
-template <int G, bool SBF, int RB, int DEPTH, int XL>
+// GLU (RB = 2 only): the linear is a fused gate|up projection (rows 0..n/2 gate, n/2..n up); the wave owns gate row
+// block u and up row block u + n/32 and writes f16(silu(gate) * up) [t][n/2] instead of the two sums — the
+// elementwise kernel between the projections (assets/ew.cu:9-32) folded into the producer, same f32 arithmetic.
+template <int G, bool SBF, int RB, int DEPTH, int XL, bool GLU = false>
 __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                             const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
                                             int k, int n, int t, int out_f16) {
@@ -58,6 +61,8 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     const int kt_n = k / W4_TILE_K;
     const int kg_n = kt_n * GPT;
     const int nb0 = blockIdx.x * RB;
+    const int glu_half = row_blocks >> 1;  // GLU: row block of rb is blockIdx.x + rb * glu_half
+    auto row_block = [&](int rb) { return GLU ? (int)blockIdx.x + rb * glu_half : min(nb0 + rb, row_blocks - 1); };
     const int kt0 = (kt_n * wave) / W, kt1 = (kt_n * (wave + 1)) / W;
     const int m = lane & 15, g = lane >> 4;
 
@@ -73,7 +78,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
         acc[rb] = (f4_t){0.f, 0.f, 0.f, 0.f};
-        const unsigned nb = (unsigned)min(nb0 + rb, row_blocks - 1);  // a tail block re-reads the last row block
+        const unsigned nb = (unsigned)row_block(rb);  // a tail block re-reads the last row block
         qoff[rb] = nb * (unsigned)kt_n * 1024u + (unsigned)lane * 16u;
     }
     // scale fetch: byte o = lane*8 + a*512 of the round's slot belongs to row block o / (DEPTH*GPT*32); the rest of o
@@ -84,7 +89,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     for (int a = 0; a < AUXN; a++) {
         const int o = lane * 8 + a * 512;
         const int rb = o / (DEPTH * GPT * 32), rem = o % (DEPTH * GPT * 32);
-        const unsigned nb = (unsigned)min(nb0 + rb, row_blocks - 1);
+        const unsigned nb = (unsigned)row_block(rb);
         aoff[a] = o < AUXB ? nb * (unsigned)kg_n * 32u + (unsigned)rem : W4_OOB;
     }
     u2_t aux[AUXN];
@@ -139,7 +144,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                 const u2_t sv = *reinterpret_cast<const u2_t*>(sc + (rb * DEPTH + d) * GPT * 32);
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    acc[rb][i] += w4_scale_fast<SBF>((sv[i >> 1] >> (16 * (i & 1))) & 0xFFFFu) * part[i];
+                    acc[rb][i] = __builtin_fmaf(w4_scale_fast<SBF>((sv[i >> 1] >> (16 * (i & 1))) & 0xFFFFu), part[i], acc[rb][i]);
             } else {
 #pragma unroll
                 for (int w = 0; w < 4; w++) {
@@ -149,7 +154,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                     const u2_t sv = *reinterpret_cast<const u2_t*>(sc + ((rb * DEPTH + d) * GPT + w % GPT) * 32);
 #pragma unroll
                     for (int i = 0; i < 4; i++)
-                        acc[rb][i] += w4_scale_fast<SBF>((sv[i >> 1] >> (16 * (i & 1))) & 0xFFFFu) * part[i];
+                        acc[rb][i] = __builtin_fmaf(w4_scale_fast<SBF>((sv[i >> 1] >> (16 * (i & 1))) & 0xFFFFu), part[i], acc[rb][i]);
                 }
             }
         }
@@ -199,6 +204,19 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
         }
     }
     if (m >= t) return;
+    if (GLU) {
+        const int n_ff = n >> 1;
+        h4_t o;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float gt = acc[0][i], up = acc[RB - 1][i];
+            float v = (gt / (1.0f + expf(-gt))) * up;
+            asm volatile("" : "+v"(v));  // the product is rounded to f32 before the f16 conversion, as in the separate kernel
+            o[i] = (_Float16)v;
+        }
+        *reinterpret_cast<h4_t*>(reinterpret_cast<_Float16*>(y) + (size_t)m * n_ff + blockIdx.x * 16 + 4 * g) = o;
+        return;
+    }
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
         if (nb0 + rb >= row_blocks) break;
@@ -244,6 +262,12 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                                                         int k, int n, int t, int out_f16) {          \
         decode_body<G, SBF, RB, DECODE_DEPTH(BUDGET, G, RB, XL), XL>(qt, st, x, y, row_blocks, k, n, t, out_f16);    \
     }
+#define DECODE_GLU_KERNEL_X(NAME, G, SBF, XL, BUDGET, ATTR)                                                           \
+    extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
+                                                                        const uint16_t* x, void* y, int row_blocks,  \
+                                                                        int k, int n, int t, int out_f16) {          \
+        decode_body<G, SBF, 2, DECODE_DEPTH(BUDGET, G, 2, XL), XL, true>(qt, st, x, y, row_blocks, k, n, t, out_f16); \
+    }
 #define DECODE_HI __attribute__((amdgpu_waves_per_eu(6, 6)))
 #define DECODE_MID __attribute__((amdgpu_waves_per_eu(5, 5)))
 #define DECODE_LO
@@ -271,3 +295,14 @@ DECODE_KERNEL_LO3(w4a16_decode_g128_bf16_rb4, 128, true, 4)
 DECODE_KERNEL_LO3(w4a16_decode_g32_bf16_rb1, 32, true, 1)
 DECODE_KERNEL_LO3(w4a16_decode_g32_bf16_rb2, 32, true, 2)
 DECODE_KERNEL_LO3(w4a16_decode_g32_bf16_rb4, 32, true, 4)
+// fused gate|up with the SiLU*up epilogue (two row blocks per wave by construction)
+#define DECODE_GLU_G128(NAME, SBF)                                                                     \
+    DECODE_GLU_KERNEL_X(NAME, 128, SBF, 1, 24, DECODE_HI) DECODE_GLU_KERNEL_X(NAME, 128, SBF, 2, 24, DECODE_MID) \
+    DECODE_GLU_KERNEL_X(NAME, 128, SBF, 4, 64, DECODE_LO)
+#define DECODE_GLU_G32(NAME, SBF)                                                                    \
+    DECODE_GLU_KERNEL_X(NAME, 32, SBF, 1, 64, DECODE_LO) DECODE_GLU_KERNEL_X(NAME, 32, SBF, 2, 64, DECODE_LO) \
+    DECODE_GLU_KERNEL_X(NAME, 32, SBF, 4, 64, DECODE_LO)
+DECODE_GLU_G128(w4a16_decode_g128_f16_glu, false)
+DECODE_GLU_G128(w4a16_decode_g128_bf16_glu, true)
+DECODE_GLU_G32(w4a16_decode_g32_f16_glu, false)
+DECODE_GLU_G32(w4a16_decode_g32_bf16_glu, true)

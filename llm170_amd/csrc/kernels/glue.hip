@@ -23,6 +23,7 @@ extern "C" __global__ __launch_bounds__(RMS_LANES) void w4a16_rms_rescale_f16(co
     const int tid = threadIdx.x;
     const float* row = v + (size_t)blockIdx.x * ld;
     double ss = 0.0;
+    float first[RMS_UNROLL];  // the row's first RMS_LANES * RMS_UNROLL columns stay in registers for the second pass
     for (int c0 = tid; c0 < ncols; c0 += RMS_LANES * RMS_UNROLL) {
         float x[RMS_UNROLL];
 #pragma unroll
@@ -34,6 +35,7 @@ extern "C" __global__ __launch_bounds__(RMS_LANES) void w4a16_rms_rescale_f16(co
         for (int j = 0; j < RMS_UNROLL; j++) {
             const double d = (double)x[j];
             ss = ss + d * d;  // a zero past the row end adds +0.0 and changes nothing
+            if (c0 == tid) first[j] = x[j];
         }
     }
     red[tid] = ss;
@@ -49,7 +51,12 @@ extern "C" __global__ __launch_bounds__(RMS_LANES) void w4a16_rms_rescale_f16(co
     r = __shfl(r, 0);
     const float inv = (float)(1.0 / sqrt(r / (double)ncols + 1e-6));
     _Float16* o = reinterpret_cast<_Float16*>(out) + (size_t)blockIdx.x * ncols;
-    for (int c = tid; c < ncols; c += RMS_LANES) o[c] = glue_round_f16(row[c] * inv);
+#pragma unroll
+    for (int j = 0; j < RMS_UNROLL; j++) {
+        const int c = tid + j * RMS_LANES;
+        if (c < ncols) o[c] = glue_round_f16(first[j] * inv);
+    }
+    for (int c = tid + RMS_LANES * RMS_UNROLL; c < ncols; c += RMS_LANES) o[c] = glue_round_f16(row[c] * inv);
 }
 
 // out[r][c] = f16((g / (1 + exp(-g))) * u),  g = gu[r][c], u = gu[r][n_ff + c], all in f32 (assets/ew.cu:19-30).

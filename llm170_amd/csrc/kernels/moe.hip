@@ -199,16 +199,16 @@ __device__ __forceinline__ void moe_dec_body(MOE_PARAMS) {
                 for (int w = 0; w < 4; w++)
                     part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
                                                                   __builtin_bit_cast(h8_t, xb[w]), part, 0, 0, 0);
-                acc[rb] += moe_scale4<G, SBF, 0>(s_.s[rb]) * part;
+                acc[rb] = w4_fma4(moe_scale4<G, SBF, 0>(s_.s[rb]), part, acc[rb]);
             } else {
                 f4_t p0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][0]), __builtin_bit_cast(h8_t, xb[0]), zero, 0, 0, 0);
                 f4_t p1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][1]), __builtin_bit_cast(h8_t, xb[1]), zero, 0, 0, 0);
                 f4_t p2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][2]), __builtin_bit_cast(h8_t, xb[2]), zero, 0, 0, 0);
                 f4_t p3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][3]), __builtin_bit_cast(h8_t, xb[3]), zero, 0, 0, 0);
-                acc[rb] += moe_scale4<G, SBF, 0>(s_.s[rb]) * p0;
-                acc[rb] += moe_scale4<G, SBF, 1>(s_.s[rb]) * p1;
-                acc[rb] += moe_scale4<G, SBF, 2>(s_.s[rb]) * p2;
-                acc[rb] += moe_scale4<G, SBF, 3>(s_.s[rb]) * p3;
+                acc[rb] = w4_fma4(moe_scale4<G, SBF, 0>(s_.s[rb]), p0, acc[rb]);
+                acc[rb] = w4_fma4(moe_scale4<G, SBF, 1>(s_.s[rb]), p1, acc[rb]);
+                acc[rb] = w4_fma4(moe_scale4<G, SBF, 2>(s_.s[rb]), p2, acc[rb]);
+                acc[rb] = w4_fma4(moe_scale4<G, SBF, 3>(s_.s[rb]), p3, acc[rb]);
             }
         }
     };
@@ -316,16 +316,16 @@ __device__ __forceinline__ void moe_down_sum_body(const char* __restrict__ qa, c
                 for (int w = 0; w < 4; w++)
                     part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
                                                                   __builtin_bit_cast(h8_t, xb[w]), part, 0, 0, 0);
-                acc[rb] += moe_scale4<G, SBF, 0>(s_.s[rb]) * part;
+                acc[rb] = w4_fma4(moe_scale4<G, SBF, 0>(s_.s[rb]), part, acc[rb]);
             } else {
                 f4_t p0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][0]), __builtin_bit_cast(h8_t, xb[0]), zero, 0, 0, 0);
                 f4_t p1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][1]), __builtin_bit_cast(h8_t, xb[1]), zero, 0, 0, 0);
                 f4_t p2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][2]), __builtin_bit_cast(h8_t, xb[2]), zero, 0, 0, 0);
                 f4_t p3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][3]), __builtin_bit_cast(h8_t, xb[3]), zero, 0, 0, 0);
-                acc[rb] += moe_scale4<G, SBF, 0>(s_.s[rb]) * p0;
-                acc[rb] += moe_scale4<G, SBF, 1>(s_.s[rb]) * p1;
-                acc[rb] += moe_scale4<G, SBF, 2>(s_.s[rb]) * p2;
-                acc[rb] += moe_scale4<G, SBF, 3>(s_.s[rb]) * p3;
+                acc[rb] = w4_fma4(moe_scale4<G, SBF, 0>(s_.s[rb]), p0, acc[rb]);
+                acc[rb] = w4_fma4(moe_scale4<G, SBF, 1>(s_.s[rb]), p1, acc[rb]);
+                acc[rb] = w4_fma4(moe_scale4<G, SBF, 2>(s_.s[rb]), p2, acc[rb]);
+                acc[rb] = w4_fma4(moe_scale4<G, SBF, 3>(s_.s[rb]), p3, acc[rb]);
             }
         }
     };
@@ -484,7 +484,7 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
                     const f4_t sc = moe_scale4<G, SBF, w>(s_.s[rb]);
 #pragma unroll
                     for (int tt = 0; tt < TT; tt++)
-                        acc[rb][tt] += sc * __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], zero, 0, 0, 0);
+                        acc[rb][tt] = w4_fma4(sc, __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], zero, 0, 0, 0), acc[rb][tt]);
                 } else {
 #pragma unroll
                     for (int tt = 0; tt < TT; tt++)
@@ -501,7 +501,7 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
             for (int rb = 0; rb < 2; rb++) {
                 const f4_t sc = moe_scale4<G, SBF, 0>(s_.s[rb]);
 #pragma unroll
-                for (int tt = 0; tt < TT; tt++) acc[rb][tt] += sc * part[rb][tt];
+                for (int tt = 0; tt < TT; tt++) acc[rb][tt] = w4_fma4(sc, part[rb][tt], acc[rb][tt]);
             }
         }
     };

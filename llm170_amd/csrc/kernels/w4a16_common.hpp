@@ -97,3 +97,13 @@ __device__ __forceinline__ float w4_scale_fast(unsigned bits16) {
     if (SBF) return __builtin_bit_cast(float, bits16 << 16);
     return (float)__builtin_bit_cast(_Float16, (unsigned short)bits16);
 }
+
+// c + a * b as one fused multiply-add per element.  Written out because the kernels are compiled without floating-point
+// contraction (a library routine such as expf must expand to the same instructions in every code object, so that a
+// fused epilogue gives the bits of the separate kernel).
+__device__ __forceinline__ f4_t w4_fma4(f4_t a, f4_t b, f4_t c) {
+    f4_t r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = __builtin_fmaf(a[i], b[i], c[i]);
+    return r;
+}

@@ -185,6 +185,10 @@ class W4a16Dec:
     def lin_forward(self, name, x_dev, dst_dev, t, out_f16=False, path=PATH_AUTO):
         ffi.check(self.cc.lib.w4a16_lin_forward(self.cc.h, name.encode(), x_dev, dst_dev, t, int(out_f16), path))
 
+    def lin_forward_glu(self, name, x_dev, y_f16_dev, t):
+        """Fused gate|up projection with the SiLU*up epilogue: y f16 [t][n/2]."""
+        ffi.check(self.cc.lib.w4a16_lin_forward_glu(self.cc.h, name.encode(), x_dev, y_f16_dev, t))
+
     def gemv_host(self, name, x, t=1, out_f16=False, path=PATH_AUTO):
         """Host operands in, host result out: y [t][n] (f32, or f16 bit patterns when out_f16)."""
         spec = self.lin_spec(name)

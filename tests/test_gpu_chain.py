@@ -72,6 +72,49 @@ def test_silu_mul_close(dec, orc, t, n_ff):
     assert np.mean(got == want) > 0.995
 
 
+# ------------------------------------------------------------------ gate|up with the SiLU*up epilogue
+@pytest.mark.parametrize("n,k,group,bf16", [(1024, 256, 128, False), (2048, 512, 32, False), (1024, 256, 128, True),
+                                            (34816, 5120, 128, False)])
+@pytest.mark.parametrize("t", [1, 3, 4, 7, 16])
+def test_fused_glu_equals_linear_then_silu_mul(dec, orc, n, k, group, bf16, t):
+    """The fused kernel gives the bits of the two-launch sequence at the same launch shape, and both stay within one
+    f16 step of the oracle's silu_mul of the lane GEMM."""
+    if n > 4096 and t not in (1, 4):
+        pytest.skip("layer shape: t = 1 and 4 only")
+    q, s, x = gen.make_linear(n, k, group, t, seed=71)
+    if bf16:
+        s = (gen.f16_bits_to_f32(s).view(np.uint32) >> 16).astype(np.uint16)
+    dec.upload_lin_g("glu", q, s, n, k, group, bf16)
+    cc = dec.cc
+    px, pg, pa, pb = cc.to_device(x), cc.alloc(t * n * 4), cc.alloc(t * (n // 2) * 2), cc.alloc(t * (n // 2) * 2)
+    dec.set_decode_shape(32, 8 if t <= 8 else 4)  # the shape the fused kernel always uses
+    try:
+        dec.lin_forward("glu", px, pg, t, path=ops.PATH_DECODE)
+    finally:
+        dec.set_decode_shape(0, 0)
+    dec.silu_mul_f16(pg, n // 2, t, pa)
+    dec.lin_forward_glu("glu", px, pb, t)
+    two, one = cc.d2h(pa, (t, n // 2), np.uint16), cc.d2h(pb, (t, n // 2), np.uint16)
+    for p in (px, pg, pa, pb):
+        cc.free(p)
+    assert np.array_equal(one, two)
+    if n <= 4096:
+        want = orc.silu_mul_f16_rows(orc.gemm_lane(x, t, q, s, n, k, group, bf16, 8))
+        a, b = _f16(one).astype(np.float64), _f16(want).astype(np.float64)
+        rms = float(np.sqrt(np.mean(b * b)))
+        assert np.all(np.abs(a - b) <= 2 * parity.f16_ulp(np.maximum(np.abs(b), rms / 128)))
+        assert np.mean(one == want) > 0.97
+
+
+def test_fused_glu_errors(dec):
+    dec.upload_lin_synth("glu_odd", 48, 256, 128, 1, 2)  # n = 48: halves are not whole row blocks
+    with pytest.raises(ops.W4a16Error):
+        dec.lin_forward_glu("glu_odd", 1, 1, 1)
+    dec.upload_lin_synth("glu_ok", 64, 256, 128, 1, 2)
+    with pytest.raises(ops.W4a16Error):
+        dec.lin_forward_glu("glu_ok", 1, 1, 17)
+
+
 # ------------------------------------------------------------------ the chain
 def _host_lins(seeds, prefix, layer, shapes, group):
     out = []
