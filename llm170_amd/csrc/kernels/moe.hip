@@ -432,18 +432,20 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
         xg_off[p] = slot < ns ? ((unsigned)(slot / x_div) * (unsigned)k + (unsigned)(tid & 15) * 8u) * 2u : W4_OOB;
         xl_off[p] = row < ROWS ? row * MOE_LDX + (tid & 15) * 8 : -1;
     }
-    u4_t xreg[TT];
-    auto load_x = [&](int kt) {
+    // x tiles travel global -> registers -> LDS two k tiles ahead of their use (two register sets): the gathered rows
+    // come from L2 with a latency longer than one k tile of compute
+    u4_t xreg[2][TT];
+    auto load_x = [&](int set, int kt) {
 #pragma unroll
         for (int p = 0; p < TT; p++)
-            xreg[p] = __builtin_amdgcn_raw_buffer_load_b128(
+            xreg[set][p] = __builtin_amdgcn_raw_buffer_load_b128(
                 xr, (kt < kt_n && xg_off[p] != W4_OOB) ? xg_off[p] + (unsigned)kt * (W4_TILE_K * 2u) : W4_OOB, 0, 0);
     };
-    auto store_x = [&](int buf) {
+    auto store_x = [&](int set, int buf) {
         _Float16* base = xs + buf * (ROWS * MOE_LDX);
 #pragma unroll
         for (int p = 0; p < TT; p++)
-            if (xl_off[p] >= 0) *reinterpret_cast<u4_t*>(base + xl_off[p]) = xreg[p];
+            if (xl_off[p] >= 0) *reinterpret_cast<u4_t*>(base + xl_off[p]) = xreg[set][p];
     };
 
     const unsigned qoff[2] = {(unsigned)rbA * (unsigned)kt_n * 1024u + (unsigned)lane * 16u,
@@ -506,20 +508,21 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
         }
     };
 
-    // prologue: x tile 0 into LDS buffer 0, DEPTH weight stages in flight
-    load_x(0);
+    // prologue: x tile 0 into LDS buffer 0, x tile 1 in registers, DEPTH weight stages in flight
+    load_x(0, 0);
+    load_x(1, 1);
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) load_w(stage[d], d);
-    store_x(0);
+    store_x(0, 0);
     __syncthreads();
     for (int kt0 = 0; kt0 < kt_n; kt0 += DEPTH) {
 #pragma unroll
-        for (int d = 0; d < DEPTH; d++) {
+        for (int d = 0; d < DEPTH; d++) {  // DEPTH is even: register set and LDS buffer of tile kt are kt & 1 = d & 1
             const int kt = kt0 + d;
-            load_x(kt + 1);  // out of range past the last tile: zeros, no traffic
             if (kt < kt_n) compute(stage[d], d & 1);
             load_w(stage[d], kt + DEPTH);
-            store_x((d + 1) & 1);
+            store_x((d + 1) & 1, (d + 1) & 1);  // tile kt+1, loaded an iteration ago, into the buffer tile kt-1 was read from
+            load_x(d & 1, kt + 2);              // out of range past the last tile: zeros, no traffic
             __syncthreads();
         }
     }
