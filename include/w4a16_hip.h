@@ -159,6 +159,11 @@ int w4a16_lin_untile(w4a16_ctx* ctx, const char* name, uint64_t q_out_dev, uint6
  * waves_per_block in 1..8.  For tuning sweeps (the reference exposes its split-K factor the same way,
  * sk_ksp, w4a16_dec/kernels/decode.rs:3-16). */
 int w4a16_set_decode_shape(w4a16_ctx* ctx, int rows_per_wave, int waves_per_block);
+/* Split-K across workgroups for the decode kernel: 0 = automatic (outputs too narrow to give every CU several equal
+ * shares of row blocks), -1 = never, 1..8 = exactly that many k slices (clamped to two k tiles per slice).  Still one
+ * launch: the workgroup that finishes last adds the slices in slice order.  Counterpart of the reference's split-K
+ * factor for its decode GEMV (sk_ksp, w4a16_dec/kernels/decode.rs:3-16, 59-127). */
+int w4a16_set_decode_ksplit(w4a16_ctx* ctx, int ksplit);
 
 /* Split-K override for the prefill kernel: 0 = automatic (split when the tile grid alone would leave most of the chip
  * idle — narrow outputs at moderate t; the reference's prefill path makes the same choice inside its vendored GEMM),

@@ -67,6 +67,9 @@ struct w4a16_ctx {
     W4ChainScratch chain;
     int moe_block = 0, moe_waves = 0;  // 0 = automatic
     int decode_rows_per_wave = 0, decode_waves_per_block = 0;  // 0 = automatic
+    int decode_ksplit = 0;                                      // 0 = automatic, -1 = never, n = exactly n k slices
+    uint64_t decode_ws = 0, decode_tickets = 0;                 // partial tiles and per-block tickets of a split launch
+    size_t decode_ws_cap = 0, decode_tickets_cap = 0;
     int prefill_ksplit = 0;                                     // 0 = automatic, -1 = never, n = exactly n slices
     uint64_t prefill_ws = 0;                                    // f32 partials of a split-K prefill launch
     size_t prefill_ws_cap = 0;

@@ -58,6 +58,33 @@ static int pick_decode_shape(const w4a16_ctx* ctx, const W4Lin& L, size_t t, int
     return 0;
 }
 
+// k slices across workgroups for a decode launch of `blocks` workgroups, and the workspace they need.  The tickets are
+// zeroed when (re)allocated; every launch leaves them zero.
+static int decode_split(w4a16_ctx* ctx, const W4Lin& L, size_t t, size_t blocks, int rb, int* waves, int* nks_out) {
+    const int kt_n = (int)(L.k / 128);
+    int nks = 1;
+    if (ctx->decode_ksplit > 0) {
+        nks = ctx->decode_ksplit;
+    } else if (ctx->decode_ksplit == 0 && t <= 8 && blocks < (size_t)std::max(ctx->cu_count, 1) && kt_n >= 64) {
+        // a long k range over fewer workgroups than CUs (the 27B down projection: 160 blocks x 136 k tiles): slices
+        // of about 16 k tiles, four waves each (measured 12.4 -> 11.8 us at t = 1, 13.3 -> 12.4 us at t = 4).  Shorter
+        // k ranges lose more to the extra workgroups than they gain.
+        nks = std::min(8, kt_n / 16);
+        *waves = std::min(*waves, 4);
+    }
+    nks = std::max(1, std::min(nks, kt_n / 2));
+    if (nks > 1) {
+        *waves = std::max(1, std::min(*waves, kt_n / nks));
+        W4_TRY(w4_ensure(ctx, &ctx->decode_ws, &ctx->decode_ws_cap, blocks * (size_t)rb * 1024 * (size_t)nks));
+        if (blocks * 4 > ctx->decode_tickets_cap) {
+            W4_TRY(w4_ensure(ctx, &ctx->decode_tickets, &ctx->decode_tickets_cap, std::max<size_t>(blocks * 4, 16384)));
+            W4_TRY(w4a16_memset0(ctx, ctx->decode_tickets, ctx->decode_tickets_cap));
+        }
+    }
+    *nks_out = nks;
+    return 0;
+}
+
 static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16) {
     if (t == 0 || t > 16) return w4_fail(W4A16_ERR_SHAPE, "decode: t=%zu outside 1..16", t);
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode: linear has no tiled copy (needs k %% 128 == 0)");
@@ -71,12 +98,16 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_rb%d_x%d", L.group, L.scale_bf16 ? "bf16" : "f16", rb, xl);
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
-    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of};
+    const size_t blocks = ceil_div(L.row_blocks, (size_t)rb);
+    int nks = 1;
+    W4_TRY(decode_split(ctx, L, t, blocks, rb, &waves, &nks));
+    uint64_t ws = ctx->decode_ws, tk = ctx->decode_tickets;
+    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk};
     // LDS: the split-K partial tiles [waves][rb][1 KiB], then two scale slots per wave; a slot holds the scales of
     // one ring round (rb x depth x groups-per-tile x 32 bytes, ring never deeper than 8 tiles) rounded up to 512
     const unsigned slot = ((unsigned)(rb * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
     const unsigned shmem = (unsigned)(waves * rb * 1024) + (unsigned)waves * 2u * slot;
-    return w4_launch(ctx, sym, ceil_div(L.row_blocks, (size_t)rb), 1, (unsigned)(waves * 64), shmem, params);
+    return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);
 }
 
 // Fused gate|up projection with the SiLU*up epilogue (decode regime): y f16 [t][n/2].
@@ -94,10 +125,14 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
     snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_glu_x%d", L.group, L.scale_bf16 ? "bf16" : "f16", xl);
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = 1;
-    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of};
+    const size_t blocks = L.row_blocks / 2;
+    int nks = 1;
+    W4_TRY(decode_split(ctx, L, t, blocks, 2, &waves, &nks));
+    uint64_t ws = ctx->decode_ws, tk = ctx->decode_tickets;
+    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk};
     const unsigned slot = ((unsigned)(2 * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
     const unsigned shmem = (unsigned)(waves * 2 * 1024) + (unsigned)waves * 2u * slot;
-    return w4_launch(ctx, sym, (unsigned)(L.row_blocks / 2), 1, (unsigned)(waves * 64), shmem, params);
+    return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);
 }
 
 // Prefill GEMM (kernels/prefill.hip).
@@ -407,6 +442,13 @@ extern "C" int w4a16_set_decode_shape(w4a16_ctx* ctx, int rows_per_wave, int wav
         return w4_fail(W4A16_ERR_ARG, "set_decode_shape: rows_per_wave in {0,16,32,64}, waves_per_block in 0..8");
     ctx->decode_rows_per_wave = rows_per_wave;
     ctx->decode_waves_per_block = waves_per_block;
+    return 0;
+}
+
+extern "C" int w4a16_set_decode_ksplit(w4a16_ctx* ctx, int ksplit) {
+    if (!ctx) return w4_fail(W4A16_ERR_ARG, "set_decode_ksplit: null context");
+    if (ksplit < -1 || ksplit > 8) return w4_fail(W4A16_ERR_ARG, "set_decode_ksplit: -1 = never, 0 = automatic, 1..8 slices");
+    ctx->decode_ksplit = ksplit;
     return 0;
 }
 

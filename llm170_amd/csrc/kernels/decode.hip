@@ -21,8 +21,14 @@
 //     operations of one wave execute in order) and each MFMA group reads its four scales back with ds_read_b64;
 //   * split-K lives inside the workgroup: the W waves of a block take consecutive k-tile slices of the same RB row
 //     blocks and wave 0 folds the partial tiles through LDS in fixed order (deterministic, no atomics, no second
-//     launch).  The host picks RB and W.
+//     launch).  The host picks RB and W;
+//   * an output too narrow to give every CU its share of row blocks is also split over k across workgroups
+//     (gridDim.y slices): each block parks its partial tile in a workspace and takes a ticket; the block that draws the
+//     last ticket of its row blocks adds the slices in slice order (whoever is last: deterministic) and runs the
+//     epilogue.  Still one launch, no atomics on data.
 #include "w4a16_common.hpp"
+
+#define W4_DECODE_MAX_KSPLIT 8  // k slices across workgroups; the host clamps to this
 
 // One pipeline stage = the loads of one k tile: RB weight tiles, their scales, and XL loads of x.
 template <int RB, int XL>
@@ -47,7 +53,7 @@ __device__ __forceinline__ u4_t w4_row_shl(u4_t v) {
 template <int G, bool SBF, int RB, int DEPTH, int XL, bool GLU = false>
 __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                             const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
-                                            int k, int n, int t, int out_f16) {
+                                            int k, int n, int t, int out_f16, f4_t* ws, int* tickets) {
     extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K, then [W][2][AUXB] scale slots
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
     constexpr int AUXB = RB * DEPTH * GPT * 32;      // bytes of scales one ring round needs: [rb][tile][group][16 rows]
@@ -63,7 +69,9 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     const int nb0 = blockIdx.x * RB;
     const int glu_half = row_blocks >> 1;  // GLU: row block of rb is blockIdx.x + rb * glu_half
     auto row_block = [&](int rb) { return GLU ? (int)blockIdx.x + rb * glu_half : min(nb0 + rb, row_blocks - 1); };
-    const int kt0 = (kt_n * wave) / W, kt1 = (kt_n * (wave + 1)) / W;
+    const int nks = gridDim.y, ky = blockIdx.y;  // k slices across workgroups
+    const int kt_lo = (kt_n * ky) / nks, kt_span = (kt_n * (ky + 1)) / nks - kt_lo;
+    const int kt0 = kt_lo + (kt_span * wave) / W, kt1 = kt_lo + (kt_span * (wave + 1)) / W;
     const int m = lane & 15, g = lane >> 4;
 
     // Every load is a raw buffer load: an out-of-range offset returns zeros and costs no memory traffic, which
@@ -203,6 +211,37 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
             for (int rb = 0; rb < RB; rb++) acc[rb] += red[(w * RB + rb) * 64 + lane];
         }
     }
+    if (nks > 1) {  // wave 0 only from here
+        // Partial tiles and tickets travel as device-scope accesses (write-through stores, cache-bypassing loads), so
+        // no cache write-back or invalidate is needed: a device-scope release fence writes back the whole L2 of the
+        // XCD and costs more per workgroup than the slice itself.
+        const __amdgpu_buffer_rsrc_t wr = w4_make_rsrc(ws, (unsigned)gridDim.x * (unsigned)nks * (RB * 1024u));
+        const unsigned mine = ((unsigned)blockIdx.x * RB * 64u + (unsigned)lane) * 16u;
+        const unsigned slice = (unsigned)gridDim.x * (RB * 1024u);  // bytes per k slice
+        constexpr int DEV = 16;                                     // cache policy: device scope (sc1)
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, acc[rb]), wr, mine + rb * 1024u, ky * slice, DEV);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores have reached memory before the ticket is drawn
+        int ticket = 0;
+        if (lane == 0) ticket = __hip_atomic_fetch_add(tickets + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ticket = __builtin_amdgcn_readfirstlane(ticket);
+        if (ticket != nks - 1) return;
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+            f4_t part[W4_DECODE_MAX_KSPLIT];
+#pragma unroll
+            for (int s_ = 0; s_ < W4_DECODE_MAX_KSPLIT; s_++)  // slices past nks: zero-length descriptor, zeros, no traffic
+                part[s_] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                                        s_ < nks ? wr : w4_make_rsrc(ws, 0u), mine + rb * 1024u, s_ * slice, DEV));
+            f4_t sum = part[0];
+#pragma unroll
+            for (int s_ = 1; s_ < W4_DECODE_MAX_KSPLIT; s_++) sum += part[s_];
+            acc[rb] = sum;
+        }
+        if (lane == 0) __hip_atomic_store(tickets + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    }
     if (m >= t) return;
     if (GLU) {
         const int n_ff = n >> 1;
@@ -259,14 +298,18 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
 #define DECODE_KERNEL_X(NAME, G, SBF, RB, XL, BUDGET, ATTR)                                                          \
     extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
                                                                         const uint16_t* x, void* y, int row_blocks,  \
-                                                                        int k, int n, int t, int out_f16) {          \
-        decode_body<G, SBF, RB, DECODE_DEPTH(BUDGET, G, RB, XL), XL>(qt, st, x, y, row_blocks, k, n, t, out_f16);    \
+                                                                        int k, int n, int t, int out_f16, f4_t* ws,  \
+                                                                        int* tickets) {                              \
+        decode_body<G, SBF, RB, DECODE_DEPTH(BUDGET, G, RB, XL), XL>(qt, st, x, y, row_blocks, k, n, t, out_f16, ws, \
+                                                                     tickets);                                       \
     }
 #define DECODE_GLU_KERNEL_X(NAME, G, SBF, XL, BUDGET, ATTR)                                                           \
     extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
                                                                         const uint16_t* x, void* y, int row_blocks,  \
-                                                                        int k, int n, int t, int out_f16) {          \
-        decode_body<G, SBF, 2, DECODE_DEPTH(BUDGET, G, 2, XL), XL, true>(qt, st, x, y, row_blocks, k, n, t, out_f16); \
+                                                                        int k, int n, int t, int out_f16, f4_t* ws,  \
+                                                                        int* tickets) {                              \
+        decode_body<G, SBF, 2, DECODE_DEPTH(BUDGET, G, 2, XL), XL, true>(qt, st, x, y, row_blocks, k, n, t, out_f16,  \
+                                                                         ws, tickets);                               \
     }
 #define DECODE_HI __attribute__((amdgpu_waves_per_eu(6, 6)))
 #define DECODE_MID __attribute__((amdgpu_waves_per_eu(5, 5)))

@@ -481,12 +481,21 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
             for (int tt = 0; tt < TT; tt++) b[tt] = *reinterpret_cast<const h8_t*>(xb + tt * 16 * MOE_LDX + w * 32);
 #pragma unroll
             for (int rb = 0; rb < 2; rb++) {
-                const h8_t a = w4_deq8(s_.q[rb][w]);
+                // G = 32: every 32-k group's products are scaled on their own, and left alone the compiler issues all 8 * TT
+                // MFMAs of a k tile into separate result registers before the first scaled sum (220 VGPRs at TT = 3,
+                // two waves per SIMD).  The empty asm statements pin the order group by group: this group's unpack
+                // starts after the previous group's sums, so one group's results are live at a time (<= 128 VGPRs, four
+                // waves per SIMD, which hide the MFMA -> VALU latency this ordering exposes).
+                unsigned qw = s_.q[rb][w];
+                if (G == 32) asm volatile("" : "+v"(qw));
+                const h8_t a = w4_deq8(qw);
                 if (G == 32) {
                     const f4_t sc = moe_scale4<G, SBF, w>(s_.s[rb]);
 #pragma unroll
                     for (int tt = 0; tt < TT; tt++)
                         acc[rb][tt] = w4_fma4(sc, __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], zero, 0, 0, 0), acc[rb][tt]);
+#pragma unroll
+                    for (int tt = 0; tt < TT; tt++) asm volatile("" : "+v"(acc[rb][tt]));
                 } else {
 #pragma unroll
                     for (int tt = 0; tt < TT; tt++)
@@ -545,24 +554,24 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     extern "C" __global__ __launch_bounds__(512) void NAME(MOE_PARAMS) {              \
         moe_mm_body<G, SBF, GLU, TT, DEPTH>(MOE_ARGS);                                \
     }
-#define MOE_FAMILY(PFX, G, SBF)                              \
+#define MOE_FAMILY(PFX, G, SBF, DMM)                             \
     MOE_DEC_KERNEL(PFX##_dec_glu_x1, G, SBF, true, 1, 4)     \
     MOE_DEC_KERNEL(PFX##_dec_glu_x4, G, SBF, true, 4, 3)     \
     MOE_DEC_KERNEL(PFX##_dec_lin_x1, G, SBF, false, 1, 4)    \
     MOE_DEC_KERNEL(PFX##_dec_lin_x4, G, SBF, false, 4, 3)    \
-    MOE_MM_KERNEL(PFX##_mm_glu_t1, G, SBF, true, 1, 4)       \
-    MOE_MM_KERNEL(PFX##_mm_glu_t2, G, SBF, true, 2, 4)       \
-    MOE_MM_KERNEL(PFX##_mm_glu_t3, G, SBF, true, 3, 4)       \
-    MOE_MM_KERNEL(PFX##_mm_glu_t4, G, SBF, true, 4, 4)       \
-    MOE_MM_KERNEL(PFX##_mm_lin_t1, G, SBF, false, 1, 4)      \
-    MOE_MM_KERNEL(PFX##_mm_lin_t2, G, SBF, false, 2, 4)      \
-    MOE_MM_KERNEL(PFX##_mm_lin_t3, G, SBF, false, 3, 4)      \
-    MOE_MM_KERNEL(PFX##_mm_lin_t4, G, SBF, false, 4, 4)
+    MOE_MM_KERNEL(PFX##_mm_glu_t1, G, SBF, true, 1, DMM)       \
+    MOE_MM_KERNEL(PFX##_mm_glu_t2, G, SBF, true, 2, DMM)       \
+    MOE_MM_KERNEL(PFX##_mm_glu_t3, G, SBF, true, 3, DMM)       \
+    MOE_MM_KERNEL(PFX##_mm_glu_t4, G, SBF, true, 4, DMM)       \
+    MOE_MM_KERNEL(PFX##_mm_lin_t1, G, SBF, false, 1, DMM)      \
+    MOE_MM_KERNEL(PFX##_mm_lin_t2, G, SBF, false, 2, DMM)      \
+    MOE_MM_KERNEL(PFX##_mm_lin_t3, G, SBF, false, 3, DMM)      \
+    MOE_MM_KERNEL(PFX##_mm_lin_t4, G, SBF, false, 4, DMM)
 
-MOE_FAMILY(w4a16_moe_g32_f16, 32, false)
-MOE_FAMILY(w4a16_moe_g32_bf16, 32, true)
-MOE_FAMILY(w4a16_moe_g128_f16, 128, false)
-MOE_FAMILY(w4a16_moe_g128_bf16, 128, true)
+MOE_FAMILY(w4a16_moe_g32_f16, 32, false, 2)
+MOE_FAMILY(w4a16_moe_g32_bf16, 32, true, 2)
+MOE_FAMILY(w4a16_moe_g128_f16, 128, false, 4)
+MOE_FAMILY(w4a16_moe_g128_bf16, 128, true, 4)
 
 // ---------------------------------------------------------------------------------------------------- routing
 // Softmax over all experts, k largest probabilities with ties to the lower index, weights renormalised by the
@@ -721,15 +730,20 @@ extern "C" __global__ __launch_bounds__(512) void w4a16_moe_align(const int* __r
     // placement in slot order: every wave walks its range 64 slots at a time; rank among equal experts in the step.
     // cnt[wave][*] is private to the wave and LDS operations of one wave execute in order, so the loop needs no
     // workgroup barrier; the wave-scope fences keep the compiler from reordering the LDS accesses.
+    int nbits = 1;  // bits that tell experts 0..n_exp-1 apart; the bit above them tells a dropped slot (-1) from all
+    while ((1 << nbits) < n_exp) nbits++;
     for (int s = 0; s < steps; s++) {
         const int e = expert_of(s);
-        unsigned rank = 0, same = 0;
-#pragma unroll
-        for (int i = 0; i < 64; i++) {
-            const int ei = __builtin_amdgcn_readlane(e, i);  // lane i's expert in a scalar register
-            same += ei == e;
-            rank += (ei == e) && (i < lane);
+        // lanes of the step with this lane's expert: one ballot per bit of the expert id, each lane keeps the side
+        // of the ballot its own bit is on (a dropped slot, e = -1, matches only other dropped slots and is not placed)
+        unsigned long long peers = ~0ull;
+        for (int bit = 0; bit <= nbits; bit++) {
+            const bool on = (e >> bit) & 1;
+            const unsigned long long bal = __ballot(on);
+            peers &= on ? bal : ~bal;
         }
+        const unsigned same = (unsigned)__popcll(peers);
+        const unsigned rank = __builtin_amdgcn_mbcnt_hi((unsigned)(peers >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)peers, 0u));
         unsigned before = 0;
         if (e >= 0) before = cnt[wave][e];
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");

@@ -131,6 +131,33 @@ def test_decode_launch_shapes_agree(dec, orc, rows, waves):
     parity.assert_close(got, want, "decode shape %d/%d" % (rows, waves))
 
 
+@pytest.mark.parametrize("nks", [2, 3, 8])
+def test_decode_split_k_across_workgroups(dec, orc, nks):
+    """k slices across workgroups: one launch, the last workgroup of a row-block group adds the slices in slice
+    order, so the result is the same on every run; the automatic choice is covered by the 17408 x 5120 shape above."""
+    n, k, group = 208, 2560, 128  # 13 row blocks, 20 k tiles
+    q, s, x = gen.make_linear(n, k, group, 16, seed=5)
+    dec.upload_lin_g("ks", q, s, n, k, group, False)
+    want = orc.gemm_lane(x, 16, q, s, n, k, group, threads=8)
+    try:
+        dec.set_decode_ksplit(nks)
+        for t in (1, 4, 8, 16):
+            say("decode ksplit", nks, t)
+            got = dec.gemv_host("ks", x[:t], t=t, path=ops.PATH_DECODE)
+            parity.assert_close(got, want[:t], "decode ksplit %d t%d" % (nks, t))
+            for _ in range(3):
+                assert np.array_equal(_bits(got), _bits(dec.gemv_host("ks", x[:t], t=t, path=ops.PATH_DECODE)))
+        # launch shapes and split together, and the tickets are back at zero for an unsplit launch afterwards
+        dec.set_decode_shape(16, 3)
+        parity.assert_close(dec.gemv_host("ks", x[:4], t=4, path=ops.PATH_DECODE), want[:4], "decode ksplit rb1")
+    finally:
+        dec.set_decode_ksplit(0)
+        dec.set_decode_shape(0, 0)
+    parity.assert_close(dec.gemv_host("ks", x[:4], t=4, path=ops.PATH_DECODE), want[:4], "decode after ksplit")
+    with pytest.raises(ops.W4a16Error):
+        dec.set_decode_ksplit(9)
+
+
 def test_decode_bf16_scales(dec, orc):
     n, k, group = 256, 2048, 32
     q, s, x = gen.make_linear(n, k, group, 4, seed=8)
