@@ -196,20 +196,21 @@ int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes) {
     return 0;
 }
 
-// Segment size (slots of one expert per workgroup).  t <= 4: an expert is chosen by at most 4 tokens -> 4;
-// t <= 16 -> 16; beyond, the smallest of 16/32/48/64 that the mean run fills to under 90 %
-// (the reference's rule over its block sizes, kernels/marlin_moe.rs:309-315).
+// Segment size (slots of one expert per workgroup).  Decode steps (t <= 4, top_k <= 8) skip the alignment; up to 8
+// tokens run the streaming kernel on 16-slot segments; beyond that the LDS-staged kernel, whose segment size follows
+// the mean run per expert: 32 slots below a mean of 24, 48 below 40, else 64.  The reference picks the smallest of
+// 16/32/48/64 that the mean run fills to under 90 % (kernels/marlin_moe.rs:309-315); measured here (128 experts,
+// top-8, T = 16..1024) 32-slot segments beat 16-slot ones at every T, and the larger sizes win once most experts would
+// need a second segment.
 static size_t pick_block(const w4a16_ctx* ctx, size_t t, size_t ns, size_t n_exp, size_t top_k) {
     if (ctx->moe_block) return (size_t)ctx->moe_block;
     if (t <= 4 && top_k <= 8) return 1;  // direct mode: no alignment, two launches (see w4a16_moe_ffn)
     if (t <= 4) return 4;
-    if (t <= 16) return 16;
-    for (size_t b : {16, 32, 48, 64})
-        if ((double)ns / (double)n_exp / (double)b < 0.9) return b;
-    return 64;
+    if (t <= 8) return 16;
+    const double mean = (double)ns / (double)n_exp;
+    return mean < 24.0 ? 32 : mean < 40.0 ? 48 : 64;
 }
 
-// One grouped GEMM: y[slot] = W[expert(slot)] * x[slot / x_div] over the aligned segments.
 static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_t x, size_t x_rows, size_t x_div,
                            uint64_t y, int y_f16, uint64_t topw, size_t ns, size_t block, size_t max_segs,
                            uint64_t sorted, uint64_t eids, uint64_t npost) {
