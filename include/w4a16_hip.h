@@ -257,6 +257,14 @@ int w4a16_upload_lin_synth(w4a16_ctx* ctx, const char* name, size_t n, size_t k,
  * c < ncols <= ld.  The sum of squares is taken in f64 in a fixed order (1024 strided partials, pairwise fold), so a
  * CPU restatement is bit-identical. */
 int w4a16_rms_rescale_f16(w4a16_ctx* ctx, uint64_t v_f32_dev, size_t ld, size_t ncols, size_t t, uint64_t out_f16_dev);
+/* norm_resid / norm_resid_g (assets/norm.cu:4-48, 97-148; launched by norm_resid_at, w4a16_dec/kernels/mod.rs:11-54):
+ * the residual add and RMS normalisation that produces the f16 A operand of a layer's first linear.  Per token row,
+ * with v = x + ab:  x <- v;  xn = v * inv * nw[w_off + c], inv = 1/sqrtf(sum(v^2)/hidden + 1e-6f);  xn32 (0 = skip) =
+ * xn rounded to f16 and widened back;  xn16 (0 = skip) = the f16 bits.  x, ab, xn, xn32: f32 [t][hidden]; nw: f32, at
+ * least w_off + hidden long; hidden <= 8192.  Same f32 operations in the same order as the reference kernel (one fused
+ * multiply-add per square, its tree reduction, correctly rounded divide and square root): bit-identical results. */
+int w4a16_norm_resid(w4a16_ctx* ctx, uint64_t x_dev, uint64_t nw_dev, uint64_t ab_dev, uint64_t xn_dev, uint64_t xn32_dev,
+                     uint64_t xn16_dev, size_t t, size_t w_off, size_t hidden);
 /* ew (assets/ew.cu:9-32): out[r][c] = f16(silu(gu[r][c]) * gu[r][n_ff + c]) for gu f32 [t][2*n_ff], f32 arithmetic. */
 int w4a16_silu_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_ff, size_t t, uint64_t out_f16_dev);
 

@@ -59,6 +59,17 @@ extern "C" int w4a16_rms_rescale_f16(w4a16_ctx* ctx, uint64_t v_f32_dev, size_t 
     return w4_launch(ctx, "w4a16_rms_rescale_f16", (unsigned)t, 1, 1024, 0, p);
 }
 
+extern "C" int w4a16_norm_resid(w4a16_ctx* ctx, uint64_t x_dev, uint64_t nw_dev, uint64_t ab_dev, uint64_t xn_dev,
+                                uint64_t xn32_dev, uint64_t xn16_dev, size_t t, size_t w_off, size_t hidden) {
+    if (!ctx || !x_dev || !nw_dev || !ab_dev || !xn_dev) return w4_fail(W4A16_ERR_ARG, "norm_resid: null argument");
+    if (t == 0 || hidden == 0 || hidden > 8192 || t > 0x7fffffffu || w_off > 0x7fffffffu - hidden)
+        return w4_fail(W4A16_ERR_SHAPE, "norm_resid: t=%zu hidden=%zu (1..8192) w_off=%zu", t, hidden, w_off);
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    int wo = (int)w_off, hd = (int)hidden;
+    void* p[] = {&x_dev, &nw_dev, &ab_dev, &xn_dev, &xn32_dev, &xn16_dev, &wo, &hd};
+    return w4_launch(ctx, "w4a16_norm_resid", (unsigned)t, 1, 1024, 0, p);
+}
+
 extern "C" int w4a16_silu_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_ff, size_t t, uint64_t out_f16_dev) {
     if (!ctx || !gu_f32_dev || !out_f16_dev) return w4_fail(W4A16_ERR_ARG, "silu_mul: null argument");
     if (t == 0 || n_ff == 0 || n_ff > 0x3fffffffu || t > 0x7fffffffu)

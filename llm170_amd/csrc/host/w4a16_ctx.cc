@@ -67,7 +67,7 @@ static const char* const kPrefillSyms[] = {"w4a16_prefill_g128_f16", "w4a16_pref
                                            "w4a16_prefill_g32_bf16", "w4a16_prefill_splitk_sum", nullptr};
 static const char* const kUtilSyms[] = {"w4a16_fill0_u32", "w4a16_copy_u4", nullptr};
 static const char* const kGlueSyms[] = {"w4a16_rms_rescale_f16", "w4a16_silu_mul_f16", "w4a16_synth_q", "w4a16_synth_s",
-                                        nullptr};
+                                        "w4a16_norm_resid", nullptr};
 #define W4_MOE_FAMILY(P)                                                                                      \
     P "_dec_glu_x1", P "_dec_glu_x4", P "_dec_lin_x1", P "_dec_lin_x4", P "_mm_glu_t1", P "_mm_glu_t2",       \
         P "_mm_glu_t3", P "_mm_glu_t4", P "_mm_lin_t1", P "_mm_lin_t2", P "_mm_lin_t3", P "_mm_lin_t4"

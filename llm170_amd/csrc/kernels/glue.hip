@@ -59,6 +59,60 @@ extern "C" __global__ __launch_bounds__(RMS_LANES) void w4a16_rms_rescale_f16(co
     for (int c = tid + RMS_LANES * RMS_UNROLL; c < ncols; c += RMS_LANES) o[c] = glue_round_f16(row[c] * inv);
 }
 
+// RMS normalisation with residual add, the producer of the f16 A operand of a layer's first linear
+// (assets/norm.cu:4-48 norm_resid and :97-148 norm_resid_g, one kernel here).  Per token row r, with v = x + ab:
+//   x <- v;  xn = v * inv * nw[w_off + c],  inv = 1 / sqrtf(sum(v^2) / hidden + 1e-6f);
+//   xn32 (optional) = xn rounded to f16 and widened back;  xn16 (optional) = the f16 bits.
+// The f32 arithmetic is the reference's, in its order, so results agree bit for bit with a CPU restatement: thread tid
+// of 1024 adds its columns tid, tid + 1024, ... with one fused multiply-add each (that kernel file is built with
+// nvcc's default -fmad=true, scripts/build_cuda_kernels.sh:67), the 1024 partials are folded pairwise at strides 512,
+// 256, ..., 1, the division and square root are correctly rounded, and v * inv * nw is two roundings.  hidden <= 8192.
+extern "C" __global__ __launch_bounds__(1024) void w4a16_norm_resid(float* __restrict__ x, const float* __restrict__ nw,
+                                                                    const float* __restrict__ ab, float* __restrict__ xn,
+                                                                    float* __restrict__ xn32, uint16_t* __restrict__ xn16,
+                                                                    int w_off, int hidden) {
+    __shared__ float red[1024];
+    const int tid = threadIdx.x;
+    const size_t base = (size_t)blockIdx.x * hidden;
+    float v[8];
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int c = j * 1024 + tid;
+        v[j] = 0.0f;
+        if (c < hidden) {
+            v[j] = x[base + c] + ab[base + c];
+            ss = __builtin_fmaf(v[j], v[j], ss);
+        }
+    }
+    red[tid] = ss;
+    __syncthreads();
+    for (int st = 512; st >= 64; st >>= 1) {
+        if (tid < st) red[tid] = red[tid] + red[tid + st];
+        __syncthreads();
+    }
+    float r = red[tid & 63];  // strides 32..1 inside every wave, same pairing; lane 0 ends with the row's sum
+#pragma unroll
+    for (int st = 32; st > 0; st >>= 1) r = r + __shfl_down(r, st);
+    r = __shfl(r, 0);
+    const float inv = 1.0f / sqrtf(r / (float)hidden + 1e-6f);
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int c = j * 1024 + tid;
+        if (c >= hidden) continue;
+        float y = v[j] * inv;
+        asm volatile("" : "+v"(y));  // two roundings, never one fused product
+        y = y * nw[w_off + c];
+        xn[base + c] = y;
+        if (xn32 || xn16) {
+            const _Float16 h = glue_round_f16(y);
+            if (xn32) xn32[base + c] = (float)h;
+            if (xn16) xn16[base + c] = __builtin_bit_cast(uint16_t, h);
+        }
+        x[base + c] = v[j];
+    }
+}
+
 // out[r][c] = f16((g / (1 + exp(-g))) * u),  g = gu[r][c], u = gu[r][n_ff + c], all in f32 (assets/ew.cu:19-30).
 // Four columns per thread when n_ff % 4 == 0.
 extern "C" __global__ __launch_bounds__(256) void w4a16_silu_mul_f16(const float* __restrict__ gu, int n_ff, int t,

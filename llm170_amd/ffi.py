@@ -75,6 +75,8 @@ _SIGS = {
     "w4a16_upload_lin_synth": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint64, C.c_uint64,
                                          C.c_float, C.c_float]),
     "w4a16_rms_rescale_f16": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint64]),
+    "w4a16_norm_resid": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64,
+                                   C.c_size_t, C.c_size_t, C.c_size_t]),
     "w4a16_silu_mul_f16": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64]),
     "w4a16_chain_forward": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64]),
     "w4a16_bench_chain": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t,

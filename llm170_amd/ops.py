@@ -321,6 +321,11 @@ class W4a16Dec:
     def rms_rescale_f16(self, v_dev, ld, ncols, t, out_dev):
         ffi.check(self.cc.lib.w4a16_rms_rescale_f16(self.cc.h, v_dev, ld, ncols, t, out_dev))
 
+    def norm_resid(self, x_dev, nw_dev, ab_dev, xn_dev, t, hidden, w_off=0, xn32_dev=0, xn16_dev=0):
+        """x <- x + ab; xn = x * inv_rms * nw[w_off:]; optional f16-rounded copies (0 = skip)."""
+        ffi.check(self.cc.lib.w4a16_norm_resid(self.cc.h, x_dev, nw_dev, ab_dev, xn_dev, xn32_dev, xn16_dev, t, w_off,
+                                               hidden))
+
     def silu_mul_f16(self, gu_dev, n_ff, t, out_dev):
         ffi.check(self.cc.lib.w4a16_silu_mul_f16(self.cc.h, gu_dev, n_ff, t, out_dev))
 

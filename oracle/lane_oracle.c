@@ -28,6 +28,10 @@
  *   orc_rms_rescale_f16 ... float64 v / sqrt(mean(v^2) + 1e-6) within one f16 step, >= 99.9 % identical; constant rows;
  *                           invariance of the output under scaling the row by a power of two
  *   orc_silu_mul_f16_rows . float64 evaluation within one f16 step; layout (gate | up) by a crafted row
+ *   orc_norm_resid ........ numpy float32 restatement whose fused multiply-add is built from exact f64 products and a
+ *                           round-to-odd sum (independent of libm's fmaf); float64 v/sqrt(mean v^2 + 1e-6)*w to a few f32
+ *                           ulp; x + ab exact; an un-fused sum of squares and a sequential (non-tree) sum are shown to
+ *                           give different bits; f16 copies against numpy float16
  * No function here is "parity unpinned".
  */
 #include <math.h>
@@ -419,6 +423,43 @@ void orc_rms_rescale_f16(const float* v, size_t ld, size_t ncols, size_t t, uint
             for (size_t i = 0; i < st; i++) red[i] = red[i] + red[i + st];
         const float inv = (float)(1.0 / sqrt(red[0] / (double)ncols + 1e-6));
         for (size_t c = 0; c < ncols; c++) out[r * ncols + c] = orc_f32_to_f16(row[c] * inv);
+    }
+}
+
+/* ---- norm_resid / norm_resid_g (crates/backend-gpu/src/rawcuda/assets/norm.cu:4-48, 97-148), f32 throughout.
+ * Thread tid of 1024 adds the squares of its columns tid, tid+1024, ... with one fused multiply-add each: the file is
+ * compiled with nvcc's default -fmad=true (scripts/build_cuda_kernels.sh:67 "build norm", unlike the kernels built
+ * with -fmad=false), which contracts ss += v*v.  Partials are folded at strides 512..1; divide and square root are
+ * IEEE (nvcc defaults -prec-div=true -prec-sqrt=true).  x is updated in place to x + ab.  xn32 / xn16 may be NULL. ---- */
+void orc_norm_resid(float* x, const float* nw, const float* ab, float* xn, float* xn32, uint16_t* xn16, size_t t,
+                    size_t w_off, size_t hidden) {
+    for (size_t r = 0; r < t; r++) {
+        float* xr = x + r * hidden;
+        const float* ar = ab + r * hidden;
+        float red[1024];
+        for (size_t tid = 0; tid < 1024; tid++) {
+            float ss = 0.0f;
+            for (size_t c = tid; c < hidden; c += 1024) {
+                const float v = xr[c] + ar[c];
+                ss = fmaf(v, v, ss);
+            }
+            red[tid] = ss;
+        }
+        for (size_t st = 512; st > 0; st >>= 1)
+            for (size_t i = 0; i < st; i++) red[i] = red[i] + red[i + st];
+        const float inv = 1.0f / sqrtf(red[0] / (float)hidden + 1e-6f);
+        for (size_t c = 0; c < hidden; c++) {
+            const float v = xr[c] + ar[c];
+            volatile float y0 = v * inv; /* two roundings */
+            const float y = y0 * nw[w_off + c];
+            xn[r * hidden + c] = y;
+            if (xn32 || xn16) {
+                const uint16_t h = orc_f32_to_f16(y);
+                if (xn32) xn32[r * hidden + c] = orc_half_to_f32(h);
+                if (xn16) xn16[r * hidden + c] = h;
+            }
+            xr[c] = v;
+        }
     }
 }
 

@@ -56,6 +56,7 @@ def lib():
         L.orc_f32_to_f16_array.argtypes, L.orc_f32_to_f16_array.restype = [f32p, sz, u16p], None
         L.orc_rms_rescale_f16.argtypes, L.orc_rms_rescale_f16.restype = [f32p, sz, sz, sz, u16p], None
         L.orc_silu_mul_f16_rows.argtypes, L.orc_silu_mul_f16_rows.restype = [f32p, sz, sz, u16p], None
+        L.orc_norm_resid.argtypes, L.orc_norm_resid.restype = [f32p, f32p, f32p, f32p, f32p, u16p, sz, sz, sz], None
         i32p = C.POINTER(C.c_int32)
         L.orc_moe_act_silu_f16.argtypes, L.orc_moe_act_silu_f16.restype = [u16p, sz, sz, u16p], None
         L.orc_moe_topk_sum_f16.argtypes, L.orc_moe_topk_sum_f16.restype = [u16p, sz, sz, sz, f32p], None
@@ -273,6 +274,18 @@ def rms_rescale_f16(v, ncols):
     out = np.empty((t, ncols), np.uint16)
     lib().orc_rms_rescale_f16(_p(v, C.c_float), ld, ncols, t, _p(out, C.c_uint16))
     return out
+
+
+def norm_resid(x, nw, ab, w_off=0):
+    """norm_resid (assets/norm.cu:4-48): returns (x + ab, xn f32, xn32 f32, xn16 f16 bits), each [t][hidden]."""
+    x = np.array(x, np.float32, order="C")  # copy: updated in place
+    ab, nw = _c(ab, np.float32), _c(nw, np.float32)
+    t, hidden = x.shape
+    assert ab.shape == x.shape and nw.size >= w_off + hidden
+    xn, xn32, xn16 = np.empty_like(x), np.empty_like(x), np.empty(x.shape, np.uint16)
+    lib().orc_norm_resid(_p(x, C.c_float), _p(nw, C.c_float), _p(ab, C.c_float), _p(xn, C.c_float), _p(xn32, C.c_float),
+                         _p(xn16, C.c_uint16), t, w_off, hidden)
+    return x, xn, xn32, xn16
 
 
 def silu_mul_f16_rows(gu):

@@ -229,3 +229,59 @@ def test_chain_errors(dec):
     dec.upload_lin_synth("brk.0.ffn_down", 128, 128, 128, 1, 2)
     with pytest.raises(ops.W4a16Error):  # qkv narrower than hidden
         dec.chain_forward("brk", 0, 1, 1, 1, 1)
+
+
+# ------------------------------------------------------------------ norm_resid (assets/norm.cu:4-48, 97-148)
+@pytest.mark.parametrize("t,hidden,w_off", [(1, 5120, 0), (4, 5120, 5120), (7, 2048, 0), (3, 1000, 24), (2, 8192, 0),
+                                            (5, 64, 0)])
+@pytest.mark.parametrize("copies", ["both", "f16 only", "none"])
+def test_norm_resid_bit_exact(dec, orc, t, hidden, w_off, copies):
+    print("norm_resid", t, hidden, w_off, copies, flush=True)
+    cc = dec.cc
+    x = gen.normal_f32(300 + hidden, (t, hidden)) * np.float32(3.0)
+    ab = gen.normal_f32(301 + hidden, (t, hidden))
+    nw = (np.float32(1.0) + gen.normal_f32(302 + hidden, (w_off + hidden,)) * np.float32(0.1)).astype(np.float32)
+    want_x, want_xn, want_xn32, want_xn16 = orc.norm_resid(x, nw, ab, w_off)
+    px, pw, pa = cc.to_device(x), cc.to_device(nw), cc.to_device(ab)
+    pn, p32, p16 = cc.alloc(t * hidden * 4), cc.alloc(t * hidden * 4), cc.alloc(t * hidden * 2)
+    dec.norm_resid(px, pw, pa, pn, t, hidden, w_off, xn32_dev=p32 if copies == "both" else 0,
+                   xn16_dev=0 if copies == "none" else p16)
+    got_x, got_xn = cc.d2h(px, (t, hidden), np.float32), cc.d2h(pn, (t, hidden), np.float32)
+    assert np.array_equal(got_x.view(np.uint32), want_x.view(np.uint32))
+    assert np.array_equal(got_xn.view(np.uint32), want_xn.view(np.uint32))
+    if copies != "none":
+        assert np.array_equal(cc.d2h(p16, (t, hidden), np.uint16), want_xn16)
+    if copies == "both":
+        assert np.array_equal(cc.d2h(p32, (t, hidden), np.float32).view(np.uint32), want_xn32.view(np.uint32))
+    for p in (px, pw, pa, pn, p32, p16):
+        cc.free(p)
+
+
+def test_norm_resid_feeds_the_linear(dec, orc):
+    """The f16 copy is the A operand of the next linear: norm_resid -> decode GEMV against the oracle's lane GEMM of
+    the oracle's f16 copy."""
+    t, hidden, n = 4, 2048, 512
+    cc = dec.cc
+    x = gen.normal_f32(11, (t, hidden))
+    ab = gen.normal_f32(12, (t, hidden))
+    nw = np.ones(hidden, np.float32)
+    q, s, _ = gen.make_linear(n, hidden, 128, 1, seed=13)
+    dec.upload_lin_g("after_norm", q, s, n, hidden, 128, False)
+    _, _, _, x16 = orc.norm_resid(x, nw, ab, 0)
+    want = orc.gemm_lane(x16, t, q, s, n, hidden, 128, threads=4)
+    px, pw, pa = cc.to_device(x), cc.to_device(nw), cc.to_device(ab)
+    pn, p16, py = cc.alloc(t * hidden * 4), cc.alloc(t * hidden * 2), cc.alloc(t * n * 4)
+    dec.norm_resid(px, pw, pa, pn, t, hidden, xn16_dev=p16)
+    dec.lin_forward("after_norm", p16, py, t, path=ops.PATH_DECODE)
+    parity.assert_close(cc.d2h(py, (t, n), np.float32), want, "norm_resid -> decode")
+    for p in (px, pw, pa, pn, p16, py):
+        cc.free(p)
+
+
+def test_norm_resid_errors(dec):
+    with pytest.raises(ops.W4a16Error):
+        dec.norm_resid(1, 1, 1, 1, 1, 8193)
+    with pytest.raises(ops.W4a16Error):
+        dec.norm_resid(0, 1, 1, 1, 1, 1024)
+    with pytest.raises(ops.W4a16Error):
+        dec.norm_resid(1, 1, 1, 1, 0, 1024)
