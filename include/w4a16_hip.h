@@ -119,6 +119,12 @@ int w4a16_upload_lin(w4a16_ctx* ctx, const char* name, const void* q, size_t qle
 /* consolidate_marlin_dense (upload.rs:67-97): free the as-given copy of one linear once the tiled one exists
  * (bit-exact path and raw dump then report W4A16_ERR_NOT_FOUND for it). */
 int w4a16_lin_drop_raw(w4a16_ctx* ctx, const char* name);
+/* Fuse registered linears that read the same activations (q/k/v, gate/up) into one, rows concatenated in the order
+ * given, so that one launch serves them all: y[:, 0:n0] is part 0, y[:, n0:n0+n1] part 1, ...  The reference reaches the
+ * same end with a table of segments for its multi-linear GEMV (build_multi_tables, w4a16_dec/buffers.rs:229-366) and with
+ * fused gate|up arenas (upload.rs:1116-1235).  Parts need the same k, group and scale type and their as-given operands;
+ * drop_parts != 0 unregisters them afterwards.  A fused gate|up linear is what w4a16_lin_forward_glu takes. */
+int w4a16_lin_fuse(w4a16_ctx* ctx, const char* name, const char* const* parts, size_t n_parts, int drop_parts);
 /* lin_spec (w4a16_dec/mod.rs:1193-1206): shape of a registered linear. */
 int w4a16_lin_info(w4a16_ctx* ctx, const char* name, size_t* n, size_t* k, size_t* group, int* scale_bf16,
                    int* has_tiled, int* has_raw);

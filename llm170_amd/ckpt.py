@@ -282,6 +282,17 @@ class W4a16Model:
             done.append(base)
         return done
 
+    def upload_fused(self, dec, name, bases):
+        """Register the linears `bases` (which share their input: q/k/v, gate/up) as ONE linear `name`, rows in the
+        order given; the parts are uploaded, fused on the device and dropped."""
+        tmp = []
+        for i, base in enumerate(bases):
+            q, s, n, k, bf = self.lin_operands(base)
+            part = "%s.__part%d" % (name, i)
+            dec.upload_lin_g(part, q, s, n, k, self.group, bf)
+            tmp.append(part)
+        dec.lin_fuse(name, tmp, drop_parts=True)
+
     def close(self):
         self.ar.close()
 

@@ -277,6 +277,61 @@ extern "C" int w4a16_upload_lin(w4a16_ctx* ctx, const char* name, const void* q,
     return w4_register_lin(ctx, name, L);
 }
 
+// Several linears that read the same x become one (rows concatenated in the order given), so that one launch serves
+// them all: the as-given operands are row-major, so the fused operands are plain concatenations.
+extern "C" int w4a16_lin_fuse(w4a16_ctx* ctx, const char* name, const char* const* parts, size_t n_parts,
+                              int drop_parts) {
+    if (!ctx || !name || !parts || n_parts == 0) return w4_fail(W4A16_ERR_ARG, "lin_fuse: null argument");
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    std::vector<W4Lin*> P(n_parts);
+    W4Lin F;
+    for (size_t i = 0; i < n_parts; i++) {
+        if (!parts[i]) return w4_fail(W4A16_ERR_ARG, "lin_fuse %s: part %zu is null", name, i);
+        if (std::string(parts[i]) == name) return w4_fail(W4A16_ERR_ARG, "lin_fuse %s: a part has the fused name", name);
+        for (size_t j = 0; j < i; j++)
+            if (std::string(parts[i]) == parts[j]) return w4_fail(W4A16_ERR_ARG, "lin_fuse %s: part %s twice", name, parts[i]);
+        W4_TRY(w4_find_lin(ctx, parts[i], &P[i]));
+        const W4Lin& L = *P[i];
+        if (!L.q_raw) return w4_fail(W4A16_ERR_NOT_FOUND, "lin_fuse %s: part %s has dropped its as-given operands", name, parts[i]);
+        if (i == 0) {
+            F.k = L.k;
+            F.group = L.group;
+            F.scale_bf16 = L.scale_bf16;
+        } else if (L.k != F.k || L.group != F.group || L.scale_bf16 != F.scale_bf16) {
+            return w4_fail(W4A16_ERR_SHAPE, "lin_fuse %s: part %s (k=%zu g=%zu bf16=%d) does not match k=%zu g=%zu bf16=%d",
+                           name, parts[i], L.k, L.group, L.scale_bf16, F.k, F.group, F.scale_bf16);
+        }
+        F.n += L.n;
+        F.scales_regular = F.scales_regular && L.scales_regular;
+    }
+    if (F.n > 0x7fffffffu) return w4_fail(W4A16_ERR_SHAPE, "lin_fuse %s: n=%zu too large", name, F.n);
+    const size_t q_row = F.k / 2, s_row = (F.k / F.group) * 2;
+    int rc = w4a16_alloc(ctx, F.n * q_row, &F.q_raw);
+    if (!rc) rc = w4a16_alloc(ctx, F.n * s_row, &F.s_raw);
+    size_t row = 0;
+    for (size_t i = 0; i < n_parts && !rc; i++) {
+        rc = w4a16_d2d(ctx, F.q_raw + row * q_row, P[i]->q_raw, P[i]->n * q_row);
+        if (!rc) rc = w4a16_d2d(ctx, F.s_raw + row * s_row, P[i]->s_raw, P[i]->n * s_row);
+        row += P[i]->n;
+    }
+    if (rc) {
+        const std::string keep = w4_err_save();
+        free_lin(ctx, F);
+        w4_err_restore(keep);
+        return rc;
+    }
+    W4_TRY(w4_register_lin(ctx, name, F));  // builds the tiled copy and waits for the stream
+    if (drop_parts)
+        for (size_t i = 0; i < n_parts; i++) {
+            auto it = ctx->lins.find(parts[i]);
+            if (it != ctx->lins.end()) {
+                free_lin(ctx, it->second);
+                ctx->lins.erase(it);
+            }
+        }
+    return 0;
+}
+
 // Second half of a registration: build the tiled copy from the as-given operands already on the device and enter
 // the linear under its name.  Frees L's buffers on failure.
 int w4_register_lin(w4a16_ctx* ctx, const char* name, W4Lin& L) {

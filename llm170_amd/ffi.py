@@ -51,6 +51,7 @@ _SIGS = {
     "w4a16_lin_forward_host": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int]),
     "w4a16_dequant_dump": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int, C.c_uint64]),
     "w4a16_lin_untile": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64]),
+    "w4a16_lin_fuse": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_char_p), C.c_size_t, C.c_int]),
     "w4a16_set_decode_shape": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "w4a16_set_decode_ksplit": (C.c_int, [C.c_void_p, C.c_int]),
     "w4a16_set_prefill_ksplit": (C.c_int, [C.c_void_p, C.c_int]),

@@ -171,6 +171,11 @@ class W4a16Dec:
         ffi.check(self.cc.lib.w4a16_upload_lin(self.cc.h, name.encode(), _ptr(q), q.nbytes, _ptr(s), s.nbytes, n, k,
                                                group, int(bool(scale_bf16))))
 
+    def lin_fuse(self, name, parts, drop_parts=False):
+        """One linear from several that share x (rows concatenated in the order given)."""
+        arr = (C.c_char_p * len(parts))(*[p.encode() for p in parts])
+        ffi.check(self.cc.lib.w4a16_lin_fuse(self.cc.h, name.encode(), arr, len(parts), int(bool(drop_parts))))
+
     def lin_spec(self, name):
         n, k, g = C.c_size_t(), C.c_size_t(), C.c_size_t()
         bf, tiled, raw = C.c_int(), C.c_int(), C.c_int()
