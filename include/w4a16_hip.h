@@ -131,10 +131,11 @@ int w4a16_lin_info(w4a16_ctx* ctx, const char* name, size_t* n, size_t* k, size_
 
 /* LinPath (w4a16_dec/mod.rs:79-84) */
 enum {
-    W4A16_PATH_AUTO = 0,   /* t <= 16 -> DECODE, else PREFILL; LANE when the linear has no tiled copy            */
+    W4A16_PATH_AUTO = 0,   /* t <= 16 -> DECODE, t <= 64 -> STREAM, else PREFILL; LANE without a tiled copy             */
     W4A16_PATH_LANE = 1,   /* bit-exact twin of lane.rs (reference: w4a16_gemm_g128, gptq4.cu:825-951)            */
     W4A16_PATH_DECODE = 2, /* HBM-streaming skinny GEMM, t <= 16 (reference: gemv_t_launch / sk_*_dev)            */
-    W4A16_PATH_PREFILL = 3 /* LDS-staged MFMA GEMM, any t (reference: gemm_launch -> marlin_gemm_try)             */
+    W4A16_PATH_PREFILL = 3, /* LDS-staged MFMA GEMM, any t (reference: gemm_launch -> marlin_gemm_try)            */
+    W4A16_PATH_STREAM = 4   /* weight-streaming kernel with x shared through LDS, segments of up to 64 rows       */
 };
 
 /* lin_forward (w4a16_dec/kernels/mod.rs:121-144): y[t][n] = x[t][k] * W^T on the launch stream, no host sync.

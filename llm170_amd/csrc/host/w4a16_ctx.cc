@@ -70,7 +70,8 @@ static const char* const kGlueSyms[] = {"w4a16_rms_rescale_f16", "w4a16_silu_mul
                                         "w4a16_norm_resid", nullptr};
 #define W4_MOE_FAMILY(P)                                                                                      \
     P "_dec_glu_x1", P "_dec_glu_x4", P "_dec_lin_x1", P "_dec_lin_x4", P "_mm_glu_t1", P "_mm_glu_t2",       \
-        P "_mm_glu_t3", P "_mm_glu_t4", P "_mm_lin_t1", P "_mm_lin_t2", P "_mm_lin_t3", P "_mm_lin_t4"
+        P "_mm_glu_t3", P "_mm_glu_t4", P "_mm_lin_t1", P "_mm_lin_t2", P "_mm_lin_t3", P "_mm_lin_t4",       \
+        P "_mm_lin_t1_ks", P "_mm_lin_t2_ks", P "_mm_lin_t3_ks", P "_mm_lin_t4_ks"
 static const char* const kMoeSyms[] = {W4_MOE_FAMILY("w4a16_moe_g32_f16"),
                                        W4_MOE_FAMILY("w4a16_moe_g32_bf16"),
                                        W4_MOE_FAMILY("w4a16_moe_g128_f16"),

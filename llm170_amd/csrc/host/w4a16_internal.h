@@ -41,6 +41,8 @@ struct W4MoeScratch {
     size_t block = 0;
     uint64_t iota = 0, always = 0;  // direct mode: identity segment table and a "padded total" no slot index reaches
     size_t iota_cap = 0;            // entries
+    uint64_t zeros = 0;             // all-zero expert table for a dense linear run as one expert
+    size_t zeros_cap = 0;           // entries
 };
 
 // Scratch of the layer chain, grown on demand (reference: dchain / dx16 / dy buffers, w4a16_dec/buffers.rs).
@@ -87,6 +89,7 @@ int w4_launch(w4a16_ctx* ctx, const char* symbol, unsigned gx, unsigned gy, unsi
 int w4_register_lin(w4a16_ctx* ctx, const char* name, W4Lin& L);
 int w4_find_lin(w4a16_ctx* ctx, const char* name, W4Lin** out);
 int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes);
+int w4_dense_grouped(w4a16_ctx* ctx, const W4Lin& L, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16);
 
 #define W4_TRY(expr)          \
     do {                      \

@@ -213,7 +213,7 @@ static size_t pick_block(const w4a16_ctx* ctx, size_t t, size_t ns, size_t n_exp
 
 static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_t x, size_t x_rows, size_t x_div,
                            uint64_t y, int y_f16, uint64_t topw, size_t ns, size_t block, size_t max_segs,
-                           uint64_t sorted, uint64_t eids, uint64_t npost) {
+                           uint64_t sorted, uint64_t eids, uint64_t npost, size_t nks = 1) {
     const size_t n = glu ? 2 * E.n_ff : E.h, k = glu ? E.h : E.n_ff;
     const size_t row_blocks = (n + 15) / 16, kt_n = k / 128;
     const size_t units = glu ? row_blocks / 2 : (row_blocks + 1) / 2;
@@ -223,7 +223,9 @@ static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_
     unsigned long long qs = glu ? E.q13_stride : E.q2_stride, ss = glu ? E.s13_stride : E.s2_stride;
     int xr = (int)x_rows, xd = (int)x_div, yf = y_f16, blk = (int)block, nsi = (int)ns, rbi = (int)row_blocks,
         ki = (int)k, ni = (int)n, nei = (int)E.n_exp;
-    void* p[] = {&qa, &sa, &qs, &ss, &x, &xr, &xd, &y, &yf, &topw, &sorted, &eids, &npost, &blk, &nsi, &rbi, &ki, &ni, &nei};
+    uint64_t ws = 0, tk = 0;
+    void* p[] = {&qa, &sa, &qs, &ss, &x, &xr, &xd, &y, &yf, &topw, &sorted, &eids, &npost, &blk, &nsi, &rbi, &ki, &ni, &nei,
+                 &ws, &tk};
     char sym[80];
     const char* fam = E.scale_bf16 ? "bf16" : "f16";
     if (block <= 16) {
@@ -237,10 +239,78 @@ static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_
     const int tt = (int)(block / 16);
     int waves = ctx->moe_waves ? ctx->moe_waves : 4;
     waves = waves >= 8 ? 8 : 4;  // the x staging needs at least 4 waves
-    const size_t groups = (units + (size_t)waves - 1) / (size_t)waves;
-    snprintf(sym, sizeof sym, "w4a16_moe_g%zu_%s_mm_%s_t%d", E.group, fam, glu ? "glu" : "lin", tt);
+    const size_t blocks = max_segs * ((units + (size_t)waves - 1) / (size_t)waves);
+    nks = std::max<size_t>(1, std::min<size_t>(std::min<size_t>(nks, 8), kt_n / 2));
+    if (nks > 1) {
+        // split over k across workgroups: partial tiles and per-(block, wave) tickets, shared with the decode kernel
+        W4_TRY(w4_ensure(ctx, &ctx->decode_ws, &ctx->decode_ws_cap, blocks * (size_t)waves * 2 * (size_t)tt * 1024 * nks));
+        if (blocks * (size_t)waves * 4 > ctx->decode_tickets_cap) {
+            W4_TRY(w4_ensure(ctx, &ctx->decode_tickets, &ctx->decode_tickets_cap,
+                             std::max<size_t>(blocks * (size_t)waves * 4, 16384)));
+            W4_TRY(w4a16_memset0(ctx, ctx->decode_tickets, ctx->decode_tickets_cap));
+        }
+        ws = ctx->decode_ws;
+        tk = ctx->decode_tickets;
+    }
+    if (nks > 1 && glu) return w4_fail(W4A16_ERR_UNSUPPORTED, "moe: the gate|up kernel does not split over k");
+    snprintf(sym, sizeof sym, "w4a16_moe_g%zu_%s_mm_%s_t%d%s", E.group, fam, glu ? "glu" : "lin", tt, nks > 1 ? "_ks" : "");
     const unsigned shmem = (unsigned)(2 * 16 * tt * 136 * 2);
-    return w4_launch(ctx, sym, (unsigned)(max_segs * groups), 1, (unsigned)(waves * 64), shmem, p);
+    return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, p);
+}
+
+// A dense linear at a few dozen rows through the LDS-staged grouped kernel: one "expert" (the linear itself), slot =
+// token, segments of up to 64 tokens.  Between the streaming decode kernel (t <= 16: x operands straight from global
+// memory) and the 128-row MFMA tiles of the prefill kernel, this regime is still bound by the weight stream, and the
+// grouped kernel shares each x tile among all waves of a workgroup through LDS.
+int w4_dense_grouped(w4a16_ctx* ctx, const W4Lin& L, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16) {
+    if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "stream: linear has no tiled copy (needs k %% 128 == 0)");
+    if (t > 0x7fffffffu / 2) return w4_fail(W4A16_ERR_SHAPE, "stream: t=%zu too large", t);
+    W4MoeScratch& S = ctx->moe;
+    const size_t block = ctx->moe_block >= 16 ? (size_t)ctx->moe_block : t <= 16 ? 16 : t <= 32 ? 32 : t <= 48 ? 48 : 64;
+    const size_t segs = (t + block - 1) / block, padded = segs * block;
+    // identity slot table (entries >= t are the padding sentinel by themselves), all-zero expert table, padded total
+    if (S.iota_cap < padded) {
+        const size_t cap = std::max<size_t>(padded, 4096);
+        std::vector<int32_t> host(cap);
+        for (size_t i = 0; i < cap; i++) host[i] = (int32_t)i;
+        size_t bytes_cap = S.iota_cap * 4;
+        W4_TRY(w4_ensure(ctx, &S.iota, &bytes_cap, cap * 4));
+        W4_TRY(w4a16_h2d(ctx, S.iota, host.data(), cap * 4));
+        S.iota_cap = cap;
+    }
+    if (S.zeros_cap < segs) {
+        const size_t cap = std::max<size_t>(segs, 1024);
+        size_t bytes_cap = S.zeros_cap * 4;
+        W4_TRY(w4_ensure(ctx, &S.zeros, &bytes_cap, cap * 4));
+        W4_TRY(w4a16_memset0(ctx, S.zeros, cap * 4));
+        S.zeros_cap = cap;
+    }
+    if (!S.always) {
+        const int32_t big[2] = {0x7fffffff, 0};
+        W4_TRY(w4a16_alloc(ctx, 8, &S.always));
+        W4_TRY(w4a16_h2d(ctx, S.always, big, 8));
+    }
+    W4Experts E;
+    E.q2 = L.q_tiled;
+    E.s2 = L.s_tiled;
+    E.n_exp = 1;
+    E.h = L.n;
+    E.n_ff = L.k;
+    E.group = L.group;
+    E.scale_bf16 = L.scale_bf16;
+    // k slices until the launch has a few workgroups per CU
+    const size_t waves = ctx->moe_waves >= 8 ? 8 : 4, units = (L.row_blocks + 1) / 2;
+    const size_t groups = (units + waves - 1) / waves;
+    size_t nks = 1;
+    if (ctx->decode_ksplit > 0) {
+        nks = (size_t)ctx->decode_ksplit;
+    } else if (ctx->decode_ksplit == 0) {
+        // only while the launch has fewer workgroups than CUs: the 27B down projection (40 unit groups) runs 8 slices
+        // (78 -> 22 us at t = 32), the wide gate|up (272 groups) none (slices cost it 1-3 us, measured)
+        while (groups * segs * nks < (size_t)std::max(ctx->cu_count, 1) && nks < 8) nks *= 2;
+    }
+    // the grid covers exactly `segs` segments, so the "padded total" may be the constant no segment start reaches
+    return launch_moe_gemm(ctx, E, false, x_dev, t, 1, y_dev, out_f16, 0, t, block, segs, S.iota, S.zeros, S.always, nks);
 }
 
 // Direct mode for decode steps: no alignment pass.  The gate|up GEMM runs one segment per slot — the segment table is

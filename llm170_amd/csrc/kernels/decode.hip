@@ -223,6 +223,10 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
         for (int rb = 0; rb < RB; rb++)
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, acc[rb]), wr, mine + rb * 1024u, ky * slice, DEV);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores have reached memory before the ticket is drawn
+        // ... and the tiles stay in their registers until then: a 16-byte buffer store with a register scalar offset
+        // reads its data after issue, and the compiler models no hazard for that form
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) asm volatile("" ::"v"(acc[rb]));
         int ticket = 0;
         if (lane == 0) ticket = __hip_atomic_fetch_add(tickets + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         ticket = __builtin_amdgcn_readfirstlane(ticket);

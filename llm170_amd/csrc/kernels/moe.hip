@@ -111,14 +111,16 @@ __device__ __forceinline__ void moe_store(f4_t a0, f4_t a1, int slot, int q, int
 //   y: GLU -> f16 [ns][n/2]; LIN -> f16 or f32 [ns][n].  topw: null or f32 [ns] (LIN only).
 //   sorted_ids[seg*blk + i]: slot id or the sentinel ns; expert_ids[seg]; num_post[0] = padded slot total.
 //   A segment whose expert id is outside 0..n_exp-1 is skipped (its slots stay unwritten).
+//   ws / tickets: workspace and zeroed counters of a launch split over k across workgroups (gridDim.y slices; the
+//   LDS-staged kernel only): [slice][block][wave][2*TT] partial tiles, one counter per (block, wave).
 #define MOE_PARAMS                                                                                                  \
     const char *__restrict__ qa, const char *__restrict__ sa, unsigned long long q_stride,                          \
         unsigned long long s_stride, const uint16_t *__restrict__ x, int x_rows, int x_div, void *__restrict__ y,   \
         int y_f16, const float *__restrict__ topw, const int *__restrict__ sorted_ids,                              \
         const int *__restrict__ expert_ids, const int *__restrict__ num_post, int blk, int ns, int row_blocks, int k, \
-        int n, int n_exp
+        int n, int n_exp, f4_t *ws, int *tickets
 #define MOE_ARGS \
-    qa, sa, q_stride, s_stride, x, x_rows, x_div, y, y_f16, topw, sorted_ids, expert_ids, num_post, blk, ns, row_blocks, k, n, n_exp
+    qa, sa, q_stride, s_stride, x, x_rows, x_div, y, y_f16, topw, sorted_ids, expert_ids, num_post, blk, ns, row_blocks, k, n, n_exp, ws, tickets
 
 // ---------------------------------------------------------------------------------------------------- moe_dec
 template <int RB, int XL>
@@ -393,8 +395,12 @@ struct MoeMmStage {
     u2_t s[RB];
 };
 
+#define MOE_MAX_KSPLIT 8  // k slices across workgroups; the host clamps to this
+
 // One block = (segment of blk = 16*TT slots, group of W units); wave w owns unit group*W + w over the whole k range.
-template <int G, bool SBF, bool GLU, int TT, int DEPTH>
+// KS: the launch may be split over k across workgroups (dense linears run as one expert; the expert FFN never splits, and
+// its kernels are built without the epilogue that costs them registers).
+template <int G, bool SBF, bool GLU, int TT, int DEPTH, bool KS>
 __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     extern __shared__ _Float16 xs[];  // [2][16*TT][MOE_LDX]
     constexpr int GPT = W4_TILE_K / G;
@@ -403,14 +409,16 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int units = GLU ? row_blocks >> 1 : (row_blocks + 1) >> 1;
     const int groups = (units + W - 1) / W;
-    const int seg = blockIdx.x / groups;
+    const int seg = blockIdx.x / groups, grp = blockIdx.x % groups;
     if (seg * blk >= num_post[0]) return;  // uniform for the block, before any barrier
-    const int u_raw = (blockIdx.x % groups) * W + wave;
+    const int u_raw = grp * W + wave;
     const bool active = u_raw < units;  // a surplus wave repeats the last unit and stores nothing
     const int u = min(u_raw, units - 1);
     const int e = __builtin_amdgcn_readfirstlane(expert_ids[seg]);
     if ((unsigned)e >= (unsigned)n_exp) return;  // uniform for the block, before any barrier
     const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
+    const int nks = KS ? (int)gridDim.y : 1, ky = KS ? (int)blockIdx.y : 0;  // k slices across workgroups
+    const int kt_lo = (kt_n * ky) / nks, kt_hi = (kt_n * (ky + 1)) / nks;
     const int c = lane & 15, q = lane >> 4;
     const int rbA = GLU ? u : 2 * u, rbB = GLU ? u + units : min(2 * u + 1, row_blocks - 1);
     const bool haveB = GLU || 2 * u + 1 < row_blocks;
@@ -439,7 +447,7 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
 #pragma unroll
         for (int p = 0; p < TT; p++)
             xreg[set][p] = __builtin_amdgcn_raw_buffer_load_b128(
-                xr, (kt < kt_n && xg_off[p] != W4_OOB) ? xg_off[p] + (unsigned)kt * (W4_TILE_K * 2u) : W4_OOB, 0, 0);
+                xr, (kt < kt_hi && xg_off[p] != W4_OOB) ? xg_off[p] + (unsigned)kt * (W4_TILE_K * 2u) : W4_OOB, 0, 0);
     };
     auto store_x = [&](int set, int buf) {
         _Float16* base = xs + buf * (ROWS * MOE_LDX);
@@ -455,7 +463,7 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
                               (unsigned)rbB * (unsigned)kg_n * 32u + sg + (unsigned)q * 8u};
     MoeMmStage<2> stage[DEPTH];
     auto load_w = [&](MoeMmStage<2>& s_, int kt) {
-        const bool live = kt < kt_n;
+        const bool live = kt < kt_hi;
 #pragma unroll
         for (int rb = 0; rb < 2; rb++)
             s_.q[rb] = __builtin_amdgcn_raw_buffer_load_b128(qr, live ? qoff[rb] + (unsigned)kt * 1024u : W4_OOB, 0, 2);
@@ -517,18 +525,18 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
         }
     };
 
-    // prologue: x tile 0 into LDS buffer 0, x tile 1 in registers, DEPTH weight stages in flight
-    load_x(0, 0);
-    load_x(1, 1);
+    // prologue: the slice's first x tile into LDS buffer 0, the second in registers, DEPTH weight stages in flight
+    load_x(0, kt_lo);
+    load_x(1, kt_lo + 1);
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) load_w(stage[d], d);
+    for (int d = 0; d < DEPTH; d++) load_w(stage[d], kt_lo + d);
     store_x(0, 0);
     __syncthreads();
-    for (int kt0 = 0; kt0 < kt_n; kt0 += DEPTH) {
+    for (int kt0 = kt_lo; kt0 < kt_hi; kt0 += DEPTH) {
 #pragma unroll
-        for (int d = 0; d < DEPTH; d++) {  // DEPTH is even: register set and LDS buffer of tile kt are kt & 1 = d & 1
+        for (int d = 0; d < DEPTH; d++) {  // DEPTH is even: register set and LDS buffer of the slice's i-th tile are i & 1 = d & 1
             const int kt = kt0 + d;
-            if (kt < kt_n) compute(stage[d], d & 1);
+            if (kt < kt_hi) compute(stage[d], d & 1);
             load_w(stage[d], kt + DEPTH);
             store_x((d + 1) & 1, (d + 1) & 1);  // tile kt+1, loaded an iteration ago, into the buffer tile kt-1 was read from
             load_x(d & 1, kt + 2);              // out of range past the last tile: zeros, no traffic
@@ -537,6 +545,51 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     }
 
     if (!active) return;
+    if (KS && nks > 1) {
+        // every wave on its own: park the partial tiles (device-scope stores), draw the (block, wave) ticket, and the
+        // wave that draws the last one adds the slices in slice order and stores (see the dense decode kernel)
+        constexpr unsigned PER_WAVE = 2u * TT * 1024u;
+        const unsigned per_slice = gridDim.x * (unsigned)W * PER_WAVE;
+        const __amdgpu_buffer_rsrc_t wr = w4_make_rsrc(ws, per_slice * (unsigned)nks);
+        const unsigned mine = (blockIdx.x * (unsigned)W + (unsigned)wave) * PER_WAVE + (unsigned)lane * 16u;
+        constexpr int DEV = 16;  // cache policy: device scope
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int tt = 0; tt < TT; tt++)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, acc[rb][tt]), wr,
+                                                       mine + (unsigned)(rb * TT + tt) * 1024u, ky * per_slice, DEV);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // The tiles stay in their registers until the stores have completed: a 16-byte buffer store with a register
+        // scalar offset reads its data after issue, and the compiler, which models no hazard for that form, otherwise
+        // reuses the first data register in the very next instruction (seen as one wrong dword in the last lanes).
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int tt = 0; tt < TT; tt++) asm volatile("" ::"v"(acc[rb][tt]));
+        int ticket = 0;
+        int* const tk = tickets + blockIdx.x * W + wave;
+        if (lane == 0) ticket = __hip_atomic_fetch_add(tk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ticket = __builtin_amdgcn_readfirstlane(ticket);
+        if (ticket != nks - 1) return;
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int tt = 0; tt < TT; tt++) {
+                f4_t part[MOE_MAX_KSPLIT];  // all slices in flight at once; slices past nks: zero-length descriptor, zeros
+#pragma unroll
+                for (int s_ = 0; s_ < MOE_MAX_KSPLIT; s_++)
+                    part[s_] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                                            s_ < nks ? wr : w4_make_rsrc(ws, 0u),
+                                                            mine + (unsigned)(rb * TT + tt) * 1024u, s_ * per_slice, DEV));
+                f4_t sum = part[0];
+#pragma unroll
+                for (int s_ = 1; s_ < MOE_MAX_KSPLIT; s_++) sum += part[s_];
+                acc[rb][tt] = sum;
+            }
+        if (lane == 0) __hip_atomic_store(tk, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
         const int slot = sorted_ids[seg * blk + tt * 16 + c];
@@ -550,23 +603,27 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     extern "C" __global__ __launch_bounds__(512) void NAME(MOE_PARAMS) {              \
         moe_dec_body<G, SBF, GLU, XL, DEPTH>(MOE_ARGS);                               \
     }
-#define MOE_MM_KERNEL(NAME, G, SBF, GLU, TT, DEPTH)                                   \
+#define MOE_MM_KERNEL(NAME, G, SBF, GLU, TT, DEPTH, KS)                               \
     extern "C" __global__ __launch_bounds__(512) void NAME(MOE_PARAMS) {              \
-        moe_mm_body<G, SBF, GLU, TT, DEPTH>(MOE_ARGS);                                \
+        moe_mm_body<G, SBF, GLU, TT, DEPTH, KS>(MOE_ARGS);                            \
     }
 #define MOE_FAMILY(PFX, G, SBF, DMM)                             \
     MOE_DEC_KERNEL(PFX##_dec_glu_x1, G, SBF, true, 1, 4)     \
     MOE_DEC_KERNEL(PFX##_dec_glu_x4, G, SBF, true, 4, 3)     \
     MOE_DEC_KERNEL(PFX##_dec_lin_x1, G, SBF, false, 1, 4)    \
     MOE_DEC_KERNEL(PFX##_dec_lin_x4, G, SBF, false, 4, 3)    \
-    MOE_MM_KERNEL(PFX##_mm_glu_t1, G, SBF, true, 1, DMM)       \
-    MOE_MM_KERNEL(PFX##_mm_glu_t2, G, SBF, true, 2, DMM)       \
-    MOE_MM_KERNEL(PFX##_mm_glu_t3, G, SBF, true, 3, DMM)       \
-    MOE_MM_KERNEL(PFX##_mm_glu_t4, G, SBF, true, 4, DMM)       \
-    MOE_MM_KERNEL(PFX##_mm_lin_t1, G, SBF, false, 1, DMM)      \
-    MOE_MM_KERNEL(PFX##_mm_lin_t2, G, SBF, false, 2, DMM)      \
-    MOE_MM_KERNEL(PFX##_mm_lin_t3, G, SBF, false, 3, DMM)      \
-    MOE_MM_KERNEL(PFX##_mm_lin_t4, G, SBF, false, 4, DMM)
+    MOE_MM_KERNEL(PFX##_mm_glu_t1, G, SBF, true, 1, DMM, false)    \
+    MOE_MM_KERNEL(PFX##_mm_glu_t2, G, SBF, true, 2, DMM, false)    \
+    MOE_MM_KERNEL(PFX##_mm_glu_t3, G, SBF, true, 3, DMM, false)    \
+    MOE_MM_KERNEL(PFX##_mm_glu_t4, G, SBF, true, 4, DMM, false)    \
+    MOE_MM_KERNEL(PFX##_mm_lin_t1, G, SBF, false, 1, DMM, false)   \
+    MOE_MM_KERNEL(PFX##_mm_lin_t2, G, SBF, false, 2, DMM, false)   \
+    MOE_MM_KERNEL(PFX##_mm_lin_t3, G, SBF, false, 3, DMM, false)   \
+    MOE_MM_KERNEL(PFX##_mm_lin_t4, G, SBF, false, 4, DMM, false)   \
+    MOE_MM_KERNEL(PFX##_mm_lin_t1_ks, G, SBF, false, 1, DMM, true) \
+    MOE_MM_KERNEL(PFX##_mm_lin_t2_ks, G, SBF, false, 2, DMM, true) \
+    MOE_MM_KERNEL(PFX##_mm_lin_t3_ks, G, SBF, false, 3, DMM, true) \
+    MOE_MM_KERNEL(PFX##_mm_lin_t4_ks, G, SBF, false, 4, DMM, true)
 
 MOE_FAMILY(w4a16_moe_g32_f16, 32, false, 2)
 MOE_FAMILY(w4a16_moe_g32_bf16, 32, true, 2)

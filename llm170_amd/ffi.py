@@ -7,7 +7,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG, "libw4a16hip.so")
 
 ERR_SHAPE, ERR_SYMBOL, ERR_UNSUPPORTED, ERR_NOT_FOUND, ERR_ARG, ERR_ASSET = 10001, 10002, 10003, 10004, 10005, 10006
-PATH_AUTO, PATH_LANE, PATH_DECODE, PATH_PREFILL = 0, 1, 2, 3
+PATH_AUTO, PATH_LANE, PATH_DECODE, PATH_PREFILL, PATH_STREAM = 0, 1, 2, 3, 4
 
 
 class W4a16Error(RuntimeError):

@@ -15,7 +15,7 @@ import ctypes as C
 import numpy as np
 
 from . import ffi
-from .ffi import PATH_AUTO, PATH_DECODE, PATH_LANE, PATH_PREFILL, W4a16Error  # noqa: F401
+from .ffi import PATH_AUTO, PATH_DECODE, PATH_LANE, PATH_PREFILL, PATH_STREAM, W4a16Error  # noqa: F401
 
 
 def check_shapes(t, qlen, slen, xlen, n, k, group):

@@ -253,7 +253,40 @@ def test_prefill_matches_oracle(dec, orc, n, k, group, t, bf16):
     got16 = _device_forward(dec, "pf", x, t, ops.PATH_PREFILL, out_f16=True)
     assert np.array_equal(got16, gen.f32_to_f16_bits(got))
     auto = _device_forward(dec, "pf", x, t, ops.PATH_AUTO)
-    assert np.array_equal(_bits(auto), _bits(got))  # t > 16 routes to the prefill kernel
+    if t > 64:
+        assert np.array_equal(_bits(auto), _bits(got))  # more than 64 rows route to the prefill kernel
+    else:
+        stream = _device_forward(dec, "pf", x, t, ops.PATH_STREAM)
+        assert np.array_equal(_bits(auto), _bits(stream))  # 17..64 rows route to the streaming kernel
+        parity.assert_close(stream, want, "stream n%d k%d g%d t%d" % (n, k, group, t))
+
+
+@pytest.mark.parametrize("n,k,group,bf16", [(416, 1024, 128, False), (1536, 2048, 32, False), (200, 256, 128, True),
+                                            (5120, 5120, 128, False)])
+@pytest.mark.parametrize("t", [17, 32, 33, 48, 64, 100])
+def test_stream_path_matches_oracle(dec, orc, n, k, group, bf16, t):
+    """A few dozen rows: the grouped kernel run on the dense linear as its one expert (x shared through LDS, segments
+    of up to 64 rows, k slices across workgroups when the output is narrow).  f32 and f16 outputs, any t."""
+    say("stream", n, k, group, bf16, t)
+    q, s, x = gen.make_linear(n, k, group, t, seed=61)
+    if bf16:
+        s = (gen.f16_bits_to_f32(s).view(np.uint32) >> 16).astype(np.uint16)
+    dec.upload_lin_g("st", q, s, n, k, group, bf16)
+    if n * t <= 1 << 18:
+        want = orc.gemm_lane(x, t, q, s, n, k, group, scale_bf16=bf16, threads=16)
+    else:
+        want = _device_forward(dec, "st", x, t, ops.PATH_LANE)  # the bit-exact device twin of the oracle
+    got = _device_forward(dec, "st", x, t, ops.PATH_STREAM)
+    m = parity.assert_close(got, want, "stream n%d k%d g%d t%d" % (n, k, group, t))
+    say("   ", {a: m[a] for a in ("rel_l2", "max_ulp", "max_ulp_strict", "strict_pass_frac", "clamped")})
+    assert np.array_equal(_device_forward(dec, "st", x, t, ops.PATH_STREAM, out_f16=True), gen.f32_to_f16_bits(got))
+    assert np.array_equal(_bits(got), _bits(_device_forward(dec, "st", x, t, ops.PATH_STREAM)))  # same bits every run
+    try:
+        for ks in (-1, 2, 5):
+            dec.set_decode_ksplit(ks)
+            parity.assert_close(_device_forward(dec, "st", x, t, ops.PATH_STREAM), want, "stream ksplit %d" % ks)
+    finally:
+        dec.set_decode_ksplit(0)
 
 
 @pytest.mark.parametrize("n,k,t", [(34816, 5120, 512), (5120, 17408, 512), (34816, 5120, 4096)])
@@ -311,3 +344,6 @@ def test_prefill_refuses_irregular_scales_and_auto_falls_back(dec, orc):
     assert e.value.code == ffi.ERR_UNSUPPORTED
     want = orc.gemm_lane(x, t, q, s, n, k, group, threads=8)
     parity.assert_close(_device_forward(dec, "irr", x, t, ops.PATH_AUTO), want, "auto fallback")
+    x_long = np.concatenate([x, x, x, x, x])[:170]  # beyond 64 rows the fallback is the streaming kernel as well
+    parity.assert_close(_device_forward(dec, "irr", x_long, 170, ops.PATH_AUTO),
+                        orc.gemm_lane(x_long, 170, q, s, n, k, group, threads=8), "auto fallback, 170 rows")
