@@ -80,6 +80,10 @@ static const char* const kMoeSyms[] = {W4_MOE_FAMILY("w4a16_moe_g32_f16"),
                                        "w4a16_moe_g32_bf16_down_sum",
                                        "w4a16_moe_g128_f16_down_sum",
                                        "w4a16_moe_g128_bf16_down_sum",
+                                       "w4a16_moe_g32_f16_down_sum1",
+                                       "w4a16_moe_g32_bf16_down_sum1",
+                                       "w4a16_moe_g128_f16_down_sum1",
+                                       "w4a16_moe_g128_bf16_down_sum1",
                                        "w4a16_moe_topk_t",
                                        "w4a16_moe_align",
                                        "w4a16_moe_topk_sum_f16",

@@ -344,14 +344,17 @@ static int moe_ffn_direct(w4a16_ctx* ctx, const char* name, const W4Experts& E, 
     // gate|up with the SiLU*up epilogue, one slot per segment
     W4_TRY(launch_moe_gemm(ctx, E, true, x_dev, t, top_k, S.act, 1, 0, ns, 1, ns, S.iota, idx_dev, S.always));
     // down + routing weight + f16 rounding + slot-order sum
-    const size_t row_blocks = (E.h + 15) / 16, units = (row_blocks + 1) / 2;
+    // units of one row block while units of two would leave CUs without a workgroup
+    const size_t row_blocks = (E.h + 15) / 16;
+    const size_t rbu = (ctx->moe_waves == 2 || (ctx->moe_waves == 0 && t * ((row_blocks + 1) / 2) < (size_t)std::max(ctx->cu_count, 1))) ? 1 : 2;
+    const size_t units = (row_blocks + rbu - 1) / rbu;
     uint64_t qa = E.q2, sa = E.s2;
     unsigned long long qs = E.q2_stride, ss = E.s2_stride;
     int tk = (int)top_k, nsi = (int)ns, rbi = (int)row_blocks, ki = (int)E.n_ff, ni = (int)E.h, nei = (int)E.n_exp;
     void* p[] = {&qa, &sa, &qs, &ss, &S.act, &idx_dev, &wt_dev, &y_dev, &tk, &nsi, &rbi, &ki, &ni, &nei};
     char sym[80];
-    snprintf(sym, sizeof sym, "w4a16_moe_g%zu_%s_down_sum", E.group, E.scale_bf16 ? "bf16" : "f16");
-    return w4_launch(ctx, sym, (unsigned)(t * units), 1, (unsigned)(top_k * 64), (unsigned)(top_k * 2 * 64 * 16), p);
+    snprintf(sym, sizeof sym, "w4a16_moe_g%zu_%s_down_sum%s", E.group, E.scale_bf16 ? "bf16" : "f16", rbu == 1 ? "1" : "");
+    return w4_launch(ctx, sym, (unsigned)(t * units), 1, (unsigned)(top_k * 64), (unsigned)(top_k * rbu * 64 * 16), p);
 }
 
 extern "C" int w4a16_moe_ffn(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t idx_dev, uint64_t wt_dev,

@@ -257,17 +257,18 @@ __device__ __forceinline__ void moe_dec_body(MOE_PARAMS) {
 // rounds to f16 exactly as the staged path materialises c2; wave 0 then adds the waves' values in slot order in f32
 // (the same order as the separate sum kernel) and writes y f32 [t][n].  No alignment pass is needed: the expert of
 // a slot is read straight from idx.
-template <int G, bool SBF, int DEPTH>
+// RB: row blocks of a workgroup's unit — 2, or 1 for a handful of tokens, when units of two leave most CUs without work.
+template <int G, bool SBF, int DEPTH, int RB>
 __device__ __forceinline__ void moe_down_sum_body(const char* __restrict__ qa, const char* __restrict__ sa,
                                                   unsigned long long q_stride, unsigned long long s_stride,
                                                   const uint16_t* __restrict__ act, const int* __restrict__ idx,
                                                   const float* __restrict__ topw, float* __restrict__ y, int top_k,
                                                   int ns, int row_blocks, int k, int n, int n_exp) {
-    extern __shared__ f4_t red[];  // [top_k][2][64]
+    extern __shared__ f4_t red[];  // [top_k][RB][64]
     constexpr int GPT = W4_TILE_K / G;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int units = (row_blocks + 1) >> 1;
+    const int units = (row_blocks + RB - 1) / RB;
     const int token = blockIdx.x / units, u = blockIdx.x % units;
     const int slot = token * top_k + wave;
     const int e_raw = __builtin_amdgcn_readfirstlane(idx[slot]);
@@ -275,8 +276,8 @@ __device__ __forceinline__ void moe_down_sum_body(const char* __restrict__ qa, c
     const int e = valid ? e_raw : 0;
     const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
     const int m = lane & 15, g = lane >> 4;
-    const int rbA = 2 * u, rbB = min(2 * u + 1, row_blocks - 1);
-    const bool haveB = 2 * u + 1 < row_blocks;
+    const int rbA = RB * u, rbB = min(RB * u + 1, row_blocks - 1);
+    const bool haveB = RB == 2 && 2 * u + 1 < row_blocks;
 
     const __amdgpu_buffer_rsrc_t qr = w4_make_rsrc(qa + (unsigned long long)e * q_stride,
                                                    valid ? (unsigned)row_blocks * (unsigned)kt_n * 1024u : 0u);
@@ -290,27 +291,29 @@ __device__ __forceinline__ void moe_down_sum_body(const char* __restrict__ qa, c
     const unsigned sg = G == 32 ? (unsigned)(lane & 3) * 32u : 0u;
     const unsigned soff[2] = {(unsigned)rbA * (unsigned)kg_n * 32u + sg + (unsigned)g * 8u,
                               (unsigned)rbB * (unsigned)kg_n * 32u + sg + (unsigned)g * 8u};
-    f4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    f4_t acc[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) acc[rb] = (f4_t){0.f, 0.f, 0.f, 0.f};
 
-    MoeDecStage<2, 1> stage[DEPTH];
-    auto load = [&](MoeDecStage<2, 1>& s_, int kt) {
+    MoeDecStage<RB, 1> stage[DEPTH];
+    auto load = [&](MoeDecStage<RB, 1>& s_, int kt) {
         const bool live = kt < kt_n;
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++)
+        for (int rb = 0; rb < RB; rb++)
             s_.q[rb] = __builtin_amdgcn_raw_buffer_load_b128(qr, live ? qoff[rb] + (unsigned)kt * 1024u : W4_OOB, 0, 2);
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++)
+        for (int rb = 0; rb < RB; rb++)
             s_.s[rb] = __builtin_amdgcn_raw_buffer_load_b64(sr, live ? soff[rb] + (unsigned)kt * (GPT * 32u) : W4_OOB, 0, 0);
         s_.x[0] = __builtin_amdgcn_raw_buffer_load_b128(xr, live ? xoff + (unsigned)(kt * W4_TILE_K) * 2u : W4_OOB, 0, 0);
     };
-    auto compute = [&](const MoeDecStage<2, 1>& s_) {
+    auto compute = [&](const MoeDecStage<RB, 1>& s_) {
         u4_t xb[4];
         xb[0] = s_.x[0];
         xb[1] = moe_row_shl<4>(s_.x[0]);
         xb[2] = moe_row_shl<8>(s_.x[0]);
         xb[3] = moe_row_shl<12>(s_.x[0]);
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++) {
+        for (int rb = 0; rb < RB; rb++) {
             const f4_t zero = {0.f, 0.f, 0.f, 0.f};
             if (G == 128) {
                 f4_t part = zero;
@@ -348,20 +351,22 @@ __device__ __forceinline__ void moe_down_sum_body(const char* __restrict__ qa, c
     // c2 of this slot: routing weight, one rounding to f16 (the value the staged path stores), back to f32
     const float wgt = topw[slot];
 #pragma unroll
-    for (int rb = 0; rb < 2; rb++)
+    for (int rb = 0; rb < RB; rb++) {
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[rb][i] = moe_round_f16(acc[rb][i] * wgt);
-    red[(wave * 2 + 0) * 64 + lane] = acc[0];
-    red[(wave * 2 + 1) * 64 + lane] = acc[1];
+        red[(wave * RB + rb) * 64 + lane] = acc[rb];
+    }
     __syncthreads();
     if (wave != 0 || m != 0) return;
-    f4_t sum[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    f4_t sum[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) sum[rb] = (f4_t){0.f, 0.f, 0.f, 0.f};
     for (int w = 0; w < top_k; w++) {
-        sum[0] += red[(w * 2 + 0) * 64 + lane];
-        sum[1] += red[(w * 2 + 1) * 64 + lane];
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) sum[rb] += red[(w * RB + rb) * 64 + lane];
     }
 #pragma unroll
-    for (int rb = 0; rb < 2; rb++) {
+    for (int rb = 0; rb < RB; rb++) {
         if (rb == 1 && !haveB) break;
         const int row = (rb == 0 ? rbA : rbB) * 16 + 4 * g;
         float* yo = y + (size_t)token * n + row;
@@ -375,18 +380,22 @@ __device__ __forceinline__ void moe_down_sum_body(const char* __restrict__ qa, c
     }
 }
 
-#define MOE_DOWN_SUM_KERNEL(NAME, G, SBF)                                                                         \
+#define MOE_DOWN_SUM_KERNEL(NAME, G, SBF, RB)                                                                     \
     extern "C" __global__ __launch_bounds__(512) void NAME(                                                       \
         const char* qa, const char* sa, unsigned long long q_stride, unsigned long long s_stride,                 \
         const uint16_t* act, const int* idx, const float* topw, float* y, int top_k, int ns, int row_blocks, int k, \
         int n, int n_exp) {                                                                                       \
-        moe_down_sum_body<G, SBF, 3>(qa, sa, q_stride, s_stride, act, idx, topw, y, top_k, ns, row_blocks, k, n,  \
-                                     n_exp);                                                                      \
+        moe_down_sum_body<G, SBF, 3, RB>(qa, sa, q_stride, s_stride, act, idx, topw, y, top_k, ns, row_blocks, k, \
+                                         n, n_exp);                                                               \
     }
-MOE_DOWN_SUM_KERNEL(w4a16_moe_g32_f16_down_sum, 32, false)
-MOE_DOWN_SUM_KERNEL(w4a16_moe_g32_bf16_down_sum, 32, true)
-MOE_DOWN_SUM_KERNEL(w4a16_moe_g128_f16_down_sum, 128, false)
-MOE_DOWN_SUM_KERNEL(w4a16_moe_g128_bf16_down_sum, 128, true)
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g32_f16_down_sum, 32, false, 2)
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g32_bf16_down_sum, 32, true, 2)
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g128_f16_down_sum, 128, false, 2)
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g128_bf16_down_sum, 128, true, 2)
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g32_f16_down_sum1, 32, false, 1)
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g32_bf16_down_sum1, 32, true, 1)
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g128_f16_down_sum1, 128, false, 1)
+MOE_DOWN_SUM_KERNEL(w4a16_moe_g128_bf16_down_sum1, 128, true, 1)
 
 // ---------------------------------------------------------------------------------------------------- moe_mm
 template <int RB>
