@@ -176,6 +176,9 @@ int w4a16_set_decode_ksplit(w4a16_ctx* ctx, int ksplit);
  * idle — narrow outputs at moderate t; the reference's prefill path makes the same choice inside its vendored GEMM),
  * -1 = never, n >= 1 = exactly n k slices (clamped so a slice has at least 4 k tiles). */
 int w4a16_set_prefill_ksplit(w4a16_ctx* ctx, int ksplit);
+/* Rows of the prefill kernel's block tile: 0 = automatic (64 up to 192 rows, else 128), 64 or 128.  The reference's
+ * vendored GEMM picks its thread-block shape per problem the same way (marlin_gemm_try, kernels/marlin.rs:94-213). */
+int w4a16_set_prefill_tile(w4a16_ctx* ctx, int rows);
 
 /* run_bench_gemv / run_bench_gemm (crates/server/src/probes/w4a16/gpu/bench.rs:366-433): `warmup` untimed then
  * `reps` timed back-to-back lin_forward launches on the launch stream, one synchronisation at the end.  Launch i

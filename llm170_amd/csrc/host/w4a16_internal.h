@@ -73,6 +73,7 @@ struct w4a16_ctx {
     uint64_t decode_ws = 0, decode_tickets = 0;                 // partial tiles and per-block tickets of a split launch
     size_t decode_ws_cap = 0, decode_tickets_cap = 0;
     int prefill_ksplit = 0;                                     // 0 = automatic, -1 = never, n = exactly n slices
+    int prefill_tile_m = 0;                                     // 0 = automatic, 64 or 128 rows per block tile
     uint64_t prefill_ws = 0;                                    // f32 partials of a split-K prefill launch
     size_t prefill_ws_cap = 0;
     int cu_count = 0;

@@ -142,10 +142,31 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
         return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has a zero or non-finite scale (use the decode path)");
     if (t * L.k * 2 >= 0x80000000ull || L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
         return w4_fail(W4A16_ERR_SHAPE, "prefill: x or the tiled weights reach 2 GiB, beyond the buffer-descriptor range");
-    // block tile 128 (m) x 256 (n); 8 x 8 super-tiles dealt round-robin to the 8 XCDs (kernels/prefill.hip)
+    // Block tile 128 x 256 (two workgroups per CU) or 64 x 256 (three per CU, 64 accumulator registers).  The 64-row
+    // tile pads less, makes twice as many workgroups and loses about 15 % per row to unpacking each weight for half as
+    // many rows; which one finishes first is mostly a matter of how the workgroups divide into the slots of the chip,
+    // so both are priced — (generations of workgroups) x (k tiles per slice) x (relative tile time) — and the cheaper
+    // one runs (sweeps over the 27B shapes, t = 65..4096: within ~5 % of the better tile everywhere).
+    const size_t tiles_n = (L.n + 255) / 256, kt_n = L.k / 128, cus = (size_t)std::max(ctx->cu_count, 1);
+    auto slices_for = [&](size_t tiles, size_t slots) {
+        size_t nks = 1;
+        if (ctx->prefill_ksplit > 0) {
+            nks = (size_t)ctx->prefill_ksplit;
+        } else if (ctx->prefill_ksplit == 0 && L.n % 4 == 0) {
+            while (tiles * nks * 20 < slots * 9 && nks < 8) nks *= 2;  // until ~45 % of the slots (see below)
+        }
+        return std::max<size_t>(1, std::min(nks, kt_n / 4));
+    };
+    auto price = [&](size_t rows) {
+        const size_t slots = cus * (rows == 64 ? 3 : 2), tiles = ((t + rows - 1) / rows) * tiles_n;
+        const size_t nks = slices_for(tiles, slots);
+        return (double)((tiles * nks + slots - 1) / slots) * (double)((kt_n + nks - 1) / nks) * (rows == 64 ? 0.85 : 1.0);
+    };
+    const size_t bm = ctx->prefill_tile_m ? (size_t)ctx->prefill_tile_m : (price(64) <= price(128) ? 64 : 128);
+    const size_t slots = cus * (bm == 64 ? 3 : 2);
+    const size_t tiles_m = (t + bm - 1) / bm;
     // Super-tile shape: up to 8 tiles along m; along n the width in {8, 4, 2, 1} that leaves the busiest XCD with the
     // fewest tiles (super-tiles are dealt round-robin to the 8 XCDs), the wider one on ties for L2 reuse.
-    const size_t tiles_m = (t + 127) / 128, tiles_n = (L.n + 255) / 256;
     const size_t sup_m = std::min<size_t>(8, tiles_m), sm_n = (tiles_m + sup_m - 1) / sup_m;
     size_t sup_n = 8, supers = 0, best_load = ~(size_t)0;
     for (size_t cand : {8, 4, 2, 1}) {
@@ -157,26 +178,21 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
         }
     }
     const size_t grid = ((supers + 7) / 8) * (sup_m * sup_n) * 8;
-    // Split-K when the tile grid alone leaves much of the chip idle (two workgroups fit a CU: 512 slots): k slices are
-    // doubled until the launch has at least 512 workgroups (measured best at the 27B down projection: 8 slices at
-    // t = 512, 4 at t = 1024), each slice at least 4 k tiles.  Partials are f32 in a context-owned workspace, added in
-    // slice order by a second launch (deterministic).
-    const size_t tiles = tiles_m * tiles_n, kt_n = L.k / 128;
-    size_t nks = 1;
-    if (ctx->prefill_ksplit > 0) {
-        nks = (size_t)ctx->prefill_ksplit;
-    } else if (ctx->prefill_ksplit == 0 && L.n % 4 == 0) {
-        while (tiles * nks < 512 && nks < 8) nks *= 2;
-    }
-    nks = std::max<size_t>(1, std::min(nks, kt_n / 4));
+    // Split-K when the tile grid alone leaves much of the chip idle: k slices are doubled until the launch has about
+    // 45 % as many workgroups as the chip holds at once (sweeps over the 27B shapes at t = 65..1024: more slices than
+    // that cost more in partial-sum traffic than they gain; e.g. gate|up at t = 384 runs 141 us unsplit, 173 us in two
+    // slices), each slice at least 4 k tiles.  Partials are f32 in a context-owned workspace, added in slice order by a
+    // second launch (deterministic).
+    const size_t nks = slices_for(tiles_m * tiles_n, slots);
     char sym[64];
-    snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s", L.group, L.scale_bf16 ? "bf16" : "f16");
+    snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s%s", L.group, L.scale_bf16 ? "bf16" : "f16", bm == 64 ? "_m64" : "");
+    const unsigned shmem = (unsigned)(2 * bm * 64 * 2);
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
     int spm = (int)sup_m, spn = (int)sup_n;
     if (nks == 1) {
         void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &spm, &spn};
-        return w4_launch(ctx, sym, (unsigned)grid, 1, 256, 2 * 128 * 64 * 2, params);
+        return w4_launch(ctx, sym, (unsigned)grid, 1, 256, shmem, params);
     }
     if (L.n % 4 != 0) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: split-K needs n %% 4 == 0");
     const size_t count = t * L.n;
@@ -184,7 +200,7 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     uint64_t ws = ctx->prefill_ws;
     int zero = 0;
     void* params[] = {&qt, &st, &x, &ws, &row_blocks, &ki, &ni, &ti, &zero, &spm, &spn};
-    W4_TRY(w4_launch(ctx, sym, (unsigned)grid, (unsigned)nks, 256, 2 * 128 * 64 * 2, params));
+    W4_TRY(w4_launch(ctx, sym, (unsigned)grid, (unsigned)nks, 256, shmem, params));
     int nksi = (int)nks;
     size_t cnt = count;
     void* rp[] = {&ws, &y, &nksi, &cnt, &of};
@@ -493,6 +509,13 @@ extern "C" int w4a16_set_decode_shape(w4a16_ctx* ctx, int rows_per_wave, int wav
         return w4_fail(W4A16_ERR_ARG, "set_decode_shape: rows_per_wave in {0,16,32,64}, waves_per_block in 0..8");
     ctx->decode_rows_per_wave = rows_per_wave;
     ctx->decode_waves_per_block = waves_per_block;
+    return 0;
+}
+
+extern "C" int w4a16_set_prefill_tile(w4a16_ctx* ctx, int rows) {
+    if (!ctx) return w4_fail(W4A16_ERR_ARG, "set_prefill_tile: null context");
+    if (rows != 0 && rows != 64 && rows != 128) return w4_fail(W4A16_ERR_ARG, "set_prefill_tile: 0 = automatic, 64 or 128 rows");
+    ctx->prefill_tile_m = rows;
     return 0;
 }
 

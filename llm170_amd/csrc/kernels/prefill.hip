@@ -20,25 +20,24 @@
 //     that all eight XCDs get work).
 #include "w4a16_common.hpp"
 
-#ifndef PF_WM
-#define PF_WM 1           // waves along m (1: block tile 128 x 256, 4 waves; 2: 256 x 256, 8 waves)
-#endif
-#define PF_BM (128 * PF_WM)
 #define PF_BN 256
 #define PF_KS 64          // k per LDS stage
 #define PF_LDA 64         // halves per staged x row (unpadded; chunks swizzled)
-#define PF_STAGE_BYTES (PF_BM * PF_LDA * 2)
-#define PF_THREADS (256 * PF_WM)
+#define PF_THREADS 256
 
-template <int G, bool SBF>
+// MI = 32-row MFMA tiles along m per wave: 4 (block tile 128 x 256, 128 accumulator registers, two workgroups per CU) or
+// 2 (64 x 256, 64 registers, three workgroups per CU) for a few dozen to a couple of hundred rows, where 128-row tiles
+// would spend half their MFMAs on padding and leave too few workgroups.
+template <int G, bool SBF, int MI>
 __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                              const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
                                              int k, int n, int t, int out_f16, int sup_m, int sup_n) {
     extern __shared__ _Float16 lds[];  // 2 stages x [PF_BM][PF_LDA]
     constexpr int GPT = W4_TILE_K / G;
+    constexpr int PF_BM = 32 * MI, PF_STAGE_BYTES = PF_BM * PF_LDA * 2;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave % PF_WM, wn = wave / PF_WM;  // PF_WM x 4 waves
+    const int wn = wave;  // 4 waves along n
     const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
 
     // XCD-aware tile numbering.  Block b runs on XCD b % 8 and is the (b / 8)-th block of that XCD; consecutive
@@ -66,15 +65,15 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     // simply fetches that k chunk.  Rows >= t fetch out of range: zeros.
     typedef __attribute__((address_space(3))) char lds_char_t;
     lds_char_t* const lds_base = (lds_char_t*)lds;
-    unsigned xa_off[4];
+    unsigned xa_off[MI];  // PF_BM * 8 chunks over 256 threads
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < MI; i++) {
         const int c = tid + i * PF_THREADS, row = c >> 3, kc = (c & 7) ^ (row & 7);
         xa_off[i] = (m0 + row < t) ? ((unsigned)(m0 + row) * (unsigned)k + (unsigned)kc * 8u) * 2u : W4_OOB;
     }
     auto load_a = [&](int s, int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < MI; i++)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 xr, (__attribute__((address_space(3))) void*)(lds_base + buf * PF_STAGE_BYTES + (i * PF_THREADS + wave * 64) * 16),
                 16, xa_off[i], s * (PF_KS * 2), 0, 0);
@@ -106,16 +105,16 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
         }
     };
 
-    f16_t acc[4][2];
+    f16_t acc[MI][2];
 #pragma unroll
-    for (int mi = 0; mi < 4; mi++)
+    for (int mi = 0; mi < MI; mi++)
 #pragma unroll
         for (int ni = 0; ni < 2; ni++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[mi][ni][e] = 0.f;
     float unit[2] = {1.f, 1.f};  // scale the accumulator of sub-tile ni is currently expressed in
 
-    const int a_row = wm * 128 + nl;  // + mi * 32
+    const int a_row = nl;  // + mi * 32
     // split-K over gridDim.y (narrow outputs at moderate t, where the tile grid alone cannot fill the chip): this
     // block covers k tiles [kt_lo, kt_hi) and writes an f32 partial; a second launch adds the partials in order
     const int kt_lo = (kt_n * (int)blockIdx.y) / (int)gridDim.y, kt_hi = (kt_n * ((int)blockIdx.y + 1)) / (int)gridDim.y;
@@ -155,9 +154,9 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
 #pragma unroll
                     for (int ni = 0; ni < 2; ni++) unit[ni] = w4_scale_fast<SBF>(sc[ni][0]);
                 }
-                h8_t a[4];
+                h8_t a[MI];
 #pragma unroll
-                for (int mi = 0; mi < 4; mi++)
+                for (int mi = 0; mi < MI; mi++)
                     a[mi] = *reinterpret_cast<const h8_t*>(abuf + mi * 32 * PF_LDA + (((kbl * 2 + khalf) ^ (nl & 7)) * 8));
                 const bool last128 = G == 128 && kb == 7;  // branch free: the last k tile multiplies by 1
                 float next_ratio[2] = {1.f, 1.f};
@@ -174,7 +173,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
                 for (int ni = 0; ni < 2; ni++) {
                     const h8_t b = w4_deq8(bq[ni][h][w]);
 #pragma unroll
-                    for (int mi = 0; mi < 4; mi++) {
+                    for (int mi = 0; mi < MI; mi++) {
                         if (boundary32) acc[mi][ni] *= ratio[ni];
                         acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b, acc[mi][ni], 0, 0, 0);
                     }
@@ -183,7 +182,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
 #pragma unroll
                     for (int ni = 0; ni < 2; ni++)
 #pragma unroll
-                        for (int mi = 0; mi < 4; mi++) acc[mi][ni] *= next_ratio[ni];
+                        for (int mi = 0; mi < MI; mi++) acc[mi][ni] *= next_ratio[ni];
                 }
             }
             __syncthreads();
@@ -204,10 +203,10 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
         const int col = n0 + wn * 64 + ni * 32 + nl;
         if (col >= n) continue;
 #pragma unroll
-        for (int mi = 0; mi < 4; mi++) {
+        for (int mi = 0; mi < MI; mi++) {
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-                const int row = m0 + wm * 128 + mi * 32 + 8 * (e >> 2) + 4 * khalf + (e & 3);
+                const int row = m0 + mi * 32 + 8 * (e >> 2) + 4 * khalf + (e & 3);
                 if (row < t) {
                     const float v = acc[mi][ni][e] * unit[ni];
                     if (out_f16)
@@ -220,12 +219,11 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     }
 }
 
-#define PREFILL_KERNEL(NAME, G, SBF)                                                                               \
-    extern "C" __global__ __launch_bounds__(PF_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void NAME(const u4_t* qt, const uint16_t* st, \
-                                                                  const uint16_t* x, void* y, int row_blocks,      \
-                                                                  int k, int n, int t, int out_f16, int sup_m,     \
-                                                                  int sup_n) {                                     \
-        prefill_body<G, SBF>(qt, st, x, y, row_blocks, k, n, t, out_f16, sup_m, sup_n);                            \
+#define PREFILL_KERNEL(NAME, G, SBF, MI, WPE)                                                                      \
+    extern "C" __global__ __launch_bounds__(PF_THREADS) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(      \
+        const u4_t* qt, const uint16_t* st, const uint16_t* x, void* y, int row_blocks, int k, int n, int t,          \
+        int out_f16, int sup_m, int sup_n) {                                                                           \
+        prefill_body<G, SBF, MI>(qt, st, x, y, row_blocks, k, n, t, out_f16, sup_m, sup_n);                            \
     }
 
 // y[i] = sum over the nks partials of a split-K launch, added in split order in f32; f32 or f16 out.
@@ -244,7 +242,11 @@ extern "C" __global__ __launch_bounds__(256) void w4a16_prefill_splitk_sum(const
     }
 }
 
-PREFILL_KERNEL(w4a16_prefill_g128_f16, 128, false)
-PREFILL_KERNEL(w4a16_prefill_g128_bf16, 128, true)
-PREFILL_KERNEL(w4a16_prefill_g32_f16, 32, false)
-PREFILL_KERNEL(w4a16_prefill_g32_bf16, 32, true)
+PREFILL_KERNEL(w4a16_prefill_g128_f16, 128, false, 4, 2)
+PREFILL_KERNEL(w4a16_prefill_g128_bf16, 128, true, 4, 2)
+PREFILL_KERNEL(w4a16_prefill_g32_f16, 32, false, 4, 2)
+PREFILL_KERNEL(w4a16_prefill_g32_bf16, 32, true, 4, 2)
+PREFILL_KERNEL(w4a16_prefill_g128_f16_m64, 128, false, 2, 3)
+PREFILL_KERNEL(w4a16_prefill_g128_bf16_m64, 128, true, 2, 3)
+PREFILL_KERNEL(w4a16_prefill_g32_f16_m64, 32, false, 2, 3)
+PREFILL_KERNEL(w4a16_prefill_g32_bf16_m64, 32, true, 2, 3)

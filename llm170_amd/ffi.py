@@ -54,6 +54,7 @@ _SIGS = {
     "w4a16_lin_fuse": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_char_p), C.c_size_t, C.c_int]),
     "w4a16_set_decode_shape": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "w4a16_set_decode_ksplit": (C.c_int, [C.c_void_p, C.c_int]),
+    "w4a16_set_prefill_tile": (C.c_int, [C.c_void_p, C.c_int]),
     "w4a16_set_prefill_ksplit": (C.c_int, [C.c_void_p, C.c_int]),
     "w4a16_bench_forward": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.c_size_t, C.c_uint64, C.c_uint64, C.c_size_t,
                                       C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.POINTER(C.c_float),

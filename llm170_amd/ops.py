@@ -228,6 +228,10 @@ class W4a16Dec:
     def set_decode_shape(self, rows_per_wave=0, waves_per_block=0):
         ffi.check(self.cc.lib.w4a16_set_decode_shape(self.cc.h, rows_per_wave, waves_per_block))
 
+    def set_prefill_tile(self, rows=0):
+        """0 = automatic, 64 or 128 rows per block tile of the prefill kernel."""
+        ffi.check(self.cc.lib.w4a16_set_prefill_tile(self.cc.h, rows))
+
     def set_decode_ksplit(self, ksplit=0):
         """0 = automatic, -1 = never, n = exactly n k slices across workgroups."""
         ffi.check(self.cc.lib.w4a16_set_decode_ksplit(self.cc.h, ksplit))
