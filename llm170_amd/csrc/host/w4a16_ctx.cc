@@ -233,7 +233,16 @@ int w4_launch(w4a16_ctx* ctx, const char* symbol, unsigned gx, unsigned gy, unsi
     if (it == ctx->functions.end()) return w4_fail(W4A16_ERR_SYMBOL, "function: symbol %s is not loaded", symbol);
     if (gx == 0 || gy == 0 || block == 0 || block > 1024)
         return w4_fail(W4A16_ERR_ARG, "launch %s: grid %ux%u block %u", symbol, gx, gy, block);
-    hipError_t e = hipModuleLaunchKernel(it->second, gx, gy, 1, block, 1, 1, shmem, ctx->stream, params, nullptr);
+    hipError_t e = hipSuccess;
+    if (shmem > 64 * 1024) {  // beyond the default limit on dynamic LDS the function has to be told (gfx950: 160 KiB)
+        if (shmem > 160 * 1024) return w4_fail(W4A16_ERR_ARG, "launch %s: %u bytes of LDS", symbol, shmem);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(it->second), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)shmem);
+        if (e != hipSuccess)
+            return w4_fail((int)e, "hipFuncSetAttribute(%s, dynamic LDS %u): %s (%d)", symbol, shmem, hipGetErrorString(e),
+                           (int)e);
+    }
+    e = hipModuleLaunchKernel(it->second, gx, gy, 1, block, 1, 1, shmem, ctx->stream, params, nullptr);
     if (e != hipSuccess)
         return w4_fail((int)e, "hipModuleLaunchKernel(%s grid %ux%u block %u shmem %u): %s (%d)", symbol, gx, gy, block,
                        shmem, hipGetErrorString(e), (int)e);

@@ -181,7 +181,8 @@ extern "C" int w4a16_moe_align(w4a16_ctx* ctx, uint64_t idx_dev, size_t ns, size
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     int nsi = (int)ns, ni = (int)n_exp, bi = (int)block;
     void* p[] = {&idx_dev, &nsi, &ni, &bi, &sorted_dev, &expert_ids_dev, &num_post_dev};
-    return w4_launch(ctx, "w4a16_moe_align", 1, 1, 512, 0, p);
+    // LDS: 16 per-wave count rows, totals and offsets, one entry per expert each
+    return w4_launch(ctx, "w4a16_moe_align", 1, 1, 1024, (unsigned)((16 + 2) * n_exp * 4), p);
 }
 
 // ------------------------------------------------------------------------------------------------ FFN

@@ -699,22 +699,28 @@ extern "C" __global__ __launch_bounds__(256) void w4a16_moe_topk_t(const float* 
 }
 
 // Stable counting sort of slots by expert with every expert's run padded to a multiple of `block`
-// (assets/moe.cu:860-908 + 1599-1633 in one launch).  One workgroup of 512 threads, n_exp <= 1024.
+// (assets/moe.cu:860-908 + 1599-1633 in one launch).  One workgroup of 1024 threads, n_exp <= 1024.
 //   sorted_ids: slot ids in expert order, padding = sentinel ns; expert_ids[b]: expert of segment b;
 //   num_post[0] = padded total, num_post[1] = number of distinct experts hit.
 // Wave w owns the contiguous slot range [w*chunk, (w+1)*chunk): per-wave counts, an exclusive prefix over the
 // waves per expert, a two-level scan over the experts' padded counts, then every wave places its slots in order.
 // An out-of-range expert id is dropped (its slot is never placed).
-#define MOE_ALIGN_WAVES 8
-#define MOE_ALIGN_KEEP 8  // 64-slot steps of a wave whose expert ids stay in registers between the two passes
-extern "C" __global__ __launch_bounds__(512) void w4a16_moe_align(const int* __restrict__ idx, int ns, int n_exp,
-                                                                  int block, int* __restrict__ sorted_ids,
-                                                                  int* __restrict__ expert_ids, int* __restrict__ num_post) {
-    __shared__ unsigned cnt[MOE_ALIGN_WAVES][1024];  // per wave count, then exclusive prefix over the waves
-    __shared__ unsigned tot[1024], poff[1024];
+#define MOE_ALIGN_WAVES 16
+#define MOE_ALIGN_THREADS (64 * MOE_ALIGN_WAVES)
+#define MOE_ALIGN_KEEP 4  // 64-slot steps of a wave whose expert ids stay in registers between the two passes
+extern "C" __global__ __launch_bounds__(MOE_ALIGN_THREADS) void w4a16_moe_align(const int* __restrict__ idx, int ns,
+                                                                               int n_exp, int block,
+                                                                               int* __restrict__ sorted_ids,
+                                                                               int* __restrict__ expert_ids,
+                                                                               int* __restrict__ num_post) {
+    extern __shared__ unsigned align_lds[];  // cnt[WAVES][n_exp] (per wave count, then exclusive prefix over the waves),
+                                             // tot[n_exp], poff[n_exp]
+    unsigned* const cnt = align_lds;
+    unsigned* const tot = cnt + MOE_ALIGN_WAVES * n_exp;
+    unsigned* const poff = tot + n_exp;
     __shared__ unsigned wsum[MOE_ALIGN_WAVES], whit[MOE_ALIGN_WAVES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int i = tid; i < MOE_ALIGN_WAVES * n_exp; i += 512) cnt[i / n_exp][i % n_exp] = 0;
+    for (int i = tid; i < MOE_ALIGN_WAVES * n_exp; i += MOE_ALIGN_THREADS) cnt[i] = 0;
     const int chunk = ((ns + MOE_ALIGN_WAVES * 64 - 1) / (MOE_ALIGN_WAVES * 64)) * 64;  // slots per wave, multiple of 64
     const int j0 = wave * chunk, steps = chunk / 64;
     int keep[MOE_ALIGN_KEEP];
@@ -739,28 +745,26 @@ extern "C" __global__ __launch_bounds__(512) void w4a16_moe_align(const int* __r
     __syncthreads();
     for (int s = 0; s < steps; s++) {
         const int e = expert_of(s);
-        if (e >= 0) atomicAdd(&cnt[wave][e], 1u);
+        if (e >= 0) atomicAdd(&cnt[wave * n_exp + e], 1u);
     }
     __syncthreads();
-    // thread i owns experts 2i, 2i+1: totals, then a scan of the padded totals over all threads
-    unsigned padded[2], hits = 0, local = 0;
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-        const int e = 2 * tid + h;
+    // thread i owns expert i: total over the waves, then a scan of the padded totals over all threads
+    unsigned padded = 0, hits = 0;
+    {
+        const int e = tid;
         unsigned run = 0;
         if (e < n_exp) {
             for (int w = 0; w < MOE_ALIGN_WAVES; w++) {
-                const unsigned c = cnt[w][e];
-                cnt[w][e] = run;
+                const unsigned c = cnt[w * n_exp + e];
+                cnt[w * n_exp + e] = run;
                 run += c;
             }
             tot[e] = run;
         }
-        padded[h] = ((run + block - 1) / block) * block;
-        hits += run != 0;
-        local += padded[h];
+        padded = ((run + block - 1) / block) * block;
+        hits = run != 0;
     }
-    unsigned incl = local, hincl = hits;
+    unsigned incl = padded, hincl = hits;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
         const unsigned v = __shfl_up(incl, off), hv = __shfl_up(hincl, off);
@@ -781,20 +785,20 @@ extern "C" __global__ __launch_bounds__(512) void w4a16_moe_align(const int* __r
         all += wsum[w];
         allhit += whit[w];
     }
-    // global stores come last: a workgroup barrier waits for every outstanding store, so none may be pending at one
-    const unsigned pos0 = base + incl - local;
-    {
-        unsigned pos = pos0;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const int e = 2 * tid + h;
-            if (e < n_exp) poff[e] = pos;
-            pos += padded[h];
-        }
+    const unsigned pos0 = base + incl - padded;
+    if (tid < n_exp) poff[tid] = pos0;
+    // every position gets the padding sentinel first, coalesced; the slots are placed over it after the barrier (a
+    // workgroup barrier waits for the stores issued before it, so the order of the two writes to a position is fixed)
+    for (unsigned p = tid; p < all; p += MOE_ALIGN_THREADS) sorted_ids[p] = ns;
+    if (tid < n_exp)
+        for (unsigned b = 0; b < padded / block; b++) expert_ids[pos0 / block + b] = tid;
+    if (tid == 0) {
+        num_post[0] = (int)all;
+        num_post[1] = (int)allhit;
     }
     __syncthreads();
     // placement in slot order: every wave walks its range 64 slots at a time; rank among equal experts in the step.
-    // cnt[wave][*] is private to the wave and LDS operations of one wave execute in order, so the loop needs no
+    // The wave's row of cnt is private to it and LDS operations of one wave execute in order, so the loop needs no
     // workgroup barrier; the wave-scope fences keep the compiler from reordering the LDS accesses.
     int nbits = 1;  // bits that tell experts 0..n_exp-1 apart; the bit above them tells a dropped slot (-1) from all
     while ((1 << nbits) < n_exp) nbits++;
@@ -811,32 +815,15 @@ extern "C" __global__ __launch_bounds__(512) void w4a16_moe_align(const int* __r
         const unsigned same = (unsigned)__popcll(peers);
         const unsigned rank = __builtin_amdgcn_mbcnt_hi((unsigned)(peers >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)peers, 0u));
         unsigned before = 0;
-        if (e >= 0) before = cnt[wave][e];
+        if (e >= 0) before = cnt[wave * n_exp + e];
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if (e >= 0) {
             sorted_ids[poff[e] + before + rank] = j0 + s * 64 + lane;
-            if (rank + 1 == same) cnt[wave][e] = before + same;
+            if (rank + 1 == same) cnt[wave * n_exp + e] = before + same;
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
-    }
-    if (tid == 0) {
-        num_post[0] = (int)all;
-        num_post[1] = (int)allhit;
-    }
-    {
-        unsigned pos = pos0;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const int e = 2 * tid + h;
-            if (e < n_exp) {
-                const unsigned c = tot[e];
-                for (unsigned p = c; p < padded[h]; p++) sorted_ids[pos + p] = ns;
-                for (unsigned b = 0; b < padded[h] / block; b++) expert_ids[pos / block + b] = e;
-            }
-            pos += padded[h];
-        }
     }
 }
 

@@ -87,7 +87,8 @@ def test_route_ties_go_to_lower_index(dec):
 
 # ------------------------------------------------------------------ align on the device
 @pytest.mark.parametrize("ns,n_exp,block", [(8, 128, 4), (32, 128, 4), (128, 128, 16), (4096, 128, 48), (4096, 128, 32),
-                                            (4096, 128, 64), (1000, 7, 64), (130, 1024, 16), (1, 1, 4), (777, 33, 16)])
+                                            (4096, 128, 64), (1000, 7, 64), (130, 1024, 16), (1, 1, 4), (777, 33, 16),
+                                            (20000, 128, 64), (9000, 1000, 16)])
 def test_align_matches_oracle(dec, orc, ns, n_exp, block):
     say("align", ns, n_exp, block)
     rng = np.random.default_rng(ns * 7 + n_exp)
