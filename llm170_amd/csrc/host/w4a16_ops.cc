@@ -45,13 +45,18 @@ static int launch_lane(w4a16_ctx* ctx, uint64_t q, uint64_t s, uint64_t x, uint6
 // a wide output runs best with one row block per wave and four waves (5.5 against 5.3 TB/s on gate+up); for 9..16
 // token rows on wide outputs four row blocks per wave halve the x operand traffic.
 static int pick_decode_shape(const w4a16_ctx* ctx, const W4Lin& L, size_t t, int* rb_out, int* waves_out) {
+    // Measured on the 27B shapes.  Wide outputs (>= 1024 row blocks): four waves per block; one row block per wave for
+    // one or two tokens, two up to six, four beyond (the more tokens, the more x bytes a weight byte drags through the
+    // L1 — wider waves share them).  Narrow outputs: two row blocks x eight waves, so that the few blocks still bring
+    // enough waves.
     const bool wide = L.row_blocks >= 1024;
-    const bool wide16 = t > 8 && wide, wide1 = t == 1 && wide;
-    int rb = ctx->decode_rows_per_wave ? ctx->decode_rows_per_wave / 16 : (wide16 ? 4 : wide1 ? 1 : 2);
+    const int rb_auto = wide ? (t <= 2 ? 1 : t <= 6 ? 2 : 4) : 2;
+    const int waves_auto = wide ? 4 : (t > 8 ? 4 : 8);
+    int rb = ctx->decode_rows_per_wave ? ctx->decode_rows_per_wave / 16 : rb_auto;
     if (rb != 1 && rb != 2 && rb != 4) return w4_fail(W4A16_ERR_ARG, "decode: rows_per_wave must be 16, 32 or 64");
     while (rb > 1 && L.row_blocks < (size_t)rb) rb >>= 1;
     const int kt_n = (int)(L.k / 128);
-    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : (wide16 ? 2 : (t > 8 || wide1) ? 4 : 8);
+    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : waves_auto;
     waves = std::max(1, std::min(std::min(waves, 8), kt_n));
     *rb_out = rb;
     *waves_out = waves;
@@ -118,7 +123,7 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
     if (L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
         return w4_fail(W4A16_ERR_SHAPE, "decode: tiled weights of 2 GiB or more exceed the buffer-descriptor range");
     const int kt_n = (int)(L.k / 128);
-    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : (t > 8 ? 4 : 8);
+    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : (t > 8 || L.row_blocks >= 1024 ? 4 : 8);
     waves = std::max(1, std::min(std::min(waves, 8), kt_n));
     const int xl = t <= 4 ? 1 : t <= 8 ? 2 : 4;
     char sym[64];
