@@ -104,3 +104,23 @@ def test_code_objects_are_gfx950():
     for asset in ffi.manifest():
         blob = open(os.path.join(adir, asset + ".hsaco"), "rb").read()
         assert blob[:4] == b"\x7fELF" and b"gfx950" in blob, asset
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The bench measures one GPU's share; asked for more it says so and exits non-zero without touching a device."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "--gpus 2" in r.stderr and r.stdout.strip() == ""
+
+
+def test_product_path_fails_loudly_without_a_gpu():
+    """No CPU fallback: creating a context where no HIP device exists raises the library's error."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from llm170_amd import ops
+    with pytest.raises(ops.W4a16Error):
+        ops.Ctx(0)
