@@ -59,6 +59,48 @@ def measured_traffic(kernel):
     return None
 
 
+def chip_probes(cc, nbytes, copies):
+    """What the chip sustains with nothing but the bounding resource in use (context for the roofline fractions, which
+    stay priced against the published peaks): a read-only stream over buffers of the headline linear's size, rotated
+    like its weight copies, launch after launch as in the timed region; the same stream as one long launch; and a loop
+    of v_mfma_f32_32x32x16_f16 on independent accumulators."""
+    import ctypes as C
+    n16 = (nbytes + 15) // 16
+    buf = cc.alloc(n16 * 16 * copies)
+    cc.memset0(buf, n16 * 16 * copies)
+    sink = cc.alloc(256)
+    e0, e1 = cc.event(), cc.event()
+
+    def read_run(blocks, reps, span, rotate):
+        for timed in (False, True):
+            e0.record()
+            for r in range(reps):
+                src = buf + (r % copies) * n16 * 16 if rotate else buf
+                cc.launch("w4a16_read_u4", blocks, 1, 256, [C.c_uint64(src), C.c_size_t(span), C.c_uint64(sink)])
+            e1.record()
+            cc.sync()
+        return e0.elapsed_ms(e1) / reps
+
+    per_launch = min(read_run(b, 400, n16, True) for b in (2048, 4096, 8192))
+    one_long = min(read_run(b, 4, n16 * copies, False) for b in (2048, 4096, 8192))
+    iters, blocks = 4096, 1024
+    for timed in (False, True):
+        e0.record()
+        for r in range(8):
+            cc.launch("w4a16_mfma_peak_f16", blocks, 1, 256, [C.c_uint64(sink), C.c_int(iters)])
+        e1.record()
+        cc.sync()
+    mfma_ms = e0.elapsed_ms(e1) / 8
+    e0.destroy()
+    e1.destroy()
+    cc.free(buf)
+    cc.free(sink)
+    return {"read_only_GBps_per_launch_same_bytes": round(n16 * 16 / per_launch / 1e6, 1),
+            "read_only_us_per_launch_same_bytes": round(per_launch * 1e3, 2),
+            "read_only_GBps_one_long_launch": round(n16 * 16 * copies / one_long / 1e6, 1),
+            "mfma_f16_loop_TFLOPs": round(blocks * 4 * iters * 4 * 32768 / mfma_ms / 1e9, 1)}
+
+
 def time_forward(dec, names, xd, yd, t, steps, warmup, path, out_f16=True):
     ms, wall = dec.bench_forward(names, xd, yd, t, steps, warmup=warmup, out_f16=out_f16, path=path)
     return ms / steps, wall / steps
@@ -204,6 +246,8 @@ def main():
              "parity_f16_out": {a: par[a] for a in ("rel_l2", "max_ulp", "max_ulp_strict", "strict_pass_frac", "clamped")},
              "parity_f32_out": {a: par_f32[a] for a in ("rel_l2", "max_ulp", "max_ulp_strict", "strict_pass_frac", "clamped")},
              "peaks": {"hbm_GBps": HBM_PEAK_GBPS, "mfma_f16_TFLOPs": MFMA_F16_PEAK_TFLOPS}}
+    if not args.no_extra:
+        extra["chip_probes"] = chip_probes(cc, nbytes, args.copies)
 
     # ---------------------------------------------------------------- prefill GEMM, M=4096 (second half of the metric)
     mp = 4096

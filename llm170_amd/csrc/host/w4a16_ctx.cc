@@ -66,7 +66,8 @@ static const char* const kDecodeSyms[] = {
 static const char* const kPrefillSyms[] = {"w4a16_prefill_g128_f16", "w4a16_prefill_g128_bf16", "w4a16_prefill_g32_f16",
                                            "w4a16_prefill_g32_bf16", "w4a16_prefill_g128_f16_m64", "w4a16_prefill_g128_bf16_m64", "w4a16_prefill_g32_f16_m64",
                                            "w4a16_prefill_g32_bf16_m64", "w4a16_prefill_splitk_sum", nullptr};
-static const char* const kUtilSyms[] = {"w4a16_fill0_u32", "w4a16_copy_u4", nullptr};
+static const char* const kUtilSyms[] = {"w4a16_fill0_u32", "w4a16_copy_u4", "w4a16_read_u4", "w4a16_mfma_peak_f16",
+                                         nullptr};
 static const char* const kGlueSyms[] = {"w4a16_rms_rescale_f16", "w4a16_silu_mul_f16", "w4a16_synth_q", "w4a16_synth_s",
                                         "w4a16_norm_resid", nullptr};
 #define W4_MOE_FAMILY(P)                                                                                      \
