@@ -107,7 +107,10 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     int nks = 1;
     W4_TRY(decode_split(ctx, L, t, blocks, rb, &waves, &nks));
     uint64_t ws = ctx->decode_ws, tk = ctx->decode_tickets;
-    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk};
+    // launch geometry as kernel arguments (the kernel reads nothing from the dispatch packet): k tiles per slice and
+    // per wave, both rounded up
+    int kt_per_slice = (int)ceil_div(L.k / 128, (size_t)nks), kt_per_wave = (kt_per_slice + waves - 1) / waves;
+    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave};
     // LDS: the split-K partial tiles [waves][rb][1 KiB], then two scale slots per wave; a slot holds the scales of
     // one ring round (rb x depth x groups-per-tile x 32 bytes, ring never deeper than 8 tiles) rounded up to 512
     const unsigned slot = ((unsigned)(rb * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
@@ -134,7 +137,8 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
     int nks = 1;
     W4_TRY(decode_split(ctx, L, t, blocks, 2, &waves, &nks));
     uint64_t ws = ctx->decode_ws, tk = ctx->decode_tickets;
-    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk};
+    int kt_per_slice = (kt_n + nks - 1) / nks, kt_per_wave = (kt_per_slice + waves - 1) / waves;
+    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave};
     const unsigned slot = ((unsigned)(2 * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
     const unsigned shmem = (unsigned)(waves * 2 * 1024) + (unsigned)waves * 2u * slot;
     return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);

@@ -53,7 +53,8 @@ __device__ __forceinline__ u4_t w4_row_shl(u4_t v) {
 template <int G, bool SBF, int RB, int DEPTH, int XL, bool GLU = false>
 __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                             const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
-                                            int k, int n, int t, int out_f16, f4_t* ws, int* tickets) {
+                                            int k, int n, int t, int out_f16, f4_t* ws, int* tickets, int W, int nks,
+                                            int kt_per_slice, int kt_per_wave) {
     extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K, then [W][2][AUXB] scale slots
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
     constexpr int AUXB = RB * DEPTH * GPT * 32;      // bytes of scales one ring round needs: [rb][tile][group][16 rows]
@@ -61,7 +62,10 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     constexpr int SLOT = AUXN * 512;                 // LDS bytes of one slot: every lane of every load has a place
     constexpr int C = 4 / XL;           // 32-k chunks (MFMAs) served by one x load
     constexpr int TPL = 16 / C;         // token columns served by one x load
-    const int lane = threadIdx.x & 63, W = blockDim.x >> 6;
+    // The launch geometry (W waves per block, nks k slices over blockIdx.y, tiles per slice and per wave) arrives as
+    // kernel arguments: read from the dispatch packet instead, the block size costs a second dependent memory round
+    // trip and the balanced split two integer divisions before the first weight load can be issued, on every wave.
+    const int lane = threadIdx.x & 63;
     // the wave index is uniform across the wave: keep it (and everything derived from it) in scalar registers
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kt_n = k / W4_TILE_K;
@@ -69,9 +73,9 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     const int nb0 = blockIdx.x * RB;
     const int glu_half = row_blocks >> 1;  // GLU: row block of rb is blockIdx.x + rb * glu_half
     auto row_block = [&](int rb) { return GLU ? (int)blockIdx.x + rb * glu_half : min(nb0 + rb, row_blocks - 1); };
-    const int nks = gridDim.y, ky = blockIdx.y;  // k slices across workgroups
-    const int kt_lo = (kt_n * ky) / nks, kt_span = (kt_n * (ky + 1)) / nks - kt_lo;
-    const int kt0 = kt_lo + (kt_span * wave) / W, kt1 = kt_lo + (kt_span * (wave + 1)) / W;
+    const int ky = blockIdx.y;  // k slice of this workgroup
+    const int kt_lo = min(kt_n, ky * kt_per_slice), kt_hi = min(kt_n, kt_lo + kt_per_slice);
+    const int kt0 = min(kt_hi, kt_lo + wave * kt_per_wave), kt1 = min(kt_hi, kt0 + kt_per_wave);
     const int m = lane & 15, g = lane >> 4;
 
     // Every load is a raw buffer load: an out-of-range offset returns zeros and costs no memory traffic, which
@@ -303,17 +307,20 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
                                                                         const uint16_t* x, void* y, int row_blocks,  \
                                                                         int k, int n, int t, int out_f16, f4_t* ws,  \
-                                                                        int* tickets) {                              \
+                                                                        int* tickets, int waves, int nks,            \
+                                                                        int kt_per_slice, int kt_per_wave) {         \
         decode_body<G, SBF, RB, DECODE_DEPTH(BUDGET, G, RB, XL), XL>(qt, st, x, y, row_blocks, k, n, t, out_f16, ws, \
-                                                                     tickets);                                       \
+                                                                     tickets, waves, nks, kt_per_slice, kt_per_wave); \
     }
 #define DECODE_GLU_KERNEL_X(NAME, G, SBF, XL, BUDGET, ATTR)                                                           \
     extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
                                                                         const uint16_t* x, void* y, int row_blocks,  \
                                                                         int k, int n, int t, int out_f16, f4_t* ws,  \
-                                                                        int* tickets) {                              \
+                                                                        int* tickets, int waves, int nks,            \
+                                                                        int kt_per_slice, int kt_per_wave) {         \
         decode_body<G, SBF, 2, DECODE_DEPTH(BUDGET, G, 2, XL), XL, true>(qt, st, x, y, row_blocks, k, n, t, out_f16,  \
-                                                                         ws, tickets);                               \
+                                                                         ws, tickets, waves, nks, kt_per_slice,      \
+                                                                         kt_per_wave);                               \
     }
 #define DECODE_HI __attribute__((amdgpu_waves_per_eu(6, 6)))
 #define DECODE_MID __attribute__((amdgpu_waves_per_eu(5, 5)))
