@@ -228,20 +228,21 @@ static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_
     int xr = (int)x_rows, xd = (int)x_div, yf = y_f16, blk = (int)block, nsi = (int)ns, rbi = (int)row_blocks,
         ki = (int)k, ni = (int)n, nei = (int)E.n_exp;
     uint64_t ws = 0, tk = 0;
+    int waves = 0;  // set below, before the launch reads it
     void* p[] = {&qa, &sa, &qs, &ss, &x, &xr, &xd, &y, &yf, &topw, &sorted, &eids, &npost, &blk, &nsi, &rbi, &ki, &ni, &nei,
-                 &ws, &tk};
+                 &ws, &tk, &waves};
     char sym[80];
     const char* fam = E.scale_bf16 ? "bf16" : "f16";
     if (block <= 16) {
         // in-block split-K: each wave needs at least one k tile
-        int waves = ctx->moe_waves ? ctx->moe_waves : 4;
+        waves = ctx->moe_waves ? ctx->moe_waves : 4;
         waves = std::max(1, std::min(std::min(waves, 8), (int)kt_n));
         snprintf(sym, sizeof sym, "w4a16_moe_g%zu_%s_dec_%s_x%d", E.group, fam, glu ? "glu" : "lin", block <= 4 ? 1 : 4);
         const unsigned shmem = waves > 1 ? (unsigned)(waves * 2 * 64 * 16) : 0;
         return w4_launch(ctx, sym, (unsigned)(max_segs * units), 1, (unsigned)(waves * 64), shmem, p);
     }
     const int tt = (int)(block / 16);
-    int waves = ctx->moe_waves ? ctx->moe_waves : 4;
+    waves = ctx->moe_waves ? ctx->moe_waves : 4;
     waves = waves >= 8 ? 8 : 4;  // the x staging needs at least 4 waves
     const size_t blocks = max_segs * ((units + (size_t)waves - 1) / (size_t)waves);
     nks = std::max<size_t>(1, std::min<size_t>(std::min<size_t>(nks, 8), kt_n / 2));

@@ -113,14 +113,16 @@ __device__ __forceinline__ void moe_store(f4_t a0, f4_t a1, int slot, int q, int
 //   A segment whose expert id is outside 0..n_exp-1 is skipped (its slots stay unwritten).
 //   ws / tickets: workspace and zeroed counters of a launch split over k across workgroups (gridDim.y slices; the
 //   LDS-staged kernel only): [slice][block][wave][2*TT] partial tiles, one counter per (block, wave).
+//   wpb: waves per block (the block size, as an argument: read from the dispatch packet it costs one more dependent
+//   scalar-cache miss before the first weight load).
 #define MOE_PARAMS                                                                                                  \
     const char *__restrict__ qa, const char *__restrict__ sa, unsigned long long q_stride,                          \
         unsigned long long s_stride, const uint16_t *__restrict__ x, int x_rows, int x_div, void *__restrict__ y,   \
         int y_f16, const float *__restrict__ topw, const int *__restrict__ sorted_ids,                              \
         const int *__restrict__ expert_ids, const int *__restrict__ num_post, int blk, int ns, int row_blocks, int k, \
-        int n, int n_exp, f4_t *ws, int *tickets
+        int n, int n_exp, f4_t *ws, int *tickets, int wpb
 #define MOE_ARGS \
-    qa, sa, q_stride, s_stride, x, x_rows, x_div, y, y_f16, topw, sorted_ids, expert_ids, num_post, blk, ns, row_blocks, k, n, n_exp, ws, tickets
+    qa, sa, q_stride, s_stride, x, x_rows, x_div, y, y_f16, topw, sorted_ids, expert_ids, num_post, blk, ns, row_blocks, k, n, n_exp, ws, tickets, wpb
 
 // ---------------------------------------------------------------------------------------------------- moe_dec
 template <int RB, int XL>
@@ -136,16 +138,27 @@ __device__ __forceinline__ void moe_dec_body(MOE_PARAMS) {
     extern __shared__ f4_t red[];  // [W][2][64]
     constexpr int GPT = W4_TILE_K / G;
     constexpr int C = 4 / XL, TPL = 16 / C;
-    const int lane = threadIdx.x & 63, W = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, W = wpb;
+    // every kernel argument is fetched here, in one batch: left to the compiler they arrive in three dependent
+    // scalar-cache misses spread over the prologue, each ahead of the first weight load
+    asm volatile("" ::"s"(qa), "s"(sa), "s"(q_stride), "s"(s_stride), "s"(x), "s"(x_rows), "s"(x_div), "s"(y), "s"(topw),
+                 "s"(sorted_ids), "s"(blk), "s"(ns), "s"(row_blocks), "s"(k), "s"(n),
+                 "s"(n_exp), "s"(wpb));
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int units = GLU ? row_blocks >> 1 : (row_blocks + 1) >> 1;
     const int seg = blockIdx.x / units, u = blockIdx.x % units;
-    if (seg * blk >= num_post[0]) return;
-    const int e = __builtin_amdgcn_readfirstlane(expert_ids[seg]);
+    const int m = lane & 15, g = lane >> 4;
+    const int xtok = m % TPL, xchunk = m / TPL;
+    // The three table reads (padded total, the segment's expert, the lane's slot id) are issued together, ahead of
+    // the tests that use them: one memory round trip before the first weight load instead of three.  The tables hold
+    // an entry for every segment the grid was sized for.
+    int np = num_post[0], e = expert_ids[seg], xslot = sorted_ids[seg * blk + min(xtok, blk - 1)];
+    asm volatile("" : "+s"(np), "+s"(e), "+v"(xslot));
+    if (seg * blk >= np) return;
     if ((unsigned)e >= (unsigned)n_exp) return;  // uniform for the block
+    if (xtok >= blk) xslot = ns;
     const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
     const int kt0 = (kt_n * wave) / W, kt1 = (kt_n * (wave + 1)) / W;
-    const int m = lane & 15, g = lane >> 4;
     const int rbA = GLU ? u : 2 * u, rbB = GLU ? u + units : min(2 * u + 1, row_blocks - 1);
     const bool haveB = GLU || 2 * u + 1 < row_blocks;
 
@@ -155,8 +168,6 @@ __device__ __forceinline__ void moe_dec_body(MOE_PARAMS) {
         w4_make_rsrc(sa + (unsigned long long)e * s_stride, (unsigned)row_blocks * (unsigned)kg_n * 32u);
     const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)x_rows * (unsigned)k * 2u);
 
-    const int xtok = m % TPL, xchunk = m / TPL;
-    const int xslot = xtok < blk ? sorted_ids[seg * blk + xtok] : ns;
     const unsigned xoff =
         xslot < ns ? ((unsigned)(xslot / x_div) * (unsigned)k + (unsigned)(xchunk * 32 + g * 8)) * 2u : W4_OOB;
     const unsigned qoff[2] = {(unsigned)rbA * (unsigned)kt_n * 1024u + (unsigned)lane * 16u,
@@ -267,6 +278,9 @@ __device__ __forceinline__ void moe_down_sum_body(const char* __restrict__ qa, c
     extern __shared__ f4_t red[];  // [top_k][RB][64]
     constexpr int GPT = W4_TILE_K / G;
     const int lane = threadIdx.x & 63;
+    // every kernel argument is fetched here, in one batch (see moe_dec_body)
+    asm volatile("" ::"s"(qa), "s"(sa), "s"(q_stride), "s"(s_stride), "s"(act), "s"(idx), "s"(topw), "s"(y), "s"(top_k),
+                 "s"(ns), "s"(row_blocks), "s"(k), "s"(n), "s"(n_exp));
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int units = (row_blocks + RB - 1) / RB;
     const int token = blockIdx.x / units, u = blockIdx.x % units;
@@ -414,16 +428,25 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     extern __shared__ _Float16 xs[];  // [2][16*TT][MOE_LDX]
     constexpr int GPT = W4_TILE_K / G;
     constexpr int ROWS = 16 * TT;
-    const int tid = threadIdx.x, lane = tid & 63, W = blockDim.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, W = wpb;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int units = GLU ? row_blocks >> 1 : (row_blocks + 1) >> 1;
     const int groups = (units + W - 1) / W;
     const int seg = blockIdx.x / groups, grp = blockIdx.x % groups;
-    if (seg * blk >= num_post[0]) return;  // uniform for the block, before any barrier
+    // the table reads (padded total, the segment's expert, this thread's slot ids) are issued together, ahead of the
+    // tests that use them (see moe_dec_body)
+    const int rows_pp = 4 * W;
+    int np = num_post[0], e = expert_ids[seg];
+    int slot_of[TT];
+#pragma unroll
+    for (int p = 0; p < TT; p++) slot_of[p] = sorted_ids[seg * blk + min(p * rows_pp + (tid >> 4), ROWS - 1)];
+    asm volatile("" : "+s"(np), "+s"(e));
+#pragma unroll
+    for (int p = 0; p < TT; p++) asm volatile("" : "+v"(slot_of[p]));
+    if (seg * blk >= np) return;  // uniform for the block, before any barrier
     const int u_raw = grp * W + wave;
     const bool active = u_raw < units;  // a surplus wave repeats the last unit and stores nothing
     const int u = min(u_raw, units - 1);
-    const int e = __builtin_amdgcn_readfirstlane(expert_ids[seg]);
     if ((unsigned)e >= (unsigned)n_exp) return;  // uniform for the block, before any barrier
     const int kt_n = k / W4_TILE_K, kg_n = kt_n * GPT;
     const int nks = KS ? (int)gridDim.y : 1, ky = KS ? (int)blockIdx.y : 0;  // k slices across workgroups
@@ -439,13 +462,12 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)x_rows * (unsigned)k * 2u);
 
     // x staging: one k tile of the segment's rows = ROWS x 256 B; 16 threads cover a row, 4*W rows per pass
-    const int rows_pp = 4 * W;
     unsigned xg_off[TT];
     int xl_off[TT];
 #pragma unroll
     for (int p = 0; p < TT; p++) {
         const int row = p * rows_pp + (tid >> 4);
-        const int slot = row < ROWS ? sorted_ids[seg * blk + row] : ns;
+        const int slot = row < ROWS ? slot_of[p] : ns;
         xg_off[p] = slot < ns ? ((unsigned)(slot / x_div) * (unsigned)k + (unsigned)(tid & 15) * 8u) * 2u : W4_OOB;
         xl_off[p] = row < ROWS ? row * MOE_LDX + (tid & 15) * 8 : -1;
     }
