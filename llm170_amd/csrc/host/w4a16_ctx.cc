@@ -140,7 +140,9 @@ static int read_file(const std::string& path, std::vector<char>* out) {
 // ------------------------------------------------------------------------------------------------ context
 extern "C" int w4a16_module_load(w4a16_ctx* ctx, const char* key, const void* image, size_t len,
                                  const char* const* symbols, size_t nsym) {
-    if (!ctx || !key || !image || len == 0) return w4_fail(W4A16_ERR_ARG, "module_load: null argument");
+    if (!ctx || !key || !image || len == 0 || (nsym && !symbols)) return w4_fail(W4A16_ERR_ARG, "module_load: null argument");
+    for (size_t i = 0; i < nsym; i++)
+        if (!symbols[i]) return w4_fail(W4A16_ERR_ARG, "module_load(%s): symbol %zu is null", key, i);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     hipModule_t mod = nullptr;
     hipError_t e = hipModuleLoadData(&mod, image);

@@ -158,6 +158,26 @@ def test_decode_split_k_across_workgroups(dec, orc, nks):
         dec.set_decode_ksplit(9)
 
 
+def test_decode_split_k_with_an_empty_slice(dec, orc):
+    """9 k tiles in 4 slices of 3 (tiles per slice are rounded up): the fourth slice is empty and adds zeros; waves
+    beyond a slice's tiles stream nothing."""
+    n, k, group = 80, 1152, 128
+    q, s, x = gen.make_linear(n, k, group, 4, seed=15)
+    dec.upload_lin_g("ks9", q, s, n, k, group, False)
+    want = orc.gemm_lane(x, 4, q, s, n, k, group, threads=8)
+    try:
+        dec.set_decode_ksplit(4)
+        for waves in (0, 2, 8):
+            dec.set_decode_shape(0, waves)
+            for t in (1, 4):
+                say("decode empty slice", waves, t)
+                parity.assert_close(dec.gemv_host("ks9", x[:t], t=t, path=ops.PATH_DECODE), want[:t],
+                                    "decode empty slice waves %d t%d" % (waves, t))
+    finally:
+        dec.set_decode_ksplit(0)
+        dec.set_decode_shape(0, 0)
+
+
 def test_decode_bf16_scales(dec, orc):
     n, k, group = 256, 2048, 32
     q, s, x = gen.make_linear(n, k, group, 4, seed=8)
