@@ -56,7 +56,7 @@ extern "C" int w4a16_rms_rescale_f16(w4a16_ctx* ctx, uint64_t v_f32_dev, size_t 
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     int ldi = (int)ld, nc = (int)ncols;
     void* p[] = {&v_f32_dev, &ldi, &nc, &out_f16_dev};
-    return w4_launch(ctx, "w4a16_rms_rescale_f16", (unsigned)t, 1, 1024, 0, p);
+    return w4_launch(ctx, "w4a16_rms_rescale_f16", (unsigned)t, 1, kW4RmsLanes, 0, p);
 }
 
 extern "C" int w4a16_norm_resid(w4a16_ctx* ctx, uint64_t x_dev, uint64_t nw_dev, uint64_t ab_dev, uint64_t xn_dev,

@@ -79,6 +79,20 @@ struct w4a16_ctx {
     int cu_count = 0;
 };
 
+// Launch constants that mirror #defines of the kernel sources (a CPU test reads both texts and compares the values):
+// name here = kW4 + CamelCase of the kernel-side macro.
+constexpr int kW4TileK = 128;               // W4_TILE_K (w4a16_common.hpp)
+constexpr int kW4TileRows = 16;             // W4_TILE_ROWS
+constexpr int kW4LaneTt = 8;                // LANE_TT (lane.hip): tokens per pass of the lane-order kernel
+constexpr int kW4DecodeMaxKsplit = 8;       // W4_DECODE_MAX_KSPLIT (decode.hip)
+constexpr int kW4MoeMaxKsplit = 8;          // MOE_MAX_KSPLIT (moe.hip)
+constexpr int kW4MoeLdx = 136;              // MOE_LDX (moe.hip): halves per staged x row
+constexpr int kW4MoeAlignWaves = 16;        // MOE_ALIGN_WAVES (moe.hip)
+constexpr int kW4RmsLanes = 1024;           // RMS_LANES (glue.hip)
+constexpr int kW4PfBn = 256;                // PF_BN (prefill.hip): block tile columns
+constexpr int kW4PfKs = 64;                 // PF_KS (prefill.hip): k per LDS stage
+constexpr int kW4PfThreads = 256;           // PF_THREADS (prefill.hip)
+
 int w4_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int w4_hip(hipError_t e, const char* api);
 // Keep the message of a failing step across clean-up calls that may fail themselves.

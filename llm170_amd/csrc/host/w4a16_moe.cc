@@ -182,7 +182,7 @@ extern "C" int w4a16_moe_align(w4a16_ctx* ctx, uint64_t idx_dev, size_t ns, size
     int nsi = (int)ns, ni = (int)n_exp, bi = (int)block;
     void* p[] = {&idx_dev, &nsi, &ni, &bi, &sorted_dev, &expert_ids_dev, &num_post_dev};
     // LDS: 16 per-wave count rows, totals and offsets, one entry per expert each
-    return w4_launch(ctx, "w4a16_moe_align", 1, 1, 1024, (unsigned)((16 + 2) * n_exp * 4), p);
+    return w4_launch(ctx, "w4a16_moe_align", 1, 1, 64 * kW4MoeAlignWaves, (unsigned)((kW4MoeAlignWaves + 2) * n_exp * 4), p);
 }
 
 // ------------------------------------------------------------------------------------------------ FFN
@@ -245,7 +245,7 @@ static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_
     waves = ctx->moe_waves ? ctx->moe_waves : 4;
     waves = waves >= 8 ? 8 : 4;  // the x staging needs at least 4 waves
     const size_t blocks = max_segs * ((units + (size_t)waves - 1) / (size_t)waves);
-    nks = std::max<size_t>(1, std::min<size_t>(std::min<size_t>(nks, 8), kt_n / 2));
+    nks = std::max<size_t>(1, std::min<size_t>(std::min<size_t>(nks, kW4MoeMaxKsplit), kt_n / 2));
     if (nks > 1) {
         // split over k across workgroups: partial tiles and per-(block, wave) tickets, shared with the decode kernel
         W4_TRY(w4_ensure(ctx, &ctx->decode_ws, &ctx->decode_ws_cap, blocks * (size_t)waves * 2 * (size_t)tt * 1024 * nks));
@@ -259,7 +259,7 @@ static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_
     }
     if (nks > 1 && glu) return w4_fail(W4A16_ERR_UNSUPPORTED, "moe: the gate|up kernel does not split over k");
     snprintf(sym, sizeof sym, "w4a16_moe_g%zu_%s_mm_%s_t%d%s", E.group, fam, glu ? "glu" : "lin", tt, nks > 1 ? "_ks" : "");
-    const unsigned shmem = (unsigned)(2 * 16 * tt * 136 * 2);
+    const unsigned shmem = (unsigned)(2 * 16 * tt * kW4MoeLdx * 2);
     return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, p);
 }
 

@@ -36,7 +36,7 @@ static int launch_lane(w4a16_ctx* ctx, uint64_t q, uint64_t s, uint64_t x, uint6
         return w4_fail(W4A16_ERR_SHAPE, "lane: n=%zu k=%zu t=%zu exceed the launch limits", n, k, t);
     int ni = (int)n, ki = (int)k, ti = (int)t;
     void* params[] = {&q, &s, &x, &out, &ni, &ki, &ti};
-    return w4_launch(ctx, sym, ceil_div(n, 4), ceil_div(t, 8), 256, 0, params);
+    return w4_launch(ctx, sym, ceil_div(n, 4), ceil_div(t, kW4LaneTt), 256, 0, params);
 }
 
 // Launch shape of the row-block decode kernel.  Measured on MI355X at the 27B layer shapes (gate+up 5120x34816, down
@@ -74,7 +74,7 @@ static int decode_split(w4a16_ctx* ctx, const W4Lin& L, size_t t, size_t blocks,
         // a long k range over fewer workgroups than CUs (the 27B down projection: 160 blocks x 136 k tiles): slices
         // of about 16 k tiles, four waves each (measured 12.4 -> 11.8 us at t = 1, 13.3 -> 12.4 us at t = 4).  Shorter
         // k ranges lose more to the extra workgroups than they gain.
-        nks = std::min(8, kt_n / 16);
+        nks = std::min(kW4DecodeMaxKsplit, kt_n / 16);
         *waves = std::min(*waves, 4);
     }
     nks = std::max(1, std::min(nks, kt_n / 2));
@@ -156,7 +156,7 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     // many rows; which one finishes first is mostly a matter of how the workgroups divide into the slots of the chip,
     // so both are priced — (generations of workgroups) x (k tiles per slice) x (relative tile time) — and the cheaper
     // one runs (sweeps over the 27B shapes, t = 65..4096: within ~5 % of the better tile everywhere).
-    const size_t tiles_n = (L.n + 255) / 256, kt_n = L.k / 128, cus = (size_t)std::max(ctx->cu_count, 1);
+    const size_t tiles_n = (L.n + kW4PfBn - 1) / kW4PfBn, kt_n = L.k / 128, cus = (size_t)std::max(ctx->cu_count, 1);
     auto slices_for = [&](size_t tiles, size_t slots) {
         size_t nks = 1;
         if (ctx->prefill_ksplit > 0) {
@@ -195,13 +195,13 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     const size_t nks = slices_for(tiles_m * tiles_n, slots);
     char sym[64];
     snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s%s", L.group, L.scale_bf16 ? "bf16" : "f16", bm == 64 ? "_m64" : "");
-    const unsigned shmem = (unsigned)(2 * bm * 64 * 2);
+    const unsigned shmem = (unsigned)(2 * bm * kW4PfKs * 2);  // two stages of bm rows x PF_KS halves
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
     int spm = (int)sup_m, spn = (int)sup_n;
     if (nks == 1) {
         void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &spm, &spn};
-        return w4_launch(ctx, sym, (unsigned)grid, 1, 256, shmem, params);
+        return w4_launch(ctx, sym, (unsigned)grid, 1, kW4PfThreads, shmem, params);
     }
     if (L.n % 4 != 0) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: split-K needs n %% 4 == 0");
     const size_t count = t * L.n;
@@ -209,7 +209,7 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     uint64_t ws = ctx->prefill_ws;
     int zero = 0;
     void* params[] = {&qt, &st, &x, &ws, &row_blocks, &ki, &ni, &ti, &zero, &spm, &spn};
-    W4_TRY(w4_launch(ctx, sym, (unsigned)grid, (unsigned)nks, 256, shmem, params));
+    W4_TRY(w4_launch(ctx, sym, (unsigned)grid, (unsigned)nks, kW4PfThreads, shmem, params));
     int nksi = (int)nks;
     size_t cnt = count;
     void* rp[] = {&ws, &y, &nksi, &cnt, &of};
@@ -530,7 +530,8 @@ extern "C" int w4a16_set_prefill_tile(w4a16_ctx* ctx, int rows) {
 
 extern "C" int w4a16_set_decode_ksplit(w4a16_ctx* ctx, int ksplit) {
     if (!ctx) return w4_fail(W4A16_ERR_ARG, "set_decode_ksplit: null context");
-    if (ksplit < -1 || ksplit > 8) return w4_fail(W4A16_ERR_ARG, "set_decode_ksplit: -1 = never, 0 = automatic, 1..8 slices");
+    if (ksplit < -1 || ksplit > kW4DecodeMaxKsplit)
+        return w4_fail(W4A16_ERR_ARG, "set_decode_ksplit: -1 = never, 0 = automatic, 1..%d slices", kW4DecodeMaxKsplit);
     ctx->decode_ksplit = ksplit;
     return 0;
 }

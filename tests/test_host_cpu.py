@@ -65,6 +65,26 @@ def test_manifest_matches_kernel_sources():
     assert hips == sorted(man), "every kernel source is a manifest asset and vice versa"
 
 
+def test_host_constants_mirror_kernel_defines():
+    """Precedent: constants of the host must equal the #defines parsed out of the kernel text
+    (w4a16_dec/tests.rs:87-202).  Host name = kW4 + CamelCase of the macro (W4_ prefix dropped)."""
+    kdir = os.path.join(ROOT, "llm170_amd", "csrc", "kernels")
+    defines = {}
+    for f in os.listdir(kdir):
+        for m in re.finditer(r"^#define\s+([A-Z0-9_]+)\s+(\d+)\b", open(os.path.join(kdir, f)).read(), flags=re.M):
+            defines[m.group(1)] = int(m.group(2))
+    host = open(os.path.join(ROOT, "llm170_amd", "csrc", "host", "w4a16_internal.h")).read()
+    consts = {m.group(1): int(m.group(2)) for m in re.finditer(r"constexpr int kW4(\w+) = (\d+);", host)}
+    assert len(consts) >= 11
+    for camel, value in consts.items():
+        macro = re.sub(r"(?<!^)(?=[A-Z])", "_", camel).upper()
+        hits = [v for k, v in defines.items() if k in (macro, "W4_" + macro)]
+        assert hits == [value], (camel, macro, hits, value)
+    # the sources use the names, not the numbers, where a launch depends on them
+    moe = open(os.path.join(ROOT, "llm170_amd", "csrc", "host", "w4a16_moe.cc")).read()
+    assert "kW4MoeAlignWaves" in moe and "kW4MoeLdx" in moe and "kW4MoeMaxKsplit" in moe
+
+
 def test_shapes_accept_contract():
     # gptq4.rs:196-208
     ops.check_shapes(1, 8 * 640, 8 * 40, 5120, 8, 5120, 128)
