@@ -150,6 +150,25 @@ int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t
  * as w4a16_lin_forward (decode path, same launch shape) followed by w4a16_silu_mul_f16. */
 int w4a16_lin_forward_glu(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_f16_dev, size_t t);
 
+/* A decode-regime linear (t <= 16) with the RMS normalisation of its input deferred across it.  The reference runs
+ * norm_resid as a launch of its own ahead of each linear (assets/norm.cu:4-48, kernels/mod.rs:11-54); a per-row
+ * factor commutes with the linear, so here the launch that PRODUCES the activations leaves partial sums of their
+ * squares and the launch that CONSUMES them scales its output instead:
+ *   y[r][c] = s[r] * (W x[r])[c],   s[r] = 1 / sqrt(sum_r / in_cols + 1e-6),
+ *   sum_r = the n_stats_in partial sums stats_in_dev[i][r] (f32 [n_stats_in][16], added in a fixed order);
+ *   stats_in_dev == 0: s = 1.
+ * x rows are ldx halves apart (0 = k; a column slice of a wider f16 matrix is allowed, ldx % 8 == 0).
+ * stats_out_dev != 0: the launch writes *n_stats_out entries [i][16] of partial sums of y[r][c]^2 (the f32 values,
+ * before any rounding to f16) over columns c < stat_rows; the buffer must hold ceil(n / 16) entries of 64 bytes.
+ * A chain of such launches needs no normalisation launch between its linears: the f16 activations travel
+ * un-normalised (same relative precision), every consumer applies the factor. */
+int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
+                                    uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_dev,
+                                    int out_f16, uint64_t stats_out_dev, size_t stat_rows, size_t* n_stats_out);
+/* The same for the fused gate|up projection: the factor multiplies gate and up before silu(g) * u. */
+int w4a16_lin_forward_glu_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
+                                        uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_f16_dev);
+
 /* gemv_host (w4a16_dec/mod.rs, host-operand convenience used by probes): lin_forward with host x / y. */
 int w4a16_lin_forward_host(w4a16_ctx* ctx, const char* name, const uint16_t* x_f16, void* y, size_t t, int out_f16,
                            int path);
@@ -288,11 +307,21 @@ int w4a16_silu_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_ff, size_t 
  * No host synchronisation. */
 int w4a16_chain_forward(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers, uint64_t x_dev, size_t t,
                         uint64_t y_dev);
+/* The same chain with the normalisations inside it deferred across the linears (w4a16_lin_forward_deferred_norm), four
+ * launches per layer instead of seven, t <= 16.  With r(v) = 1/sqrt(mean(v^2) + 1e-6) per row, s0 = 1 and x0 = x:
+ *     v1 = s[l] * qkv(x[l])[:, :hidden]      a = f16(v1)
+ *     v2 = r(v1) * attn_output(a)            b = f16(v2)
+ *     gu = r(v2) * ffn_gate_up(b)            c = silu_mul_f16(gu)
+ *     v4 = ffn_down(c)                       x[l+1] = f16(v4), s[l+1] = r(v4)
+ * and y = rms_f16(v4) after the last layer: the function of w4a16_chain_forward with the factors applied after the
+ * linears instead of before the roundings to f16 (results agree to those roundings). */
+int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers, uint64_t x_dev,
+                              size_t t, uint64_t y_dev);
 /* Timed chain passes (decode_bench, w4a16_dec/probe.rs:1123-1289): `warmup` untimed then `reps` timed passes over
  * layers 0..n_layers-1.  use_graph != 0 captures one pass into a HIP graph and times graph launches
- * (forward_graph, w4a16_dec/graphs.rs). */
+ * (forward_graph, w4a16_dec/graphs.rs); fused != 0 times w4a16_chain_forward_fused. */
 int w4a16_bench_chain(w4a16_ctx* ctx, const char* prefix, size_t n_layers, uint64_t x_dev, size_t t, uint64_t y_dev,
-                      size_t warmup, size_t reps, int use_graph, float* ms_events, double* ms_wall);
+                      size_t warmup, size_t reps, int use_graph, int fused, float* ms_events, double* ms_wall);
 
 #ifdef __cplusplus
 }

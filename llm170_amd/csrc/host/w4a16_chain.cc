@@ -128,14 +128,68 @@ extern "C" int w4a16_chain_forward(w4a16_ctx* ctx, const char* prefix, size_t la
     return 0;
 }
 
+// The same chain with the three normalisations inside a layer deferred across the linears that follow them
+// (w4a16_lin_forward_deferred_norm): four launches per layer instead of seven.
+extern "C" int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers,
+                                         uint64_t x_dev, size_t t, uint64_t y_dev) {
+    if (!ctx || !prefix || !x_dev || !y_dev) return w4_fail(W4A16_ERR_ARG, "chain_forward_fused: null argument");
+    if (n_layers == 0 || t == 0 || t > 16)
+        return w4_fail(W4A16_ERR_SHAPE, "chain_forward_fused: n_layers=%zu t=%zu (decode regime: 1..16 rows)", n_layers, t);
+    W4ChainScratch& S = ctx->chain;
+    uint64_t cur = x_dev;
+    size_t n_prev = 0;  // partial sums the previous layer's down projection left in S.stats[2]
+    for (size_t l = layer0; l < layer0 + n_layers; l++) {
+        char nm[4][160];
+        const char* role[4] = {"attn_qkv", "attn_output", "ffn_gate_up", "ffn_down"};
+        W4Lin* L[4];
+        for (int i = 0; i < 4; i++) {
+            snprintf(nm[i], sizeof nm[i], "%s.%zu.%s", prefix, l, role[i]);
+            W4_TRY(w4_find_lin(ctx, nm[i], &L[i]));
+        }
+        const size_t hidden = L[0]->k, n_ff = L[3]->k, n_qkv = L[0]->n;
+        if (n_qkv < hidden || n_qkv % 8 != 0 || L[1]->k != hidden || L[1]->n != hidden || L[2]->k != hidden ||
+            L[2]->n != 2 * n_ff || L[3]->n != hidden)
+            return w4_fail(W4A16_ERR_SHAPE, "chain_forward_fused %s.%zu: linears do not chain (hidden %zu, n_ff %zu)", prefix,
+                           l, hidden, n_ff);
+        W4_TRY(w4_ensure(ctx, &S.y32, &S.y32_cap, t * hidden * 4));
+        W4_TRY(w4_ensure(ctx, &S.a16, &S.a16_cap, t * n_qkv * 2));
+        W4_TRY(w4_ensure(ctx, &S.h16a, &S.h16a_cap, t * hidden * 2));
+        W4_TRY(w4_ensure(ctx, &S.h16b, &S.h16b_cap, t * n_ff * 2));
+        W4_TRY(w4_ensure(ctx, &S.ping[0], &S.ping_cap[0], t * hidden * 2));
+        for (int i = 0; i < 3; i++)
+            W4_TRY(w4_ensure(ctx, &S.stats[i], &S.stats_cap[i], ((std::max(n_qkv, hidden) + 15) / 16) * 64));
+        const bool last = l + 1 == layer0 + n_layers;
+        size_t n_a = 0, n_b = 0, n_d = 0;
+        // a = qkv(x)[:, :hidden], its statistics over those columns only
+        W4_TRY(w4a16_lin_forward_deferred_norm(ctx, nm[0], cur, 0, t, n_prev ? S.stats[2] : 0, n_prev, hidden, S.a16, 1,
+                                               S.stats[0], hidden, &n_a));
+        W4_TRY(w4a16_lin_forward_deferred_norm(ctx, nm[1], S.a16, n_qkv, t, S.stats[0], n_a, hidden, S.h16a, 1, S.stats[1],
+                                               hidden, &n_b));
+        W4_TRY(w4a16_lin_forward_glu_deferred_norm(ctx, nm[2], S.h16a, 0, t, S.stats[1], n_b, hidden, S.h16b));
+        if (last) {
+            // the chain's output is normalised: one launch per call, not per layer
+            W4_TRY(w4a16_lin_forward(ctx, nm[3], S.h16b, S.y32, t, 0, W4A16_PATH_DECODE));
+            W4_TRY(w4a16_rms_rescale_f16(ctx, S.y32, hidden, hidden, t, y_dev));
+        } else {
+            W4_TRY(w4a16_lin_forward_deferred_norm(ctx, nm[3], S.h16b, 0, t, 0, 0, 0, S.ping[0], 1, S.stats[2], hidden, &n_d));
+            cur = S.ping[0];
+            n_prev = n_d;
+        }
+    }
+    return 0;
+}
+
 extern "C" int w4a16_bench_chain(w4a16_ctx* ctx, const char* prefix, size_t n_layers, uint64_t x_dev, size_t t,
-                                 uint64_t y_dev, size_t warmup, size_t reps, int use_graph, float* ms_events,
+                                 uint64_t y_dev, size_t warmup, size_t reps, int use_graph, int fused, float* ms_events,
                                  double* ms_wall) {
     if (!ctx || !prefix || reps == 0) return w4_fail(W4A16_ERR_ARG, "bench_chain: null argument");
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     // one untimed pass always runs first: it sizes the scratch, which must not happen while capturing
-    for (size_t i = 0; i < std::max<size_t>(warmup, 1); i++)
-        W4_TRY(w4a16_chain_forward(ctx, prefix, 0, n_layers, x_dev, t, y_dev));
+    auto pass = [&]() {
+        return fused ? w4a16_chain_forward_fused(ctx, prefix, 0, n_layers, x_dev, t, y_dev)
+                     : w4a16_chain_forward(ctx, prefix, 0, n_layers, x_dev, t, y_dev);
+    };
+    for (size_t i = 0; i < std::max<size_t>(warmup, 1); i++) W4_TRY(pass());
     W4_TRY(w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"));
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
@@ -143,7 +197,7 @@ extern "C" int w4a16_bench_chain(w4a16_ctx* ctx, const char* prefix, size_t n_la
     if (use_graph) {
         rc = w4_hip(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
         if (!rc) {
-            int frc = w4a16_chain_forward(ctx, prefix, 0, n_layers, x_dev, t, y_dev);
+            int frc = pass();
             const std::string keep = w4_err_save();
             rc = w4_hip(hipStreamEndCapture(ctx->stream, &graph), "hipStreamEndCapture");
             if (frc) {
@@ -161,8 +215,7 @@ extern "C" int w4a16_bench_chain(w4a16_ctx* ctx, const char* prefix, size_t n_la
     auto w0 = std::chrono::steady_clock::now();
     if (!rc) rc = w4_hip(hipEventRecord(e0, ctx->stream), "hipEventRecord");
     for (size_t i = 0; i < reps && !rc; i++)
-        rc = use_graph ? w4_hip(hipGraphLaunch(exec, ctx->stream), "hipGraphLaunch")
-                       : w4a16_chain_forward(ctx, prefix, 0, n_layers, x_dev, t, y_dev);
+        rc = use_graph ? w4_hip(hipGraphLaunch(exec, ctx->stream), "hipGraphLaunch") : pass();
     if (!rc) rc = w4_hip(hipEventRecord(e1, ctx->stream), "hipEventRecord");
     if (!rc) rc = w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
     auto w1 = std::chrono::steady_clock::now();

@@ -49,6 +49,8 @@ struct W4MoeScratch {
 struct W4ChainScratch {
     uint64_t y32 = 0, h16a = 0, h16b = 0, ping[2] = {0, 0};
     size_t y32_cap = 0, h16a_cap = 0, h16b_cap = 0, ping_cap[2] = {0, 0};
+    uint64_t a16 = 0, stats[3] = {0, 0, 0};  // fused chain: f16 qkv output, partial sums of squares per stage
+    size_t a16_cap = 0, stats_cap[3] = {0, 0, 0};
 };
 
 struct w4a16_event {

@@ -90,7 +90,34 @@ static int decode_split(w4a16_ctx* ctx, const W4Lin& L, size_t t, size_t blocks,
     return 0;
 }
 
-static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16) {
+// RMS normalisation deferred across a decode launch (kernels/decode.hip): the input's 1/rms comes from the partial
+// sums of squares its producer left (stats_in, n_stats_in entries of 16 floats) and multiplies the output; the
+// launch leaves its own partial sums over output rows below stat_rows in stats_out.  Zero pointers switch either off.
+struct DecodeNorm {
+    size_t ldx = 0;  // halves between x rows, 0 = k
+    uint64_t stats_in = 0;
+    size_t n_stats_in = 0, in_cols = 0;
+    uint64_t stats_out = 0;
+    size_t stat_rows = 0;
+    size_t n_stats_out = 0;  // set by the launch: entries written to stats_out
+};
+
+static unsigned decode_stats_lds(const DecodeNorm& nm) {
+    return nm.stats_in ? (unsigned)std::min<size_t>((nm.n_stats_in + 63) / 64, 8) * 1024u : 0u;
+}
+
+static int check_decode_norm(const W4Lin& L, size_t t, const DecodeNorm& nm) {
+    const size_t ldx = nm.ldx ? nm.ldx : L.k;
+    if (ldx < L.k || ldx % 8 != 0) return w4_fail(W4A16_ERR_SHAPE, "decode: ldx=%zu must be a multiple of 8 and >= k=%zu", ldx, L.k);
+    if (((t - 1) * ldx + L.k) * 2 >= 0x80000000ull) return w4_fail(W4A16_ERR_SHAPE, "decode: x reaches 2 GiB");
+    if (nm.stats_in && (nm.n_stats_in == 0 || nm.n_stats_in > 0x7fffffffu / 16 || nm.in_cols == 0))
+        return w4_fail(W4A16_ERR_ARG, "decode: input statistics need n_stats_in and in_cols (got %zu, %zu)", nm.n_stats_in, nm.in_cols);
+    if (nm.stats_out && nm.stat_rows == 0) return w4_fail(W4A16_ERR_ARG, "decode: output statistics over zero rows");
+    return 0;
+}
+
+static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16,
+                         DecodeNorm* norm = nullptr) {
     if (t == 0 || t > 16) return w4_fail(W4A16_ERR_SHAPE, "decode: t=%zu outside 1..16", t);
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode: linear has no tiled copy (needs k %% 128 == 0)");
     int rb = 0, waves = 0;
@@ -110,16 +137,25 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     // launch geometry as kernel arguments (the kernel reads nothing from the dispatch packet): k tiles per slice and
     // per wave, both rounded up
     int kt_per_slice = (int)ceil_div(L.k / 128, (size_t)nks), kt_per_wave = (kt_per_slice + waves - 1) / waves;
-    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave};
+    DecodeNorm none;
+    DecodeNorm& nm = norm ? *norm : none;
+    W4_TRY(check_decode_norm(L, t, nm));
+    int ldx = (int)(nm.ldx ? nm.ldx : L.k), n_in = (int)nm.n_stats_in, stat_rows = (int)std::min<size_t>(nm.stat_rows, L.n);
+    float inv_cols = nm.in_cols ? 1.0f / (float)nm.in_cols : 0.0f;
+    uint64_t s_in = nm.stats_in, s_out = nm.stats_out;
+    nm.n_stats_out = s_out ? std::min(blocks, (size_t)ceil_div((size_t)stat_rows, (size_t)rb * 16)) : 0;
+    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
+                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows};
     // LDS: the split-K partial tiles [waves][rb][1 KiB], then two scale slots per wave; a slot holds the scales of
     // one ring round (rb x depth x groups-per-tile x 32 bytes, ring never deeper than 8 tiles) rounded up to 512
     const unsigned slot = ((unsigned)(rb * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
-    const unsigned shmem = (unsigned)(waves * rb * 1024) + (unsigned)waves * 2u * slot;
+    // ... then the staging area of the input statistics: 1 KiB per 64 entries, at most 8
+    const unsigned shmem = (unsigned)(waves * rb * 1024) + (unsigned)waves * 2u * slot + decode_stats_lds(nm);
     return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);
 }
 
 // Fused gate|up projection with the SiLU*up epilogue (decode regime): y f16 [t][n/2].
-static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t) {
+static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, DecodeNorm* norm = nullptr) {
     if (t == 0 || t > 16) return w4_fail(W4A16_ERR_SHAPE, "decode glu: t=%zu outside 1..16", t);
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode glu: linear has no tiled copy (needs k %% 128 == 0)");
     if (L.n % 32 != 0) return w4_fail(W4A16_ERR_SHAPE, "decode glu: n=%zu must be a multiple of 32 (gate and up halves of whole row blocks)", L.n);
@@ -138,9 +174,17 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
     W4_TRY(decode_split(ctx, L, t, blocks, 2, &waves, &nks));
     uint64_t ws = ctx->decode_ws, tk = ctx->decode_tickets;
     int kt_per_slice = (kt_n + nks - 1) / nks, kt_per_wave = (kt_per_slice + waves - 1) / waves;
-    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave};
+    DecodeNorm none;
+    DecodeNorm& nm = norm ? *norm : none;
+    W4_TRY(check_decode_norm(L, t, nm));
+    if (nm.stats_out) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode glu: the gated output carries no statistics");
+    int ldx = (int)(nm.ldx ? nm.ldx : L.k), n_in = (int)nm.n_stats_in, stat_rows = 0;
+    float inv_cols = nm.in_cols ? 1.0f / (float)nm.in_cols : 0.0f;
+    uint64_t s_in = nm.stats_in, s_out = 0;
+    void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
+                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows};
     const unsigned slot = ((unsigned)(2 * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
-    const unsigned shmem = (unsigned)(waves * 2 * 1024) + (unsigned)waves * 2u * slot;
+    const unsigned shmem = (unsigned)(waves * 2 * 1024) + (unsigned)waves * 2u * slot + decode_stats_lds(nm);
     return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);
 }
 
@@ -452,6 +496,42 @@ extern "C" int w4a16_lin_forward_glu(w4a16_ctx* ctx, const char* name, uint64_t 
     if (!x_dev || !y_f16_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_glu %s: null operand or t=0", name);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t);
+}
+
+extern "C" int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
+                                               uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_dev,
+                                               int out_f16, uint64_t stats_out_dev, size_t stat_rows,
+                                               size_t* n_stats_out) {
+    W4Lin* L = nullptr;
+    W4_TRY(w4_find_lin(ctx, name, &L));
+    if (!x_dev || !y_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_deferred_norm %s: null operand or t=0", name);
+    if (stats_out_dev && !n_stats_out) return w4_fail(W4A16_ERR_ARG, "lin_forward_deferred_norm %s: n_stats_out is null", name);
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    DecodeNorm nm;
+    nm.ldx = ldx;
+    nm.stats_in = stats_in_dev;
+    nm.n_stats_in = n_stats_in;
+    nm.in_cols = in_cols;
+    nm.stats_out = stats_out_dev;
+    nm.stat_rows = stat_rows;
+    W4_TRY(launch_decode(ctx, *L, x_dev, y_dev, t, out_f16, &nm));
+    if (n_stats_out) *n_stats_out = nm.n_stats_out;
+    return 0;
+}
+
+extern "C" int w4a16_lin_forward_glu_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
+                                                   uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols,
+                                                   uint64_t y_f16_dev) {
+    W4Lin* L = nullptr;
+    W4_TRY(w4_find_lin(ctx, name, &L));
+    if (!x_dev || !y_f16_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_glu_deferred_norm %s: null operand or t=0", name);
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    DecodeNorm nm;
+    nm.ldx = ldx;
+    nm.stats_in = stats_in_dev;
+    nm.n_stats_in = n_stats_in;
+    nm.in_cols = in_cols;
+    return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t, &nm);
 }
 
 extern "C" int w4a16_lin_forward_host(w4a16_ctx* ctx, const char* name, const uint16_t* x_f16, void* y, size_t t,

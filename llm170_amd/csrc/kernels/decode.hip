@@ -54,7 +54,9 @@ template <int G, bool SBF, int RB, int DEPTH, int XL, bool GLU = false>
 __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                             const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
                                             int k, int n, int t, int out_f16, f4_t* ws, int* tickets, int W, int nks,
-                                            int kt_per_slice, int kt_per_wave) {
+                                            int kt_per_slice, int kt_per_wave, int ldx,
+                                            const float* __restrict__ stats_in, int n_stats_in, float inv_cols_in,
+                                            float* __restrict__ stats_out, int stat_rows) {
     extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K, then [W][2][AUXB] scale slots
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
     constexpr int AUXB = RB * DEPTH * GPT * 32;      // bytes of scales one ring round needs: [rb][tile][group][16 rows]
@@ -82,9 +84,9 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     // predicates token columns >= t without a branch.
     // x load l of a tile: lane (m, g) fetches, for token m % TPL, the 8 halves of chunk l*C + m / TPL at k offset g*8
     const int xtok = m % TPL, xchunk = m / TPL;
-    const unsigned xoff = xtok < t ? ((unsigned)xtok * (unsigned)k + (unsigned)(xchunk * 32 + g * 8)) * 2u : W4_OOB;
+    const unsigned xoff = xtok < t ? ((unsigned)xtok * (unsigned)ldx + (unsigned)(xchunk * 32 + g * 8)) * 2u : W4_OOB;
     const unsigned q_bytes = (unsigned)row_blocks * (unsigned)kt_n * 1024u, s_bytes = (unsigned)row_blocks * (unsigned)kg_n * 32u,
-                   x_bytes = (unsigned)t * (unsigned)k * 2u;
+                   x_bytes = ((unsigned)(t - 1) * (unsigned)ldx + (unsigned)k) * 2u;  // x rows are ldx halves apart
     f4_t acc[RB];
     unsigned qoff[RB];
 #pragma unroll
@@ -172,6 +174,50 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
         }
     };
 
+    // Deferred RMS normalisation of the input (the linear commutes with a per-row factor): the launch that produced x
+    // left n_stats_in partial sums of squares per row, [n_stats_in][16] floats.  Wave 0 turns them into this lane's
+    // 1/sqrt(mean + 1e-6).  The entries of token columns 0..3 are fetched here, ahead of the ring, by LDS DMA (no
+    // registers held across the fill) into a staging area behind the scale slots, 64 entries per instruction, lane l
+    // entry c*64 + l; once the first weight tiles are in flight lane l adds its entries, a butterfly adds the lanes
+    // (fixed order: the same bits on every run), and the factor is parked in the wave's own slot of `red`, which the
+    // in-block reduction never writes.  The epilogue multiplies the sums by it.  Further token quads and entries
+    // beyond the staging area (8 x 64) repeat the fetch inside input_scale.
+    typedef __attribute__((address_space(3))) char lds_char_t;
+    lds_char_t* const stage_lds = (lds_char_t*)(reinterpret_cast<char*>(red) + W * RB * 1024 + W * (2 * SLOT));
+    const int stat_chunks = min((n_stats_in + 63) >> 6, 8);
+    auto fetch_stats = [&](int c0, int qd) {
+        const __amdgpu_buffer_rsrc_t sr_in = w4_make_rsrc(stats_in, (unsigned)n_stats_in * 64u);
+        for (int c = 0; c < stat_chunks; c++)  // entries past n_stats_in read as zeros
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(sr_in, (__attribute__((address_space(3))) void*)(stage_lds + c * 1024), 16,
+                                                     (unsigned)((c0 + c) * 64 + lane) * 64u + (unsigned)qd * 16u, 0, 0, 0);
+    };
+    if (stats_in != nullptr && wave == 0) fetch_stats(0, 0);
+    auto input_scale = [&]() {
+        const f4_t* const staged = reinterpret_cast<const f4_t*>(reinterpret_cast<char*>(red) + W * RB * 1024 + W * (2 * SLOT));
+        float mine = 0.f;
+        for (int qd = 0; qd * 4 < t; qd++) {  // a quad of token columns at a time
+            f4_t sum = {0.f, 0.f, 0.f, 0.f};
+            for (int c0 = 0; c0 * 64 < n_stats_in; c0 += 8) {
+                if (qd > 0 || c0 > 0) {
+                    fetch_stats(c0, qd);
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                } else {
+                    // the first fetch is older than the fill's loads (scales, then DEPTH stages): wait for it alone
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AUXN + DEPTH * (RB + XL) < 63 ? AUXN + DEPTH * (RB + XL) : 63) : "memory");
+                }
+                for (int c = 0; c < stat_chunks; c++) sum += staged[c * 64 + lane];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float v = sum[j];
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+                if (m == qd * 4 + j) mine = v;
+            }
+        }
+        reinterpret_cast<float*>(red)[lane] = (float)(1.0 / sqrt((double)mine * (double)inv_cols_in + 1e-6));
+    };
+
     // One counted loop does the pipeline fill (round -1, compute skipped) and the steady state, so on every path
     // into a stage's compute the outstanding loads are in ring order and the wait can leave the younger stages' loads
     // in flight (s_waitcnt vmcnt(N > 0)).  Tiles past kt1 load zeros and are never computed; the last partial round
@@ -195,6 +241,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
         }
         store_aux((r + 1) & 1);
         __builtin_amdgcn_sched_barrier(0);
+        if (r == -1 && stats_in != nullptr && wave == 0) input_scale();  // behind the first ring loads, once
     }
     {
         const char* sc = sc0 + (rounds & 1) * SLOT;
@@ -249,6 +296,28 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
             acc[rb] = sum;
         }
         if (lane == 0) __hip_atomic_store(tickets + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    }
+    if (stats_in != nullptr) {
+        const float inv = reinterpret_cast<const float*>(red)[lane];
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[rb][i] *= inv;
+    }
+    if (!GLU && stats_out != nullptr) {
+        // this block's share of the rows' sums of squares (rows below stat_rows only), for the launch that consumes y
+        float p = 0.f;
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = (nb0 + rb) * 16 + 4 * g + i;
+                if (nb0 + rb < row_blocks && row < stat_rows) p = __builtin_fmaf(acc[rb][i], acc[rb][i], p);
+            }
+        }
+        p += __shfl_xor(p, 16);
+        p += __shfl_xor(p, 32);
+        if (g == 0 && m < t) stats_out[blockIdx.x * 16 + m] = p;
     }
     if (m >= t) return;
     if (GLU) {
@@ -308,19 +377,26 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                                                         const uint16_t* x, void* y, int row_blocks,  \
                                                                         int k, int n, int t, int out_f16, f4_t* ws,  \
                                                                         int* tickets, int waves, int nks,            \
-                                                                        int kt_per_slice, int kt_per_wave) {         \
-        decode_body<G, SBF, RB, DECODE_DEPTH(BUDGET, G, RB, XL), XL>(qt, st, x, y, row_blocks, k, n, t, out_f16, ws, \
-                                                                     tickets, waves, nks, kt_per_slice, kt_per_wave); \
+                                                                        int kt_per_slice, int kt_per_wave, int ldx,  \
+                                                                        const float* stats_in, int n_stats_in,       \
+                                                                        float inv_cols_in, float* stats_out,         \
+                                                                        int stat_rows) {                             \
+        decode_body<G, SBF, RB, DECODE_DEPTH(BUDGET, G, RB, XL), XL>(                                                \
+            qt, st, x, y, row_blocks, k, n, t, out_f16, ws, tickets, waves, nks, kt_per_slice, kt_per_wave, ldx,     \
+            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows);                                                \
     }
 #define DECODE_GLU_KERNEL_X(NAME, G, SBF, XL, BUDGET, ATTR)                                                           \
     extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
                                                                         const uint16_t* x, void* y, int row_blocks,  \
                                                                         int k, int n, int t, int out_f16, f4_t* ws,  \
                                                                         int* tickets, int waves, int nks,            \
-                                                                        int kt_per_slice, int kt_per_wave) {         \
-        decode_body<G, SBF, 2, DECODE_DEPTH(BUDGET, G, 2, XL), XL, true>(qt, st, x, y, row_blocks, k, n, t, out_f16,  \
-                                                                         ws, tickets, waves, nks, kt_per_slice,      \
-                                                                         kt_per_wave);                               \
+                                                                        int kt_per_slice, int kt_per_wave, int ldx,  \
+                                                                        const float* stats_in, int n_stats_in,       \
+                                                                        float inv_cols_in, float* stats_out,         \
+                                                                        int stat_rows) {                             \
+        decode_body<G, SBF, 2, DECODE_DEPTH(BUDGET, G, 2, XL), XL, true>(                                            \
+            qt, st, x, y, row_blocks, k, n, t, out_f16, ws, tickets, waves, nks, kt_per_slice, kt_per_wave, ldx,     \
+            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows);                                                \
     }
 #define DECODE_HI __attribute__((amdgpu_waves_per_eu(6, 6)))
 #define DECODE_MID __attribute__((amdgpu_waves_per_eu(5, 5)))

@@ -194,6 +194,20 @@ class W4a16Dec:
         """Fused gate|up projection with the SiLU*up epilogue: y f16 [t][n/2]."""
         ffi.check(self.cc.lib.w4a16_lin_forward_glu(self.cc.h, name.encode(), x_dev, y_f16_dev, t))
 
+    def lin_forward_deferred_norm(self, name, x_dev, t, y_dev, out_f16=False, ldx=0, stats_in=0, n_stats_in=0, in_cols=0,
+                                  stats_out=0, stat_rows=0):
+        """y = s * (W x) with s = 1/rms of the input from its producer's partial sums; returns the number of partial
+        sums this launch wrote to stats_out (0 without one)."""
+        n_out = C.c_size_t(0)
+        ffi.check(self.cc.lib.w4a16_lin_forward_deferred_norm(self.cc.h, name.encode(), x_dev, ldx, t, stats_in, n_stats_in,
+                                                              in_cols, y_dev, int(out_f16), stats_out, stat_rows,
+                                                              C.byref(n_out)))
+        return n_out.value
+
+    def lin_forward_glu_deferred_norm(self, name, x_dev, t, y_f16_dev, ldx=0, stats_in=0, n_stats_in=0, in_cols=0):
+        ffi.check(self.cc.lib.w4a16_lin_forward_glu_deferred_norm(self.cc.h, name.encode(), x_dev, ldx, t, stats_in,
+                                                                  n_stats_in, in_cols, y_f16_dev))
+
     def gemv_host(self, name, x, t=1, out_f16=False, path=PATH_AUTO):
         """Host operands in, host result out: y [t][n] (f32, or f16 bit patterns when out_f16)."""
         spec = self.lin_spec(name)
@@ -342,10 +356,14 @@ class W4a16Dec:
         """chain_device_body (w4a16_dec/chains.rs:195-304) reduced to its linears and glue."""
         ffi.check(self.cc.lib.w4a16_chain_forward(self.cc.h, prefix.encode(), layer0, n_layers, x_dev, t, y_dev))
 
-    def bench_chain(self, prefix, n_layers, x_dev, t, y_dev, reps, warmup=1, use_graph=False):
+    def chain_forward_fused(self, prefix, layer0, n_layers, x_dev, t, y_dev):
+        """The chain with its normalisations deferred across the linears: four launches per layer, t <= 16."""
+        ffi.check(self.cc.lib.w4a16_chain_forward_fused(self.cc.h, prefix.encode(), layer0, n_layers, x_dev, t, y_dev))
+
+    def bench_chain(self, prefix, n_layers, x_dev, t, y_dev, reps, warmup=1, use_graph=False, fused=False):
         ms, wall = C.c_float(), C.c_double()
         ffi.check(self.cc.lib.w4a16_bench_chain(self.cc.h, prefix.encode(), n_layers, x_dev, t, y_dev, warmup, reps,
-                                                int(use_graph), C.byref(ms), C.byref(wall)))
+                                                int(use_graph), int(fused), C.byref(ms), C.byref(wall)))
         return ms.value, wall.value
 
 

@@ -313,3 +313,30 @@ def chain_layer(x, lins, group=128, threads=1):
     st["d"] = gemm_lane(st["c"], t, q3, s3, n3, k3, group, False, threads)
     st["x"] = rms_rescale_f16(st["d"], hidden)
     return st
+
+
+def rms_inv(v, ncols):
+    """Per row: f32(1 / sqrt(mean(v[:, :ncols]^2) + 1e-6)), the mean taken in f64 (the factor rms_rescale_f16 applies)."""
+    v64 = _c(v, np.float32)[:, :ncols].astype(np.float64)
+    return (1.0 / np.sqrt(np.mean(v64 * v64, axis=1) + 1e-6)).astype(np.float32)
+
+
+def chain_layer_fused(x, s_in, lins, group=128, threads=1):
+    """chain_layer with each normalisation applied after the linear that follows it: x f16 bits [t][hidden] travel
+    un-normalised, s_in f32 [t] is the factor they still lack (ones for a normalised input).  Every product is one f32
+    rounding.  Returns the stage values {v1, a, v2, b, gu, c, v4, x, s}: x = f16(v4), s = rms_inv(v4)."""
+    x = _c(x, np.uint16)
+    t, hidden = x.shape
+    s_in = _c(s_in, np.float32).reshape(t, 1)
+    (q0, s0, n0, k0), (q1, s1, n1, k1), (q2, s2, n2, k2), (q3, s3, n3, k3) = lins
+    st = {}
+    st["v1"] = (s_in * gemm_lane(x, t, q0, s0, n0, k0, group, False, threads)[:, :hidden]).astype(np.float32)
+    st["a"] = f32_to_f16_array(st["v1"]).reshape(t, -1)
+    st["v2"] = (rms_inv(st["v1"], hidden).reshape(t, 1) * gemm_lane(st["a"], t, q1, s1, n1, k1, group, False, threads)).astype(np.float32)
+    st["b"] = f32_to_f16_array(st["v2"]).reshape(t, -1)
+    st["gu"] = (rms_inv(st["v2"], hidden).reshape(t, 1) * gemm_lane(st["b"], t, q2, s2, n2, k2, group, False, threads)).astype(np.float32)
+    st["c"] = silu_mul_f16_rows(st["gu"])
+    st["v4"] = gemm_lane(st["c"], t, q3, s3, n3, k3, group, False, threads)
+    st["x"] = f32_to_f16_array(st["v4"]).reshape(t, -1)
+    st["s"] = rms_inv(st["v4"], hidden)
+    return st

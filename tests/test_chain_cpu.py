@@ -76,3 +76,56 @@ def test_chain_layer_against_float64(orc):
     want = rms(c @ w[3].T)
     got = _f16(st["x"])
     assert np.linalg.norm(got - want) / np.linalg.norm(want) < 3e-3  # four f16 roundings of intermediates
+
+
+def test_rms_inv_against_float64_and_rms_rescale(orc):
+    rng = np.random.default_rng(8)
+    v = (rng.standard_normal((4, 700)) * rng.uniform(0.05, 30, (4, 1))).astype(np.float32)
+    v[:, 500:] = 1e5  # columns past ncols stay out of the mean
+    inv = orc.rms_inv(v, 500)
+    v64 = v[:, :500].astype(np.float64)
+    want = 1.0 / np.sqrt(np.mean(v64 * v64, axis=1) + 1e-6)
+    assert inv.dtype == np.float32 and np.allclose(inv, want, rtol=1e-6)
+    # it is the factor rms_rescale_f16 applies: f16(v * inv) agrees with it to a rounding flip
+    a = _f16(orc.rms_rescale_f16(v, 500))
+    b = (v[:, :500] * inv[:, None]).astype(np.float32).astype(np.float16).astype(np.float64)
+    assert np.mean(a == b) > 0.999 and np.all(np.abs(a - b) <= _step(a))
+    # a constant row of 3s: mean square 9
+    assert np.allclose(orc.rms_inv(np.full((1, 64), 3.0, np.float32), 64), 1.0 / 3.0, rtol=1e-6)
+
+
+def test_chain_layer_fused_against_float64_and_unfused(orc):
+    """The deferred statement is the same function of x as chain_layer: the factor of a stage's input commutes with the
+    linear.  Checked against float64 and against the unfused oracle, with an un-normalised input and its factor."""
+    hidden, n_qkv, n_ff, g, t = 256, 384, 512, 128, 3
+    shapes = [(n_qkv, hidden), (hidden, hidden), (2 * n_ff, hidden), (hidden, n_ff)]
+    lins = []
+    for i, (n, k) in enumerate(shapes):
+        q = gen.weights_q(gen.shape_seed(n, k, tensor=50 + i), n, k)
+        s = gen.scales_f16(gen.shape_seed(n, k, tensor=60 + i), n, k, g)
+        lins.append((q, s, n, k))
+    rng = np.random.default_rng(2)
+    v0 = (rng.standard_normal((t, hidden)) * np.array([[0.3], [5.0], [40.0]])).astype(np.float32)  # un-normalised rows
+    x_un = orc.f32_to_f16_array(v0).reshape(t, hidden)
+    s0 = orc.rms_inv(v0, hidden)
+    st = orc.chain_layer_fused(x_un, s0, lins, g)
+    w = [orc.dequant_matrix(q, s, n, k, g).astype(np.float64) for (q, s, n, k) in lins]
+    rms = lambda v: v / np.sqrt(np.mean(v * v, axis=1, keepdims=True) + 1e-6)
+    a = rms((rms(v0.astype(np.float64)) @ w[0].T)[:, :hidden])
+    b = rms(a @ w[1].T)
+    gu = b @ w[2].T
+    c = gu[:, :n_ff] / (1.0 + np.exp(-gu[:, :n_ff])) * gu[:, n_ff:]
+    want = rms(c @ w[3].T)
+    got = st["v4"].astype(np.float64) * st["s"].astype(np.float64)[:, None]
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) < 3e-3
+    # each stage's activations carry the scale of a normalised input (about 4 here), not of x
+    assert np.all(np.abs(np.sqrt(np.mean(st["v1"].astype(np.float64) ** 2, axis=1)) / np.sqrt(np.mean((rms(v0.astype(np.float64)) @ w[0].T)[:, :hidden] ** 2, axis=1)) - 1) < 1e-2)
+    # against the unfused oracle fed the normalised input
+    x_n = orc.rms_rescale_f16(v0, hidden)
+    un = _f16(orc.chain_layer(x_n, lins, g)["x"])
+    assert np.linalg.norm(un - want) / np.linalg.norm(want) < 3e-3
+    fused_x = _f16(orc.rms_rescale_f16(st["v4"], hidden))
+    assert np.linalg.norm(fused_x - un) / np.linalg.norm(un) < 5e-3
+    # forgetting the factor of the input changes v1 by far more than rounding
+    wrong = orc.chain_layer_fused(x_un, np.ones(t, np.float32), lins, g)
+    assert np.linalg.norm(wrong["v1"] - st["v1"]) / np.linalg.norm(st["v1"]) > 0.5

@@ -231,6 +231,148 @@ def test_chain_errors(dec):
         dec.chain_forward("brk", 0, 1, 1, 1, 1)
 
 
+# ------------------------------------------------------------------ normalisation deferred across a linear
+@pytest.mark.parametrize("t,group", [(1, 128), (4, 128), (6, 128), (16, 128), (3, 32)])
+def test_deferred_norm_linear(dec, orc, t, group):
+    """y = s * (W x) with s from the producer's partial sums, x a column slice of a wider matrix, and the launch's own
+    partial sums over the first stat_rows outputs — for every launch shape; bits repeat from run to run."""
+    n, k, ldx, stat_rows, in_cols, n_in = 400, 1024, 1536, 300, 777, 7
+    q, s, _ = gen.make_linear(n, k, group, 1, seed=21 + t)
+    dec.upload_lin_g("dn", q, s, n, k, group, False)
+    xw = gen.normal_f16(5 + t, (t, ldx))
+    x = np.ascontiguousarray(xw[:, :k])
+    rng = np.random.default_rng(t)
+    prev = (rng.standard_normal((n_in, 16)) ** 2 * 100).astype(np.float32)
+    s_in = (1.0 / np.sqrt(prev.astype(np.float64).sum(0)[:t] / in_cols + 1e-6)).astype(np.float32)
+    lane = orc.gemm_lane(x, t, q, s, n, k, group, False, 4)
+    want = (s_in[:, None] * lane).astype(np.float32)
+    cc = dec.cc
+    cap = ((n + 15) // 16) * 64
+    px, pp, py, ps = cc.to_device(xw), cc.to_device(prev), cc.alloc(t * n * 4), cc.alloc(cap)
+    try:
+        for rows, waves in ((0, 0), (16, 4), (32, 8), (64, 2), (16, 1)):
+            say("deferred norm", t, group, rows, waves)
+            dec.set_decode_shape(rows, waves)
+            cc.memset0(ps, cap)
+            n_out = dec.lin_forward_deferred_norm("dn", px, t, py, ldx=ldx, stats_in=pp, n_stats_in=n_in, in_cols=in_cols,
+                                                  stats_out=ps, stat_rows=stat_rows)
+            y = cc.d2h(py, (t, n), np.float32)
+            st = cc.d2h(ps, (n_out, 16), np.float32)
+            parity.assert_close(y, want, "deferred norm t%d rows%d waves%d" % (t, rows, waves))
+            assert 1 <= n_out <= (n + 15) // 16
+            got_ss = st.astype(np.float64).sum(0)[:t]
+            want_ss = (y[:, :stat_rows].astype(np.float64) ** 2).sum(1)  # the launch's own outputs
+            assert np.all(np.abs(got_ss / want_ss - 1.0) < 1e-5)
+            # f16 output: the scaled f32 value rounded once
+            n2 = dec.lin_forward_deferred_norm("dn", px, t, py, out_f16=True, ldx=ldx, stats_in=pp, n_stats_in=n_in,
+                                               in_cols=in_cols, stats_out=ps, stat_rows=stat_rows)
+            y16 = cc.d2h(py, (t, n), np.uint16)
+            assert n2 == n_out and np.array_equal(y16, gen.f32_to_f16_bits(y))
+            assert np.array_equal(cc.d2h(ps, (n_out, 16), np.float32)[:, :t], st[:, :t])  # same bits every run
+        dec.set_decode_shape(0, 0)
+        # without statistics either way it is the plain decode launch
+        dec.lin_forward_deferred_norm("dn", px, t, py, ldx=ldx)
+        plain = dec.gemv_host("dn", x, t=t, path=ops.PATH_DECODE)
+        assert np.array_equal(cc.d2h(py, (t, n), np.float32).view(np.uint32), plain.view(np.uint32))
+    finally:
+        dec.set_decode_shape(0, 0)
+        for p_ in (px, pp, py, ps):
+            cc.free(p_)
+
+
+def test_deferred_norm_many_partial_sums_and_glu(dec, orc):
+    """More partial sums than one staging pass holds (8 x 64 entries), and the gated projection: the factor reaches
+    gate and up before silu(g) * u."""
+    n, k, t, n_in, in_cols = 512, 512, 5, 700, 4096
+    q, s, x = gen.make_linear(n, k, 128, t, seed=77)
+    dec.upload_lin_g("dg", q, s, n, k, 128, False)
+    prev = (np.random.default_rng(9).standard_normal((n_in, 16)) ** 2).astype(np.float32)
+    s_in = (1.0 / np.sqrt(prev.astype(np.float64).sum(0)[:t] / in_cols + 1e-6)).astype(np.float32)
+    gu = (s_in[:, None] * orc.gemm_lane(x, t, q, s, n, k, 128, False, 4)).astype(np.float32)
+    cc = dec.cc
+    px, pp, py, pc = cc.to_device(x), cc.to_device(prev), cc.alloc(t * n * 4), cc.alloc(t * (n // 2) * 2)
+    try:
+        dec.lin_forward_deferred_norm("dg", px, t, py, stats_in=pp, n_stats_in=n_in, in_cols=in_cols)
+        parity.assert_close(cc.d2h(py, (t, n), np.float32), gu, "deferred norm, 700 partial sums")
+        dec.lin_forward_glu_deferred_norm("dg", px, t, pc, stats_in=pp, n_stats_in=n_in, in_cols=in_cols)
+        c = cc.d2h(pc, (t, n // 2), np.uint16)
+        cw = orc.silu_mul_f16_rows(gu)
+        assert np.all(np.abs(_f16(c).astype(np.float64) - _f16(cw)) <= parity.f16_ulp(_f16(cw)))
+        with pytest.raises(ops.W4a16Error):  # x rows closer together than k
+            dec.lin_forward_deferred_norm("dg", px, t, py, ldx=k - 8)
+        with pytest.raises(ops.W4a16Error):  # statistics without their count
+            dec.lin_forward_deferred_norm("dg", px, t, py, stats_in=pp, n_stats_in=0, in_cols=in_cols)
+        with pytest.raises(ops.W4a16Error):  # decode regime only
+            dec.lin_forward_deferred_norm("dg", px, 17, py)
+    finally:
+        for p_ in (px, pp, py, pc):
+            cc.free(p_)
+
+
+def _fused_oracle(orc, prefix, seeds, shapes, group, layers, x, threads):
+    cur, sc = x, np.ones(x.shape[0], np.float32)
+    for l in range(layers):
+        st = orc.chain_layer_fused(cur, sc, _host_lins(seeds, prefix, l, shapes, group), group, threads)
+        cur, sc = st["x"], st["s"]
+    return orc.rms_rescale_f16(st["v4"], shapes["attn_output"][0])
+
+
+@pytest.mark.parametrize("t", [1, 4, 13])
+def test_fused_chain_small_many_layers(dec, orc, t):
+    """24 small layers with the normalisations deferred across the linears: close to the oracle's statement of the
+    same chain and to the chain that keeps the normalisation launches; graph replays repeat the eager bits."""
+    say("fused chain small", t)
+    hidden, n_qkv, n_ff, group, layers = 256, 384, 512, 128, 24
+    shapes = {"attn_qkv": (n_qkv, hidden), "attn_output": (hidden, hidden), "ffn_gate_up": (2 * n_ff, hidden),
+              "ffn_down": (hidden, n_ff)}
+    seeds = dec.upload_chain_synth("fsmall", layers, hidden, n_qkv, n_ff, group)
+    x = gen.normal_f16(131 + t, (t, hidden))
+    cc = dec.cc
+    px, py, pz = cc.to_device(x), cc.alloc(t * hidden * 2), cc.alloc(t * hidden * 2)
+    try:
+        dec.chain_forward_fused("fsmall", 0, layers, px, t, py)
+        got = cc.d2h(py, (t, hidden), np.uint16)
+        want = _fused_oracle(orc, "fsmall", seeds, shapes, group, layers, x, 4)
+        m = parity.compare(_f16(got), _f16(want))
+        say("  fused vs oracle rel_l2", m["rel_l2"])
+        assert m["rel_l2"] < 2e-2  # rounding flips of f16 intermediates accumulate over 96 linears
+        dec.chain_forward("fsmall", 0, layers, px, t, pz)
+        m2 = parity.compare(_f16(got), _f16(cc.d2h(pz, (t, hidden), np.uint16)))
+        say("  fused vs unfused rel_l2", m2["rel_l2"])
+        assert m2["rel_l2"] < 2e-2
+        for _ in range(2):
+            dec.chain_forward_fused("fsmall", 0, layers, px, t, py)
+            assert np.array_equal(cc.d2h(py, (t, hidden), np.uint16), got)  # deterministic
+        dec.bench_chain("fsmall", layers, px, t, py, reps=3, warmup=1, use_graph=True, fused=True)
+        assert np.array_equal(cc.d2h(py, (t, hidden), np.uint16), got)  # graph replays give the same bits
+        with pytest.raises(ops.W4a16Error):
+            dec.chain_forward_fused("fsmall", 0, layers, px, 17, py)
+    finally:
+        for p_ in (px, py, pz):
+            cc.free(p_)
+
+
+def test_fused_chain_27b_layer_shapes(dec, orc):
+    """Two layers at the 27B-dense shapes, M = 4: stage by stage against the oracle's fused statement on the device's
+    own inputs would repeat test_deferred_norm_linear; here the end-to-end result against the oracle."""
+    hidden, n_qkv, n_ff, group, layers, t = 5120, 7168, 17408, 128, 2, 4
+    shapes = {"attn_qkv": (n_qkv, hidden), "attn_output": (hidden, hidden), "ffn_gate_up": (2 * n_ff, hidden),
+              "ffn_down": (hidden, n_ff)}
+    seeds = dec.upload_chain_synth("f27", layers, hidden, n_qkv, n_ff, group)
+    x = gen.normal_f16(4, (t, hidden))
+    cc = dec.cc
+    px, py = cc.to_device(x), cc.alloc(t * hidden * 2)
+    say("fused chain 27b")
+    dec.chain_forward_fused("f27", 0, layers, px, t, py)
+    got = cc.d2h(py, (t, hidden), np.uint16)
+    cc.free(px)
+    cc.free(py)
+    want = _fused_oracle(orc, "f27", seeds, shapes, group, layers, x, 16)
+    m = parity.compare(_f16(got), _f16(want))
+    say("  rel_l2", m["rel_l2"], "identical", float(np.mean(got == want)))
+    assert m["rel_l2"] < 3e-3
+
+
 # ------------------------------------------------------------------ norm_resid (assets/norm.cu:4-48, 97-148)
 @pytest.mark.parametrize("t,hidden,w_off", [(1, 5120, 0), (4, 5120, 5120), (7, 2048, 0), (3, 1000, 24), (2, 8192, 0),
                                             (5, 64, 0)])
