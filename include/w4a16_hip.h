@@ -161,10 +161,17 @@ int w4a16_lin_forward_glu(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint
  * stats_out_dev != 0: the launch writes *n_stats_out entries [i][16] of partial sums of y[r][c]^2 (the f32 values,
  * before any rounding to f16) over columns c < stat_rows; the buffer must hold ceil(n / 16) entries of 64 bytes.
  * A chain of such launches needs no normalisation launch between its linears: the f16 activations travel
- * un-normalised (same relative precision), every consumer applies the factor. */
+ * un-normalised (same relative precision), every consumer applies the factor.
+ * The rest of norm_resid belongs to the producer and is folded into the same launch when the pointers are non-zero:
+ *   resid_dev  f32 [t][n], the residual stream: v = resid + y is written back to it (norm.cu:11-13), the statistics are
+ *              those of v, and v is what continues;
+ *   nw_dev     f32 [n], the norm weight of the output rows (norm.cu:19-23): y_dev receives v * nw.
+ * The consumer's output is then 1/rms(v) * W2 (v * nw), the reference's W2 (v * 1/rms(v) * nw) with the f16 rounding
+ * of the activations taken before the 1/rms factor instead of after it. */
 int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
                                     uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_dev,
-                                    int out_f16, uint64_t stats_out_dev, size_t stat_rows, size_t* n_stats_out);
+                                    int out_f16, uint64_t stats_out_dev, size_t stat_rows, size_t* n_stats_out,
+                                    uint64_t resid_dev, uint64_t nw_dev);
 /* The same for the fused gate|up projection: the factor multiplies gate and up before silu(g) * u. */
 int w4a16_lin_forward_glu_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
                                         uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_f16_dev);

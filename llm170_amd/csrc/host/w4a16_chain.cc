@@ -162,16 +162,16 @@ extern "C" int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, siz
         size_t n_a = 0, n_b = 0, n_d = 0;
         // a = qkv(x)[:, :hidden], its statistics over those columns only
         W4_TRY(w4a16_lin_forward_deferred_norm(ctx, nm[0], cur, 0, t, n_prev ? S.stats[2] : 0, n_prev, hidden, S.a16, 1,
-                                               S.stats[0], hidden, &n_a));
+                                               S.stats[0], hidden, &n_a, 0, 0));
         W4_TRY(w4a16_lin_forward_deferred_norm(ctx, nm[1], S.a16, n_qkv, t, S.stats[0], n_a, hidden, S.h16a, 1, S.stats[1],
-                                               hidden, &n_b));
+                                               hidden, &n_b, 0, 0));
         W4_TRY(w4a16_lin_forward_glu_deferred_norm(ctx, nm[2], S.h16a, 0, t, S.stats[1], n_b, hidden, S.h16b));
         if (last) {
             // the chain's output is normalised: one launch per call, not per layer
             W4_TRY(w4a16_lin_forward(ctx, nm[3], S.h16b, S.y32, t, 0, W4A16_PATH_DECODE));
             W4_TRY(w4a16_rms_rescale_f16(ctx, S.y32, hidden, hidden, t, y_dev));
         } else {
-            W4_TRY(w4a16_lin_forward_deferred_norm(ctx, nm[3], S.h16b, 0, t, 0, 0, 0, S.ping[0], 1, S.stats[2], hidden, &n_d));
+            W4_TRY(w4a16_lin_forward_deferred_norm(ctx, nm[3], S.h16b, 0, t, 0, 0, 0, S.ping[0], 1, S.stats[2], hidden, &n_d, 0, 0));
             cur = S.ping[0];
             n_prev = n_d;
         }

@@ -100,6 +100,8 @@ struct DecodeNorm {
     uint64_t stats_out = 0;
     size_t stat_rows = 0;
     size_t n_stats_out = 0;  // set by the launch: entries written to stats_out
+    uint64_t resid = 0;      // f32 [t][n] residual stream, takes the output: v = resid + y, written back
+    uint64_t nw = 0;         // f32 [n] norm weight of the output rows, multiplies what y_dev receives
 };
 
 static unsigned decode_stats_lds(const DecodeNorm& nm) {
@@ -142,10 +144,10 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     W4_TRY(check_decode_norm(L, t, nm));
     int ldx = (int)(nm.ldx ? nm.ldx : L.k), n_in = (int)nm.n_stats_in, stat_rows = (int)std::min<size_t>(nm.stat_rows, L.n);
     float inv_cols = nm.in_cols ? 1.0f / (float)nm.in_cols : 0.0f;
-    uint64_t s_in = nm.stats_in, s_out = nm.stats_out;
+    uint64_t s_in = nm.stats_in, s_out = nm.stats_out, resid = nm.resid, nw = nm.nw;
     nm.n_stats_out = s_out ? std::min(blocks, (size_t)ceil_div((size_t)stat_rows, (size_t)rb * 16)) : 0;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
-                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows};
+                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw};
     // LDS: the split-K partial tiles [waves][rb][1 KiB], then two scale slots per wave; a slot holds the scales of
     // one ring round (rb x depth x groups-per-tile x 32 bytes, ring never deeper than 8 tiles) rounded up to 512
     const unsigned slot = ((unsigned)(rb * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
@@ -177,12 +179,13 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
     DecodeNorm none;
     DecodeNorm& nm = norm ? *norm : none;
     W4_TRY(check_decode_norm(L, t, nm));
-    if (nm.stats_out) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode glu: the gated output carries no statistics");
+    if (nm.stats_out || nm.resid || nm.nw)
+        return w4_fail(W4A16_ERR_UNSUPPORTED, "decode glu: the gated output takes no statistics, residual or norm weight");
     int ldx = (int)(nm.ldx ? nm.ldx : L.k), n_in = (int)nm.n_stats_in, stat_rows = 0;
     float inv_cols = nm.in_cols ? 1.0f / (float)nm.in_cols : 0.0f;
-    uint64_t s_in = nm.stats_in, s_out = 0;
+    uint64_t s_in = nm.stats_in, s_out = 0, resid = 0, nw = 0;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
-                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows};
+                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw};
     const unsigned slot = ((unsigned)(2 * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
     const unsigned shmem = (unsigned)(waves * 2 * 1024) + (unsigned)waves * 2u * slot + decode_stats_lds(nm);
     return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);
@@ -501,7 +504,7 @@ extern "C" int w4a16_lin_forward_glu(w4a16_ctx* ctx, const char* name, uint64_t 
 extern "C" int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
                                                uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_dev,
                                                int out_f16, uint64_t stats_out_dev, size_t stat_rows,
-                                               size_t* n_stats_out) {
+                                               size_t* n_stats_out, uint64_t resid_dev, uint64_t nw_dev) {
     W4Lin* L = nullptr;
     W4_TRY(w4_find_lin(ctx, name, &L));
     if (!x_dev || !y_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_deferred_norm %s: null operand or t=0", name);
@@ -514,6 +517,8 @@ extern "C" int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name,
     nm.in_cols = in_cols;
     nm.stats_out = stats_out_dev;
     nm.stat_rows = stat_rows;
+    nm.resid = resid_dev;
+    nm.nw = nw_dev;
     W4_TRY(launch_decode(ctx, *L, x_dev, y_dev, t, out_f16, &nm));
     if (n_stats_out) *n_stats_out = nm.n_stats_out;
     return 0;

@@ -56,7 +56,8 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                             int k, int n, int t, int out_f16, f4_t* ws, int* tickets, int W, int nks,
                                             int kt_per_slice, int kt_per_wave, int ldx,
                                             const float* __restrict__ stats_in, int n_stats_in, float inv_cols_in,
-                                            float* __restrict__ stats_out, int stat_rows) {
+                                            float* __restrict__ stats_out, int stat_rows, float* __restrict__ resid,
+                                            const float* __restrict__ nw) {
     extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K, then [W][2][AUXB] scale slots
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
     constexpr int AUXB = RB * DEPTH * GPT * 32;      // bytes of scales one ring round needs: [rb][tile][group][16 rows]
@@ -304,6 +305,24 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[rb][i] *= inv;
     }
+    // The element-wise part of the reference's norm_resid (assets/norm.cu:9-23) that belongs to the producer of an
+    // activation: the residual stream takes the linear's output (v = resid + y, written back) and, after the
+    // statistics of v, the norm weight of each output row multiplies what the next linear will read.
+    if (!GLU && resid != nullptr && m < t) {
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = (nb0 + rb) * 16 + 4 * g + i;
+                if (nb0 + rb < row_blocks && row < n) {
+                    float* const rp = resid + (size_t)m * n + row;
+                    const float v = *rp + acc[rb][i];
+                    *rp = v;
+                    acc[rb][i] = v;
+                }
+            }
+        }
+    }
     if (!GLU && stats_out != nullptr) {
         // this block's share of the rows' sums of squares (rows below stat_rows only), for the launch that consumes y
         float p = 0.f;
@@ -318,6 +337,16 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
         p += __shfl_xor(p, 16);
         p += __shfl_xor(p, 32);
         if (g == 0 && m < t) stats_out[blockIdx.x * 16 + m] = p;
+    }
+    if (!GLU && nw != nullptr) {
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = (nb0 + rb) * 16 + 4 * g + i;
+                if (nb0 + rb < row_blocks && row < n) acc[rb][i] *= nw[row];
+            }
+        }
     }
     if (m >= t) return;
     if (GLU) {
@@ -380,10 +409,11 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                                                         int kt_per_slice, int kt_per_wave, int ldx,  \
                                                                         const float* stats_in, int n_stats_in,       \
                                                                         float inv_cols_in, float* stats_out,         \
-                                                                        int stat_rows) {                             \
+                                                                        int stat_rows, float* resid,                 \
+                                                                        const float* nw) {                           \
         decode_body<G, SBF, RB, DECODE_DEPTH(BUDGET, G, RB, XL), XL>(                                                \
             qt, st, x, y, row_blocks, k, n, t, out_f16, ws, tickets, waves, nks, kt_per_slice, kt_per_wave, ldx,     \
-            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows);                                                \
+            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw);                                     \
     }
 #define DECODE_GLU_KERNEL_X(NAME, G, SBF, XL, BUDGET, ATTR)                                                           \
     extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
@@ -393,10 +423,11 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                                                         int kt_per_slice, int kt_per_wave, int ldx,  \
                                                                         const float* stats_in, int n_stats_in,       \
                                                                         float inv_cols_in, float* stats_out,         \
-                                                                        int stat_rows) {                             \
+                                                                        int stat_rows, float* resid,                 \
+                                                                        const float* nw) {                           \
         decode_body<G, SBF, 2, DECODE_DEPTH(BUDGET, G, 2, XL), XL, true>(                                            \
             qt, st, x, y, row_blocks, k, n, t, out_f16, ws, tickets, waves, nks, kt_per_slice, kt_per_wave, ldx,     \
-            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows);                                                \
+            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw);                                     \
     }
 #define DECODE_HI __attribute__((amdgpu_waves_per_eu(6, 6)))
 #define DECODE_MID __attribute__((amdgpu_waves_per_eu(5, 5)))

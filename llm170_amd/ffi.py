@@ -50,7 +50,7 @@ _SIGS = {
     "w4a16_lin_forward_glu": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_size_t]),
     "w4a16_lin_forward_deferred_norm": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64,
                                                   C.c_size_t, C.c_size_t, C.c_uint64, C.c_int, C.c_uint64, C.c_size_t,
-                                                  C.POINTER(C.c_size_t)]),
+                                                  C.POINTER(C.c_size_t), C.c_uint64, C.c_uint64]),
     "w4a16_lin_forward_glu_deferred_norm": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_size_t, C.c_size_t,
                                                       C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64]),
     "w4a16_lin_forward_host": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int]),

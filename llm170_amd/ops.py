@@ -195,13 +195,13 @@ class W4a16Dec:
         ffi.check(self.cc.lib.w4a16_lin_forward_glu(self.cc.h, name.encode(), x_dev, y_f16_dev, t))
 
     def lin_forward_deferred_norm(self, name, x_dev, t, y_dev, out_f16=False, ldx=0, stats_in=0, n_stats_in=0, in_cols=0,
-                                  stats_out=0, stat_rows=0):
+                                  stats_out=0, stat_rows=0, resid=0, nw=0):
         """y = s * (W x) with s = 1/rms of the input from its producer's partial sums; returns the number of partial
         sums this launch wrote to stats_out (0 without one)."""
         n_out = C.c_size_t(0)
         ffi.check(self.cc.lib.w4a16_lin_forward_deferred_norm(self.cc.h, name.encode(), x_dev, ldx, t, stats_in, n_stats_in,
                                                               in_cols, y_dev, int(out_f16), stats_out, stat_rows,
-                                                              C.byref(n_out)))
+                                                              C.byref(n_out), resid, nw))
         return n_out.value
 
     def lin_forward_glu_deferred_norm(self, name, x_dev, t, y_f16_dev, ldx=0, stats_in=0, n_stats_in=0, in_cols=0):

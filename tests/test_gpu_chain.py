@@ -309,6 +309,48 @@ def test_deferred_norm_many_partial_sums_and_glu(dec, orc):
             cc.free(p_)
 
 
+@pytest.mark.parametrize("t", [1, 4, 11])
+def test_deferred_norm_with_residual_and_norm_weight(dec, orc, t):
+    """Two linears with a norm_resid between them (x += ab; xn = x * inv * nw; y = W2 xn16, kernels/mod.rs:11-54),
+    as two launches: the first adds its output to the residual stream, leaves the statistics of the sum and emits
+    f16(v * nw); the second multiplies by 1/rms(v).  Residual stream and statistics against the oracle of the first
+    linear; the final result against the reference sequence (oracle linears around the oracle's norm_resid)."""
+    hidden, n2, k1, group = 640, 272, 512, 128
+    q1, s1, x = gen.make_linear(hidden, k1, group, t, seed=300 + t)
+    q2, s2, _ = gen.make_linear(n2, hidden, group, 1, seed=310 + t)
+    dec.upload_lin_g("nr1", q1, s1, hidden, k1, group, False)
+    dec.upload_lin_g("nr2", q2, s2, n2, hidden, group, False)
+    rng = np.random.default_rng(40 + t)
+    resid0 = (rng.standard_normal((t, hidden)) * 3).astype(np.float32)
+    nw = (1.0 + 0.3 * rng.standard_normal(hidden)).astype(np.float32)
+    # reference sequence
+    ab = orc.gemm_lane(x, t, q1, s1, hidden, k1, group, False, 4)
+    ref_x, _, _, ref_xn16 = orc.norm_resid(resid0, nw, ab)
+    want = orc.gemm_lane(ref_xn16, t, q2, s2, n2, hidden, group, False, 4)
+    cc = dec.cc
+    cap = ((hidden + 15) // 16) * 64
+    px, pr, pw = cc.to_device(x), cc.to_device(resid0), cc.to_device(nw)
+    pa, ps, py = cc.alloc(t * hidden * 2), cc.alloc(cap), cc.alloc(t * n2 * 4)
+    try:
+        n_st = dec.lin_forward_deferred_norm("nr1", px, t, pa, out_f16=True, stats_out=ps, stat_rows=hidden, resid=pr, nw=pw)
+        v = cc.d2h(pr, (t, hidden), np.float32)
+        parity.assert_close(v, ref_x, "residual stream t%d" % t)
+        a16 = cc.d2h(pa, (t, hidden), np.uint16)
+        assert np.array_equal(a16, gen.f32_to_f16_bits((v * nw[None, :]).astype(np.float32)))  # one f32 product, one rounding
+        ss = cc.d2h(ps, (n_st, 16), np.float32).astype(np.float64).sum(0)[:t]
+        assert np.all(np.abs(ss / (v.astype(np.float64) ** 2).sum(1) - 1.0) < 1e-5)
+        dec.lin_forward_deferred_norm("nr2", pa, t, py, stats_in=ps, n_stats_in=n_st, in_cols=hidden)
+        got = cc.d2h(py, (t, n2), np.float32)
+        m = parity.compare(got, want)
+        say("  norm_resid deferred t", t, "rel_l2", m["rel_l2"])
+        assert m["rel_l2"] < 1e-3  # the f16 rounding of the activations falls before the 1/rms factor instead of after
+        with pytest.raises(ops.W4a16Error):  # the gated projection takes neither
+            dec.lin_forward_glu_deferred_norm("nr1", px, t, pa, stats_in=ps, n_stats_in=0, in_cols=hidden)
+    finally:
+        for p_ in (px, pr, pw, pa, ps, py):
+            cc.free(p_)
+
+
 def _fused_oracle(orc, prefix, seeds, shapes, group, layers, x, threads):
     cur, sc = x, np.ones(x.shape[0], np.float32)
     for l in range(layers):
