@@ -270,12 +270,23 @@ def test_deferred_norm_linear(dec, orc, t, group):
             assert n2 == n_out and np.array_equal(y16, gen.f32_to_f16_bits(y))
             assert np.array_equal(cc.d2h(ps, (n_out, 16), np.float32)[:, :t], st[:, :t])  # same bits every run
         dec.set_decode_shape(0, 0)
+        # split over k across workgroups: the workgroup that adds the slices applies the factor and leaves the sums
+        dec.set_decode_ksplit(2)
+        cc.memset0(ps, cap)
+        n_out = dec.lin_forward_deferred_norm("dn", px, t, py, ldx=ldx, stats_in=pp, n_stats_in=n_in, in_cols=in_cols,
+                                              stats_out=ps, stat_rows=stat_rows)
+        y = cc.d2h(py, (t, n), np.float32)
+        parity.assert_close(y, want, "deferred norm t%d, two k slices" % t)
+        got_ss = cc.d2h(ps, (n_out, 16), np.float32).astype(np.float64).sum(0)[:t]
+        assert np.all(np.abs(got_ss / (y[:, :stat_rows].astype(np.float64) ** 2).sum(1) - 1.0) < 1e-5)
+        dec.set_decode_ksplit(0)
         # without statistics either way it is the plain decode launch
         dec.lin_forward_deferred_norm("dn", px, t, py, ldx=ldx)
         plain = dec.gemv_host("dn", x, t=t, path=ops.PATH_DECODE)
         assert np.array_equal(cc.d2h(py, (t, n), np.float32).view(np.uint32), plain.view(np.uint32))
     finally:
         dec.set_decode_shape(0, 0)
+        dec.set_decode_ksplit(0)
         for p_ in (px, pp, py, ps):
             cc.free(p_)
 
@@ -332,6 +343,7 @@ def test_deferred_norm_with_residual_and_norm_weight(dec, orc, t):
     px, pr, pw = cc.to_device(x), cc.to_device(resid0), cc.to_device(nw)
     pa, ps, py = cc.alloc(t * hidden * 2), cc.alloc(cap), cc.alloc(t * n2 * 4)
     try:
+        cc.memset0(ps, cap)  # token columns >= t are never written
         n_st = dec.lin_forward_deferred_norm("nr1", px, t, pa, out_f16=True, stats_out=ps, stat_rows=hidden, resid=pr, nw=pw)
         v = cc.d2h(pr, (t, hidden), np.float32)
         parity.assert_close(v, ref_x, "residual stream t%d" % t)
