@@ -259,7 +259,7 @@ int w4a16_moe_align(w4a16_ctx* ctx, uint64_t idx_dev, size_t ns, size_t n_exp, s
  *               -> y[token] = sum over the token's slots of c2, in slot order, f32.
  *   x_dev f16 [t][h]; idx_dev int32 [t*top_k]; wt_dev f32 [t*top_k]; y_dev f32 [t][h].
  * Scratch (sorted ids, act, c2) is owned by the context and grown on demand.
- * For t <= 12 and top_k <= 8 the call runs in direct mode: no alignment, the gate|up GEMM takes one segment per slot and
+ * For t <= 15 and top_k <= 8 the call runs in direct mode: no alignment, the gate|up GEMM takes one segment per slot and
  * one more launch does the down projections of a token's experts, the weight multiply, the f16 rounding of c2 and
  * the slot-order sum (same values, c2 never reaches memory). */
 int w4a16_moe_ffn(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t idx_dev, uint64_t wt_dev, size_t t,

@@ -197,7 +197,7 @@ int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes) {
     return 0;
 }
 
-// Segment size (slots of one expert per workgroup).  Up to 12 tokens (top_k <= 8) skip the alignment; otherwise up to 8
+// Segment size (slots of one expert per workgroup).  Up to 15 tokens (top_k <= 8) skip the alignment; otherwise up to 8
 // tokens run the streaming kernel on 16-slot segments; beyond that the LDS-staged kernel, whose segment size follows
 // the mean run per expert: 32 slots below a mean of 24, 48 below 40, else 64.  The reference picks the smallest of
 // 16/32/48/64 that the mean run fills to under 90 % (kernels/marlin_moe.rs:309-315); measured here (128 experts,
@@ -206,9 +206,9 @@ int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes) {
 static size_t pick_block(const w4a16_ctx* ctx, size_t t, size_t ns, size_t n_exp, size_t top_k) {
     if (ctx->moe_block) return (size_t)ctx->moe_block;
     // direct mode (no alignment, two launches, see w4a16_moe_ffn): streams an expert once per token that chose it,
-    // which still beats the two extra launches up to a dozen tokens (128 experts, top-8: 39.6 vs 52.9 us at t = 8,
-    // 56.8 vs 61.3 us at t = 12, 70.7 vs 65.5 us at t = 16)
-    if (t <= 12 && top_k <= 8) return 1;
+    // which still beats the two extra launches up to fifteen tokens (128 experts, top-8: 35.6 vs 52.9 us at t = 8,
+    // 49.3 vs 61.3 us at t = 12, 62.9 vs 64.7 us at t = 15, level at t = 16, 79.3 vs 65.4 us at t = 20)
+    if (t <= 15 && top_k <= 8) return 1;
     if (t <= 4) return 4;
     if (t <= 8) return 16;
     const double mean = (double)ns / (double)n_exp;
