@@ -395,8 +395,9 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
 // (a deep-ring build at three waves per SIMD ran the grid in two uneven generations: 4.6 -> 5.0 TB/s at M = 1).
 //   HI: ring sized for 24 VGPRs of load buffers, amdgpu_waves_per_eu(6,6)   — variants that fit 80 VGPRs unspilled
 //   MID: the same ring at five waves per SIMD (<= 102 VGPRs)
-//   LO: ring sized for 64 VGPRs, occupancy left to the compiler             — the wide variants (4 row blocks, 4 x
-//       loads) and group size 32
+//   LO: occupancy left to the compiler — the wide variants (4 row blocks, 4 x loads) and group size 32; their ring
+//       is as short (a 64-register ring measured 11-18 % slower at group 32, M <= 4: 20.7 -> 18.4 us on the
+//       5120 x 34816 shape, 14.8 -> 12.4 us on 17408 x 5120, and no faster anywhere)
 #define DECODE_STAGE_REGS(G, RB, XL) (4 * RB + 4 * XL)
 #define DECODE_DEPTH(BUDGET, G, RB, XL) \
     ((BUDGET / DECODE_STAGE_REGS(G, RB, XL)) < 2 ? 2 : (BUDGET / DECODE_STAGE_REGS(G, RB, XL)) > 8 ? 8 : (BUDGET / DECODE_STAGE_REGS(G, RB, XL)))
@@ -441,8 +442,8 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     DECODE_KERNEL_X(NAME, 128, SBF, 2, 1, 24, DECODE_HI) DECODE_KERNEL_X(NAME, 128, SBF, 2, 2, 24, DECODE_MID) \
     DECODE_KERNEL_X(NAME, 128, SBF, 2, 4, 64, DECODE_LO)
 #define DECODE_KERNEL_LO3(NAME, G, SBF, RB)                                                   \
-    DECODE_KERNEL_X(NAME, G, SBF, RB, 1, 64, DECODE_LO) DECODE_KERNEL_X(NAME, G, SBF, RB, 2, 64, DECODE_LO) \
-    DECODE_KERNEL_X(NAME, G, SBF, RB, 4, 64, DECODE_LO)
+    DECODE_KERNEL_X(NAME, G, SBF, RB, 1, 24, DECODE_LO) DECODE_KERNEL_X(NAME, G, SBF, RB, 2, 24, DECODE_LO) \
+    DECODE_KERNEL_X(NAME, G, SBF, RB, 4, 24, DECODE_LO)
 
 DECODE_KERNEL_RB1(w4a16_decode_g128_f16_rb1, 128, false)
 DECODE_KERNEL_RB2_G128(w4a16_decode_g128_f16_rb2, false)
@@ -461,8 +462,8 @@ DECODE_KERNEL_LO3(w4a16_decode_g32_bf16_rb4, 32, true, 4)
     DECODE_GLU_KERNEL_X(NAME, 128, SBF, 1, 24, DECODE_HI) DECODE_GLU_KERNEL_X(NAME, 128, SBF, 2, 24, DECODE_MID) \
     DECODE_GLU_KERNEL_X(NAME, 128, SBF, 4, 64, DECODE_LO)
 #define DECODE_GLU_G32(NAME, SBF)                                                                    \
-    DECODE_GLU_KERNEL_X(NAME, 32, SBF, 1, 64, DECODE_LO) DECODE_GLU_KERNEL_X(NAME, 32, SBF, 2, 64, DECODE_LO) \
-    DECODE_GLU_KERNEL_X(NAME, 32, SBF, 4, 64, DECODE_LO)
+    DECODE_GLU_KERNEL_X(NAME, 32, SBF, 1, 24, DECODE_LO) DECODE_GLU_KERNEL_X(NAME, 32, SBF, 2, 24, DECODE_LO) \
+    DECODE_GLU_KERNEL_X(NAME, 32, SBF, 4, 24, DECODE_LO)
 DECODE_GLU_G128(w4a16_decode_g128_f16_glu, false)
 DECODE_GLU_G128(w4a16_decode_g128_bf16_glu, true)
 DECODE_GLU_G32(w4a16_decode_g32_f16_glu, false)
