@@ -639,12 +639,13 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
         moe_mm_body<G, SBF, GLU, TT, DEPTH, KS>(MOE_ARGS);                            \
     }
 // Ring depths, from sweeps on the 128-expert shape: the one-slot segments of the direct mode run best with two k tiles
-// in flight per wave (T = 4..12: 9-11 % faster than four: fewer registers, more waves resident at once).
+// in flight per wave (T = 4..12: 9-11 % faster than four: fewer registers, more waves resident at once); so do the
+// segments of up to 16 slots (5 % faster than three).
 #define MOE_FAMILY(PFX, G, SBF, DMM)                             \
     MOE_DEC_KERNEL(PFX##_dec_glu_x1, G, SBF, true, 1, 2)     \
-    MOE_DEC_KERNEL(PFX##_dec_glu_x4, G, SBF, true, 4, 3)     \
+    MOE_DEC_KERNEL(PFX##_dec_glu_x4, G, SBF, true, 4, 2)     \
     MOE_DEC_KERNEL(PFX##_dec_lin_x1, G, SBF, false, 1, 2)    \
-    MOE_DEC_KERNEL(PFX##_dec_lin_x4, G, SBF, false, 4, 3)    \
+    MOE_DEC_KERNEL(PFX##_dec_lin_x4, G, SBF, false, 4, 2)    \
     MOE_MM_KERNEL(PFX##_mm_glu_t1, G, SBF, true, 1, DMM, false)    \
     MOE_MM_KERNEL(PFX##_mm_glu_t2, G, SBF, true, 2, DMM, false)    \
     MOE_MM_KERNEL(PFX##_mm_glu_t3, G, SBF, true, 3, DMM, false)    \
