@@ -425,6 +425,7 @@ struct MoeMmStage {
 // its kernels are built without the epilogue that costs them registers).
 template <int G, bool SBF, bool GLU, int TT, int DEPTH, bool KS>
 __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
+    static_assert(DEPTH % 2 == 0, "the x double buffer alternates with the ring position");
     extern __shared__ _Float16 xs[];  // [2][16*TT][MOE_LDX]
     constexpr int GPT = W4_TILE_K / G;
     constexpr int ROWS = 16 * TT;
@@ -640,8 +641,8 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     }
 // Ring depths, from sweeps on the 128-expert shape: the one-slot segments of the direct mode run best with two k tiles
 // in flight per wave (T = 4..12: 9-11 % faster than four: fewer registers, more waves resident at once); so do the
-// segments of up to 16 slots (5 % faster than three).  The LDS-staged kernels keep two (group 32) or three (group 128;
-// a dense linear at 17..64 rows runs 4-5 % faster than with four).
+// segments of up to 16 slots (5 % faster than three).  The LDS-staged kernels keep two (group 32) or four (group 128);
+// their ring depth must be even (the x double buffer alternates with the ring position).
 #define MOE_FAMILY(PFX, G, SBF, DMM)                             \
     MOE_DEC_KERNEL(PFX##_dec_glu_x1, G, SBF, true, 1, 2)     \
     MOE_DEC_KERNEL(PFX##_dec_glu_x4, G, SBF, true, 4, 2)     \
@@ -662,8 +663,8 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
 
 MOE_FAMILY(w4a16_moe_g32_f16, 32, false, 2)
 MOE_FAMILY(w4a16_moe_g32_bf16, 32, true, 2)
-MOE_FAMILY(w4a16_moe_g128_f16, 128, false, 3)
-MOE_FAMILY(w4a16_moe_g128_bf16, 128, true, 3)
+MOE_FAMILY(w4a16_moe_g128_f16, 128, false, 4)
+MOE_FAMILY(w4a16_moe_g128_bf16, 128, true, 4)
 
 // ---------------------------------------------------------------------------------------------------- routing
 // Softmax over all experts, k largest probabilities with ties to the lower index, weights renormalised by the
