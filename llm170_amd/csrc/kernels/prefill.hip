@@ -20,6 +20,11 @@
 //     that all eight XCDs get work).
 #include "w4a16_common.hpp"
 
+// s_prev / s_cur of a group boundary.  The accumulators only need a factor close to the quotient — whatever it is, it
+// is what the running unit is divided by, to within the rounding the multiply makes anyway — so the hardware
+// reciprocal (1 ulp) replaces the ten-instruction IEEE division: +2 % at group 128, +4.5 % at group 32 (M = 4096).
+__device__ __forceinline__ float pf_ratio(float s_prev, float s_cur) { return s_prev * __builtin_amdgcn_rcpf(s_cur); }
+
 #define PF_BN 256
 #define PF_KS 64          // k per LDS stage
 #define PF_LDA 64         // halves per staged x row (unpadded; chunks swizzled)
@@ -146,7 +151,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
 #pragma unroll
                     for (int ni = 0; ni < 2; ni++) {
                         const float s_cur = w4_scale_fast<SBF>(sc[ni][w]);
-                        ratio[ni] = unit[ni] / s_cur;
+                        ratio[ni] = pf_ratio(unit[ni], s_cur);
                         unit[ni] = s_cur;
                     }
                 }
@@ -165,7 +170,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
 #pragma unroll
                     for (int ni = 0; ni < 2; ni++) {
                         const float s_next = more ? w4_scale_fast<SBF>(scn[ni][0]) : unit[ni];
-                        next_ratio[ni] = unit[ni] / s_next;
+                        next_ratio[ni] = pf_ratio(unit[ni], s_next);
                         unit[ni] = s_next;
                     }
                 }
