@@ -103,10 +103,10 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
         for (int ni = 0; ni < 2; ni++) {
 #pragma unroll
             for (int h = 0; h < 2; h++)
-                dst[ni][h] = __builtin_amdgcn_raw_buffer_load_b128(qr, q_off[ni][h] + (unsigned)kt * 1024u, 0, 0);
+                dst[ni][h] = __builtin_amdgcn_raw_buffer_load_b128(qr, q_off[ni][h], kt * 1024, 0);  // k tile in the scalar offset
 #pragma unroll
             for (int gi = 0; gi < GPT; gi++)
-                sdst[ni][gi] = __builtin_amdgcn_raw_buffer_load_b16(sr, s_off[ni] + (unsigned)(kt * GPT + gi) * 32u, 0, 0);
+                sdst[ni][gi] = __builtin_amdgcn_raw_buffer_load_b16(sr, s_off[ni], (kt * GPT + gi) * 32, 0);
         }
     };
 
