@@ -264,6 +264,13 @@ int w4a16_moe_align(w4a16_ctx* ctx, uint64_t idx_dev, size_t ns, size_t n_exp, s
  * the slot-order sum (same values, c2 never reaches memory). */
 int w4a16_moe_ffn(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t idx_dev, uint64_t wt_dev, size_t t,
                   size_t top_k, uint64_t y_dev);
+/* The same with the activation chosen per call, the `gelu` flag of marlin_moe_ffn_dev (marlin_moe.rs:298, 372-376):
+ * W4A16_ACT_SILU = act[slot] = f16(silu(g) * u) (w4a16_moe_act_silu_f16), W4A16_ACT_GELU_TANH =
+ * f16(0.5 g (1 + tanh(0.7978846 (g + 0.044715 g^3))) * u) (w4a16_moe_act_gelu_f16, assets/moe.cu:1635-1647), g and u
+ * the gate and up sums rounded to f16, f32 arithmetic. */
+enum { W4A16_ACT_SILU = 0, W4A16_ACT_GELU_TANH = 1 };
+int w4a16_moe_ffn_act(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t idx_dev, uint64_t wt_dev, size_t t,
+                      size_t top_k, uint64_t y_dev, int act);
 /* Scratch of the last w4a16_moe_ffn call, for stage-by-stage checks (the reference exposes the same buffers to
  * its moe_selfcheck, w4a16_dec/probe.rs:153): which = 0 sorted ids (int32), 1 expert ids (int32), 2 num_post
  * (int32 [2]), 3 act (f16 [ns][n_ff]), 4 c2 (f16 [ns][h]).  Also reports the segment size used (1 = direct mode, where only

@@ -70,6 +70,7 @@ struct w4a16_ctx {
     W4MoeScratch moe;
     W4ChainScratch chain;
     int moe_block = 0, moe_waves = 0;  // 0 = automatic
+    int moe_act_kind = 0;              // activation of the expert FFN call in progress (W4A16_ACT_*)
     int decode_rows_per_wave = 0, decode_waves_per_block = 0;  // 0 = automatic
     int decode_ksplit = 0;                                      // 0 = automatic, -1 = never, n = exactly n k slices
     uint64_t decode_ws = 0, decode_tickets = 0;                 // partial tiles and per-block tickets of a split launch

@@ -229,8 +229,9 @@ static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_
         ki = (int)k, ni = (int)n, nei = (int)E.n_exp;
     uint64_t ws = 0, tk = 0;
     int waves = 0;  // set below, before the launch reads it
+    int act_kind = ctx->moe_act_kind;  // read by the gate|up kernels only
     void* p[] = {&qa, &sa, &qs, &ss, &x, &xr, &xd, &y, &yf, &topw, &sorted, &eids, &npost, &blk, &nsi, &rbi, &ki, &ni, &nei,
-                 &ws, &tk, &waves};
+                 &ws, &tk, &waves, &act_kind};
     char sym[80];
     const char* fam = E.scale_bf16 ? "bf16" : "f16";
     if (block <= 16) {
@@ -364,9 +365,17 @@ static int moe_ffn_direct(w4a16_ctx* ctx, const char* name, const W4Experts& E, 
 
 extern "C" int w4a16_moe_ffn(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t idx_dev, uint64_t wt_dev,
                              size_t t, size_t top_k, uint64_t y_dev) {
+    return w4a16_moe_ffn_act(ctx, name, x_dev, idx_dev, wt_dev, t, top_k, y_dev, W4A16_ACT_SILU);
+}
+
+extern "C" int w4a16_moe_ffn_act(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t idx_dev, uint64_t wt_dev,
+                                 size_t t, size_t top_k, uint64_t y_dev, int act) {
     W4Experts* E = nullptr;
     W4_TRY(find_experts(ctx, name, &E));
     if (!x_dev || !idx_dev || !wt_dev || !y_dev) return w4_fail(W4A16_ERR_ARG, "moe_ffn %s: null operand", name);
+    if (act != W4A16_ACT_SILU && act != W4A16_ACT_GELU_TANH)
+        return w4_fail(W4A16_ERR_ARG, "moe_ffn %s: activation %d (0 = silu, 1 = gelu, tanh form)", name, act);
+    ctx->moe_act_kind = act;  // read by the gate|up launches of this call
     if (t == 0 || top_k == 0 || top_k > E->n_exp || t > 0x3fffffffu / top_k)
         return w4_fail(W4A16_ERR_SHAPE, "moe_ffn %s: t=%zu top_k=%zu experts=%zu", name, t, top_k, E->n_exp);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));

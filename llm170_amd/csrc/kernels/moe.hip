@@ -65,14 +65,19 @@ __device__ __forceinline__ float moe_round_f16(float v) { return (float)(_Float1
 // LIN: rows of row blocks rbA / rbB, scaled by wgt, as f16 or f32.
 template <bool GLU>
 __device__ __forceinline__ void moe_store(f4_t a0, f4_t a1, int slot, int q, int u, int rbA, int rbB, bool haveB,
-                                          void* __restrict__ y, int y_f16, float wgt, int n) {
+                                          void* __restrict__ y, int y_f16, float wgt, int n, int act_kind) {
     if (GLU) {
         const int n_ff = n >> 1;
         h4_t o;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const float g = moe_round_f16(a0[i]), up = moe_round_f16(a1[i]);
-            o[i] = (_Float16)((g / (1.0f + expf(-g))) * up);
+            if (act_kind == 1) {  // uniform
+                const float x3 = g * g * g;
+                o[i] = (_Float16)((0.5f * g * (1.0f + tanhf(0.7978846f * (g + 0.044715f * x3)))) * up);
+            } else {
+                o[i] = (_Float16)((g / (1.0f + expf(-g))) * up);
+            }
         }
         *reinterpret_cast<h4_t*>(reinterpret_cast<_Float16*>(y) + (size_t)slot * n_ff + u * 16 + 4 * q) = o;
     } else {
@@ -113,6 +118,8 @@ __device__ __forceinline__ void moe_store(f4_t a0, f4_t a1, int slot, int q, int
 //   A segment whose expert id is outside 0..n_exp-1 is skipped (its slots stay unwritten).
 //   ws / tickets: workspace and zeroed counters of a launch split over k across workgroups (gridDim.y slices; the
 //   LDS-staged kernel only): [slice][block][wave][2*TT] partial tiles, one counter per (block, wave).
+//   act_kind (GLU only): 0 = silu(gate) * up (w4a16_moe_act_silu_f16), 1 = the tanh form of gelu on the gate
+//   (w4a16_moe_act_gelu_f16, assets/moe.cu:1635-1647).
 //   wpb: waves per block (the block size, as an argument: read from the dispatch packet it costs one more dependent
 //   scalar-cache miss before the first weight load).
 #define MOE_PARAMS                                                                                                  \
@@ -120,9 +127,9 @@ __device__ __forceinline__ void moe_store(f4_t a0, f4_t a1, int slot, int q, int
         unsigned long long s_stride, const uint16_t *__restrict__ x, int x_rows, int x_div, void *__restrict__ y,   \
         int y_f16, const float *__restrict__ topw, const int *__restrict__ sorted_ids,                              \
         const int *__restrict__ expert_ids, const int *__restrict__ num_post, int blk, int ns, int row_blocks, int k, \
-        int n, int n_exp, f4_t *ws, int *tickets, int wpb
+        int n, int n_exp, f4_t *ws, int *tickets, int wpb, int act_kind
 #define MOE_ARGS \
-    qa, sa, q_stride, s_stride, x, x_rows, x_div, y, y_f16, topw, sorted_ids, expert_ids, num_post, blk, ns, row_blocks, k, n, n_exp, ws, tickets, wpb
+    qa, sa, q_stride, s_stride, x, x_rows, x_div, y, y_f16, topw, sorted_ids, expert_ids, num_post, blk, ns, row_blocks, k, n, n_exp, ws, tickets, wpb, act_kind
 
 // ---------------------------------------------------------------------------------------------------- moe_dec
 template <int RB, int XL>
@@ -258,7 +265,7 @@ __device__ __forceinline__ void moe_dec_body(MOE_PARAMS) {
     const int slot = m < blk ? sorted_ids[seg * blk + m] : ns;
     if (slot >= ns) return;
     const float wgt = (!GLU && topw) ? topw[slot] : 1.0f;
-    moe_store<GLU>(acc[0], acc[1], slot, g, u, rbA, rbB, haveB, y, y_f16, wgt, n);
+    moe_store<GLU>(acc[0], acc[1], slot, g, u, rbA, rbB, haveB, y, y_f16, wgt, n, act_kind);
 }
 
 // ---------------------------------------------------------------------------------------------------- moe_down_sum
@@ -627,7 +634,7 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
         const int slot = sorted_ids[seg * blk + tt * 16 + c];
         if (slot >= ns) continue;
         const float wgt = (!GLU && topw) ? topw[slot] : 1.0f;
-        moe_store<GLU>(acc[0][tt], acc[1][tt], slot, q, u, rbA, rbB, haveB, y, y_f16, wgt, n);
+        moe_store<GLU>(acc[0][tt], acc[1][tt], slot, q, u, rbA, rbB, haveB, y, y_f16, wgt, n, act_kind);
     }
 }
 

@@ -8,6 +8,7 @@ LIB_PATH = os.path.join(PKG, "libw4a16hip.so")
 
 ERR_SHAPE, ERR_SYMBOL, ERR_UNSUPPORTED, ERR_NOT_FOUND, ERR_ARG, ERR_ASSET = 10001, 10002, 10003, 10004, 10005, 10006
 PATH_AUTO, PATH_LANE, PATH_DECODE, PATH_PREFILL, PATH_STREAM = 0, 1, 2, 3, 4
+ACT_SILU, ACT_GELU_TANH = 0, 1
 
 
 class W4a16Error(RuntimeError):
@@ -76,6 +77,8 @@ _SIGS = {
                                   C.c_uint64]),
     "w4a16_moe_ffn": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t, C.c_size_t,
                                 C.c_uint64]),
+    "w4a16_moe_ffn_act": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t, C.c_size_t,
+                                    C.c_uint64, C.c_int]),
     "w4a16_moe_scratch": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_size_t),
                                     C.POINTER(C.c_size_t)]),
     "w4a16_set_moe_shape": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),

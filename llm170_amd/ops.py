@@ -15,7 +15,7 @@ import ctypes as C
 import numpy as np
 
 from . import ffi
-from .ffi import PATH_AUTO, PATH_DECODE, PATH_LANE, PATH_PREFILL, PATH_STREAM, W4a16Error  # noqa: F401
+from .ffi import ACT_GELU_TANH, ACT_SILU, PATH_AUTO, PATH_DECODE, PATH_LANE, PATH_PREFILL, PATH_STREAM, W4a16Error  # noqa: F401
 
 
 def check_shapes(t, qlen, slen, xlen, n, k, group):
@@ -296,9 +296,12 @@ class W4a16Dec:
         ffi.check(self.cc.lib.w4a16_moe_align(self.cc.h, idx_dev, ns, n_exp, block, sorted_dev, expert_ids_dev,
                                               num_post_dev))
 
-    def moe_ffn(self, name, x_dev, idx_dev, wt_dev, t, top_k, y_dev):
-        """marlin_moe_ffn_dev (kernels/marlin_moe.rs:290-422)."""
-        ffi.check(self.cc.lib.w4a16_moe_ffn(self.cc.h, name.encode(), x_dev, idx_dev, wt_dev, t, top_k, y_dev))
+    def moe_ffn(self, name, x_dev, idx_dev, wt_dev, t, top_k, y_dev, gelu=False):
+        """marlin_moe_ffn_dev (kernels/marlin_moe.rs:290-422); gelu = its flag of the same name."""
+        if gelu:
+            ffi.check(self.cc.lib.w4a16_moe_ffn_act(self.cc.h, name.encode(), x_dev, idx_dev, wt_dev, t, top_k, y_dev, ACT_GELU_TANH))
+        else:
+            ffi.check(self.cc.lib.w4a16_moe_ffn(self.cc.h, name.encode(), x_dev, idx_dev, wt_dev, t, top_k, y_dev))
 
     def moe_scratch(self, which, dtype):
         """Scratch buffer of the last moe_ffn call as a flat numpy array, plus the segment size used."""

@@ -23,6 +23,8 @@
  *   orc_exact_dot ......... exact-rational brute force (quant/exact.rs:77-135 precedent)
  *   orc_moe_act_silu_f16 .. float64 evaluation of g/(1+exp(-g))*u within one f16 step; special cases g = 0, u = 0,
  *                           large |g| (silu -> g, -> 0)
+ *   orc_moe_act_gelu_f16 .. float64 evaluation of 0.5 g (1 + tanh(0.7978846 (g + 0.044715 g^3))) u within one f16 step;
+ *                           against the erf form of gelu to 1e-3; g = 0, large |g| (-> g, -> 0); swapped operands fail
  *   orc_moe_topk_sum_f16 .. numpy float32 sequential sum; exactly-summable inputs
  *   orc_moe_align ......... numpy stable argsort by expert + padding arithmetic; tiny hand-worked case
  *   orc_rms_rescale_f16 ... float64 v / sqrt(mean(v^2) + 1e-6) within one f16 step, >= 99.9 % identical; constant rows;
@@ -358,6 +360,23 @@ void orc_moe_act_silu_f16(const uint16_t* c13, size_t ns, size_t n_ff, uint16_t*
             const float g = orc_half_to_f32(c13[r * 2 * n_ff + c]);
             const float u = orc_half_to_f32(c13[r * 2 * n_ff + n_ff + c]);
             act[r * n_ff + c] = orc_silu_mul_f16(g, u);
+        }
+}
+
+/* ---- w4a16_moe_act_gelu_f16 (crates/backend-gpu/src/rawcuda/assets/moe.cu:1635-1647): the tanh form of gelu on the
+ * gate, times up, f32 arithmetic in the reference's order, one rounding to f16. ---- */
+uint16_t orc_gelu_mul_f16(float g, float u) {
+    const float x3 = g * g * g;
+    const float a = (0.5f * g * (1.0f + tanhf(0.7978846f * (g + 0.044715f * x3)))) * u;
+    return orc_f32_to_f16(a);
+}
+
+void orc_moe_act_gelu_f16(const uint16_t* c13, size_t ns, size_t n_ff, uint16_t* act) {
+    for (size_t r = 0; r < ns; r++)
+        for (size_t c = 0; c < n_ff; c++) {
+            const float g = orc_half_to_f32(c13[r * 2 * n_ff + c]);
+            const float u = orc_half_to_f32(c13[r * 2 * n_ff + n_ff + c]);
+            act[r * n_ff + c] = orc_gelu_mul_f16(g, u);
         }
 }
 

@@ -59,6 +59,7 @@ def lib():
         L.orc_norm_resid.argtypes, L.orc_norm_resid.restype = [f32p, f32p, f32p, f32p, f32p, u16p, sz, sz, sz], None
         i32p = C.POINTER(C.c_int32)
         L.orc_moe_act_silu_f16.argtypes, L.orc_moe_act_silu_f16.restype = [u16p, sz, sz, u16p], None
+        L.orc_moe_act_gelu_f16.argtypes, L.orc_moe_act_gelu_f16.restype = [u16p, sz, sz, u16p], None
         L.orc_moe_topk_sum_f16.argtypes, L.orc_moe_topk_sum_f16.restype = [u16p, sz, sz, sz, f32p], None
         L.orc_moe_align.argtypes, L.orc_moe_align.restype = [i32p, sz, sz, sz, i32p, i32p], sz
         _lib = L
@@ -205,6 +206,14 @@ def moe_act_silu_f16(c13, ns, n_ff):
     return act
 
 
+def moe_act_gelu_f16(c13, ns, n_ff):
+    """w4a16_moe_act_gelu_f16 (assets/moe.cu:1635-1647): f16 bits [ns][2*n_ff] -> f16 bits [ns][n_ff]."""
+    c13 = _c(c13, np.uint16).reshape(ns, 2 * n_ff)
+    act = np.empty((ns, n_ff), np.uint16)
+    lib().orc_moe_act_gelu_f16(_p(c13, C.c_uint16), ns, n_ff, _p(act, C.c_uint16))
+    return act
+
+
 def moe_topk_sum_f16(c2, t, h, top_k):
     c2 = _c(c2, np.uint16).reshape(t * top_k, h)
     out = np.empty((t, h), np.float32)
@@ -234,10 +243,10 @@ def moe_topk_batch(logits, k):
     return idx, w
 
 
-def moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, scale_bf16=False, threads=1, act_in=None):
+def moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, scale_bf16=False, threads=1, act_in=None, gelu=False):
     """The routed-expert FFN of the reference's device path (kernels/marlin_moe.rs:290-422) with every GEMM done by
     the lane contract: per slot j (token j // top_k, expert idx[j])
-        c13 = f16(lane(W13[e], x[token]));  act = f16(silu(gate) * up)
+        c13 = f16(lane(W13[e], x[token]));  act = f16(silu(gate) * up)   (gelu: the tanh form of gelu instead of silu)
         c2  = f16(wt[j] * lane(W2[e], act));  y[token] = sum_k c2 in slot order (f32).
     x: f16 bits [t][h]; idx int32 [t][top_k]; wt f32 [t][top_k]; q13 u32 [E][2*n_ff][h/8] ...
     act_in (f16 bits [ns][n_ff]) replaces the first stage's result when given (stage-wise checks).
@@ -259,7 +268,7 @@ def moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, scale_bf16=False, thre
             xs = x[slots // top_k]
             y13 = gemm_lane(xs, len(slots), q13[e], s13[e], 2 * n_ff, h, group, scale_bf16, threads)
             c13[slots] = f32_to_f16_array(y13).reshape(len(slots), 2 * n_ff)
-            act[slots] = moe_act_silu_f16(c13[slots], len(slots), n_ff)
+            act[slots] = (moe_act_gelu_f16 if gelu else moe_act_silu_f16)(c13[slots], len(slots), n_ff)
         y2 = gemm_lane(act[slots], len(slots), q2[e], s2[e], h, n_ff, group, scale_bf16, threads)
         y2 = (y2 * wflat[slots][:, None]).astype(np.float32)
         c2[slots] = f32_to_f16_array(y2).reshape(len(slots), h)

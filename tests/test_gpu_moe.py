@@ -109,10 +109,10 @@ def test_align_matches_oracle(dec, orc, ns, n_exp, block):
 
 
 # ------------------------------------------------------------------ the FFN, stage by stage and end to end
-def _run_ffn(dec, name, x, idx, wt, t, k, h):
+def _run_ffn(dec, name, x, idx, wt, t, k, h, gelu=False):
     cc = dec.cc
     px, pi, pw, py = cc.to_device(x), cc.to_device(idx), cc.to_device(wt), cc.alloc(t * h * 4)
-    dec.moe_ffn(name, px, pi, pw, t, k, py)
+    dec.moe_ffn(name, px, pi, pw, t, k, py, gelu=gelu)
     y = cc.d2h(py, (t, h), np.float32)
     ns = t * k
     spec = dec.experts_spec(name)
@@ -123,9 +123,13 @@ def _run_ffn(dec, name, x, idx, wt, t, k, h):
     return y, act.reshape(ns, spec["n_ff"]), c2, blk
 
 
-def _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, what, threads=8):
+def _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, what, threads=8, gelu=False):
     t, k = idx.shape
-    full = orc.moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, threads=threads)
+    full = orc.moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, threads=threads, gelu=gelu)
+    if gelu:
+        fn = lambda g1, u1: 0.5 * g1 * (1.0 + np.tanh(0.7978846 * (g1 + 0.044715 * g1 ** 3))) * u1
+    else:
+        fn = lambda g1, u1: g1 / (1.0 + np.exp(-g1)) * u1
     # stage 1: act against the oracle's act.  The device's gate/up sums differ from the lane order by f32 rounding
     # (about 1e-6 absolute here), so a few round to the neighbouring f16 before the activation, and a sum that
     # cancelled to almost nothing moves by many of its own tiny f16 steps.  Tolerance: the device value must lie
@@ -142,7 +146,7 @@ def _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf
     for gs in (-1.0, 0.0, 1.0):
         for us in (-1.0, 0.0, 1.0):
             g1, u1 = g0 + gs * dg, u0 + us * du
-            v = g1 / (1.0 + np.exp(-g1)) * u1
+            v = fn(g1, u1)
             lo, hi = np.minimum(lo, v), np.maximum(hi, v)
     a = _f16(act).astype(np.float64)
     pad = 1.5 * parity.f16_ulp(np.maximum(np.abs(lo), np.abs(hi)))
@@ -151,7 +155,7 @@ def _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf
     same = float(np.mean(act == full["act"]))
     assert same > 0.97, (what, "act identical fraction", same)
     # stage 2: c2 from the device's own act, against the oracle run on that same act
-    st2 = orc.moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, threads=threads, act_in=act)
+    st2 = orc.moe_ffn(x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, threads=threads, act_in=act, gelu=gelu)
     if c2 is not None:
         m2 = parity.assert_close(_f16(c2), _f16(st2["c2"]), what + " c2")
         # stage 3: the slot-order f32 sum of the device's c2 is exact arithmetic on f16 inputs -> bit for bit
@@ -183,6 +187,26 @@ def test_moe_ffn_small(dec, orc, small_experts, group, bf, t):
     idx, wt = ops.moe_topk(gen.router_logits(t, E, seed=t), k)
     y, act, c2, blk = _run_ffn(dec, name, x, idx, wt, t, k, h)
     _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, "small g%d bf%d t%d blk%d" % (group, bf, t, blk))
+
+
+@pytest.mark.parametrize("group,bf", [(32, False), (128, True)])
+@pytest.mark.parametrize("t", [1, 4, 9, 40, 200])
+def test_moe_ffn_gelu(dec, orc, small_experts, group, bf, t):
+    """The gelu flag of marlin_moe_ffn_dev: tanh-form gelu on the gate instead of silu, every regime of the FFN."""
+    say("moe_ffn gelu", group, bf, t)
+    name, q13, s13, q2, s2 = small_experts[(group, bf)]
+    E, h, n_ff, k = SMALL["E"], SMALL["h"], SMALL["n_ff"], SMALL["k"]
+    x = gen.normal_f16(3000 + t, (t, h))
+    idx, wt = ops.moe_topk(gen.router_logits(t, E, seed=50 + t), k)
+    y, act, c2, blk = _run_ffn(dec, name, x, idx, wt, t, k, h, gelu=True)
+    _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, "gelu g%d bf%d t%d blk%d" % (group, bf, t, blk),
+               gelu=True)
+    # and it is not silu
+    y_s, act_s, _, _ = _run_ffn(dec, name, x, idx, wt, t, k, h)
+    assert np.mean(act != act_s) > 0.5
+    from llm170_amd import ffi
+    with pytest.raises(ops.W4a16Error):  # an activation that does not exist
+        ffi.check(dec.cc.lib.w4a16_moe_ffn_act(dec.cc.h, name.encode(), 1, 1, 1, 1, k, 1, 7))
 
 
 @pytest.mark.parametrize("block,waves", [(1, 0), (1, 2), (4, 1), (4, 2), (16, 1), (16, 4), (32, 4), (48, 8), (64, 4)])

@@ -50,6 +50,32 @@ def test_oracle_act_layout(orc):
     assert np.array_equal(got, 30.0 * np.arange(ns * n_ff).reshape(ns, n_ff) / 8.0)
 
 
+def test_oracle_gelu_act(orc):
+    """f16(gelu_tanh(g) * u): float64 evaluation of the same formula within one f16 step; close to the erf form of
+    gelu; special cases; gate and up are not interchangeable."""
+    rng = np.random.default_rng(15)
+    g = (rng.standard_normal(4096) * 3).astype(np.float16)
+    u = (rng.standard_normal(4096) * 3).astype(np.float16)
+    c13 = np.concatenate([g.view(np.uint16), u.view(np.uint16)])[None, :]
+    got = _f16(orc.moe_act_gelu_f16(c13, 1, 4096)).ravel()
+    g64, u64 = g.astype(np.float64), u.astype(np.float64)
+    want = 0.5 * g64 * (1.0 + np.tanh(0.7978846 * (g64 + 0.044715 * g64 ** 3))) * u64
+    step = np.maximum(np.abs(want), 2.0 ** -14) * 2.0 ** -10
+    assert np.all(np.abs(got - want) <= 0.51 * step + 1e-6)
+    erf_form = 0.5 * g64 * (1.0 + np.array([math.erf(v / math.sqrt(2.0)) for v in g64])) * u64
+    assert np.max(np.abs(want - erf_form) / (np.abs(u64) + 1e-9)) < 2e-3  # the tanh form approximates gelu
+    swapped = 0.5 * u64 * (1.0 + np.tanh(0.7978846 * (u64 + 0.044715 * u64 ** 3))) * g64
+    assert np.mean(np.abs(got - swapped) > step) > 0.9
+    silu = g64 / (1.0 + np.exp(-g64)) * u64
+    assert np.mean(np.abs(got - silu) > step) > 0.9  # and it is not the silu kernel
+    h = lambda v: int(np.float16(v).view(np.uint16))
+    act = lambda gg, uu: float(_f16(orc.moe_act_gelu_f16(np.array([[h(gg), h(uu)]], np.uint16), 1, 1))[0, 0])
+    assert act(0.0, 3.0) == 0.0 and act(2.5, 0.0) == 0.0
+    assert act(10.0, 2.0) == 20.0                      # gelu(g) -> g
+    assert act(-10.0, 2.0) == pytest.approx(0.0, abs=1e-7)  # gelu(g) -> 0
+    assert act(1.0, 1.0) == float(np.float16(0.5 * (1.0 + math.tanh(0.7978846 * 1.044715))))
+
+
 # ---------------------------------------------------------------- top-k sum
 def test_oracle_topk_sum(orc):
     rng = np.random.default_rng(7)
