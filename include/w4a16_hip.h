@@ -149,6 +149,11 @@ int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t
  * the gate and n/2..n the up projection (n % 32 == 0).  t <= 16 (decode regime); y_f16_dev: f16 [t][n/2].  Same values
  * as w4a16_lin_forward (decode path, same launch shape) followed by w4a16_silu_mul_f16. */
 int w4a16_lin_forward_glu(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_f16_dev, size_t t);
+/* The same with the activation named: act = W4A16_ACT_SILU (above) or W4A16_ACT_GELU_TANH, the elementwise kernel the
+ * reference launches for gelu-gated models (ew_gelu, assets/ew.cu:34-57):
+ * y = f16(0.5 g (1 + tanh(0.7978846 (g + 0.044715 g^3))) * u).  Same values as w4a16_lin_forward followed by
+ * w4a16_act_mul_f16 with the same act. */
+int w4a16_lin_forward_glu_act(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_f16_dev, size_t t, int act);
 
 /* A decode-regime linear (t <= 16) with the RMS normalisation of its input deferred across it.  The reference runs
  * norm_resid as a launch of its own ahead of each linear (assets/norm.cu:4-48, kernels/mod.rs:11-54); a per-row
@@ -172,9 +177,11 @@ int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x
                                     uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_dev,
                                     int out_f16, uint64_t stats_out_dev, size_t stat_rows, size_t* n_stats_out,
                                     uint64_t resid_dev, uint64_t nw_dev);
-/* The same for the fused gate|up projection: the factor multiplies gate and up before silu(g) * u. */
+/* The same for the fused gate|up projection: the factor multiplies gate and up before the activation (act as in
+ * w4a16_lin_forward_glu_act). */
 int w4a16_lin_forward_glu_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
-                                        uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_f16_dev);
+                                        uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_f16_dev,
+                                        int act);
 
 /* gemv_host (w4a16_dec/mod.rs, host-operand convenience used by probes): lin_forward with host x / y. */
 int w4a16_lin_forward_host(w4a16_ctx* ctx, const char* name, const uint16_t* x_f16, void* y, size_t t, int out_f16,
@@ -310,6 +317,9 @@ int w4a16_norm_resid(w4a16_ctx* ctx, uint64_t x_dev, uint64_t nw_dev, uint64_t a
                      uint64_t xn16_dev, size_t t, size_t w_off, size_t hidden);
 /* ew (assets/ew.cu:9-32): out[r][c] = f16(silu(gu[r][c]) * gu[r][n_ff + c]) for gu f32 [t][2*n_ff], f32 arithmetic. */
 int w4a16_silu_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_ff, size_t t, uint64_t out_f16_dev);
+/* ew / ew_gelu (assets/ew.cu:9-32, 34-57) chosen by act (W4A16_ACT_SILU, W4A16_ACT_GELU_TANH); the gelu is the tanh
+ * form, out = f16(0.5 g (1 + tanh(0.7978846 (g + 0.044715 g^3))) * u) in f32 arithmetic. */
+int w4a16_act_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_ff, size_t t, uint64_t out_f16_dev, int act);
 
 /* chain_device_body (w4a16_dec/chains.rs:195-304) reduced to its linears: for layer l = layer0 .. layer0+n_layers-1,
  * with the linears registered as "<prefix>.<l>.attn_qkv", ".attn_output", ".ffn_gate_up", ".ffn_down":

@@ -71,12 +71,18 @@ extern "C" int w4a16_norm_resid(w4a16_ctx* ctx, uint64_t x_dev, uint64_t nw_dev,
 }
 
 extern "C" int w4a16_silu_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_ff, size_t t, uint64_t out_f16_dev) {
+    return w4a16_act_mul_f16(ctx, gu_f32_dev, n_ff, t, out_f16_dev, W4A16_ACT_SILU);
+}
+
+extern "C" int w4a16_act_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_ff, size_t t, uint64_t out_f16_dev, int act) {
     if (!ctx || !gu_f32_dev || !out_f16_dev) return w4_fail(W4A16_ERR_ARG, "silu_mul: null argument");
+    if (act != W4A16_ACT_SILU && act != W4A16_ACT_GELU_TANH)
+        return w4_fail(W4A16_ERR_ARG, "act_mul: activation %d (0 = silu, 1 = gelu, tanh form)", act);
     if (t == 0 || n_ff == 0 || n_ff > 0x3fffffffu || t > 0x7fffffffu)
         return w4_fail(W4A16_ERR_SHAPE, "silu_mul: t=%zu n_ff=%zu", t, n_ff);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     int nf = (int)n_ff, ti = (int)t;
-    void* p[] = {&gu_f32_dev, &nf, &ti, &out_f16_dev};
+    void* p[] = {&gu_f32_dev, &nf, &ti, &out_f16_dev, &act};
     return w4_launch(ctx, "w4a16_silu_mul_f16", std::min<unsigned>(ceil_div(t * n_ff / (n_ff % 4 == 0 ? 4 : 1), 256), 4096), 1, 256, 0, p);
 }
 
@@ -165,7 +171,7 @@ extern "C" int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, siz
                                                S.stats[0], hidden, &n_a, 0, 0));
         W4_TRY(w4a16_lin_forward_deferred_norm(ctx, nm[1], S.a16, n_qkv, t, S.stats[0], n_a, hidden, S.h16a, 1, S.stats[1],
                                                hidden, &n_b, 0, 0));
-        W4_TRY(w4a16_lin_forward_glu_deferred_norm(ctx, nm[2], S.h16a, 0, t, S.stats[1], n_b, hidden, S.h16b));
+        W4_TRY(w4a16_lin_forward_glu_deferred_norm(ctx, nm[2], S.h16a, 0, t, S.stats[1], n_b, hidden, S.h16b, W4A16_ACT_SILU));
         if (last) {
             // the chain's output is normalised: one launch per call, not per layer
             W4_TRY(w4a16_lin_forward(ctx, nm[3], S.h16b, S.y32, t, 0, W4A16_PATH_DECODE));

@@ -102,6 +102,7 @@ struct DecodeNorm {
     size_t n_stats_out = 0;  // set by the launch: entries written to stats_out
     uint64_t resid = 0;      // f32 [t][n] residual stream, takes the output: v = resid + y, written back
     uint64_t nw = 0;         // f32 [n] norm weight of the output rows, multiplies what y_dev receives
+    int act = 0;             // gated projection only: W4A16_ACT_*
 };
 
 static unsigned decode_stats_lds(const DecodeNorm& nm) {
@@ -145,9 +146,10 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     int ldx = (int)(nm.ldx ? nm.ldx : L.k), n_in = (int)nm.n_stats_in, stat_rows = (int)std::min<size_t>(nm.stat_rows, L.n);
     float inv_cols = nm.in_cols ? 1.0f / (float)nm.in_cols : 0.0f;
     uint64_t s_in = nm.stats_in, s_out = nm.stats_out, resid = nm.resid, nw = nm.nw;
+    int act_kind = 0;  // no activation in the plain linear
     nm.n_stats_out = s_out ? std::min(blocks, (size_t)ceil_div((size_t)stat_rows, (size_t)rb * 16)) : 0;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
-                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw};
+                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind};
     // LDS: the split-K partial tiles [waves][rb][1 KiB], then two scale slots per wave; a slot holds the scales of
     // one ring round (rb x depth x groups-per-tile x 32 bytes, ring never deeper than 8 tiles) rounded up to 512
     const unsigned slot = ((unsigned)(rb * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
@@ -184,8 +186,11 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
     int ldx = (int)(nm.ldx ? nm.ldx : L.k), n_in = (int)nm.n_stats_in, stat_rows = 0;
     float inv_cols = nm.in_cols ? 1.0f / (float)nm.in_cols : 0.0f;
     uint64_t s_in = nm.stats_in, s_out = 0, resid = 0, nw = 0;
+    if (nm.act != W4A16_ACT_SILU && nm.act != W4A16_ACT_GELU_TANH)
+        return w4_fail(W4A16_ERR_ARG, "decode glu: activation %d (0 = silu, 1 = gelu, tanh form)", nm.act);
+    int act_kind = nm.act;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
-                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw};
+                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind};
     const unsigned slot = ((unsigned)(2 * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
     const unsigned shmem = (unsigned)(waves * 2 * 1024) + (unsigned)waves * 2u * slot + decode_stats_lds(nm);
     return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);
@@ -494,11 +499,18 @@ extern "C" int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_de
 }
 
 extern "C" int w4a16_lin_forward_glu(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_f16_dev, size_t t) {
+    return w4a16_lin_forward_glu_act(ctx, name, x_dev, y_f16_dev, t, W4A16_ACT_SILU);
+}
+
+extern "C" int w4a16_lin_forward_glu_act(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_f16_dev, size_t t,
+                                         int act) {
     W4Lin* L = nullptr;
     W4_TRY(w4_find_lin(ctx, name, &L));
     if (!x_dev || !y_f16_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_glu %s: null operand or t=0", name);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
-    return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t);
+    DecodeNorm nm;
+    nm.act = act;
+    return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t, &nm);
 }
 
 extern "C" int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
@@ -526,7 +538,7 @@ extern "C" int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name,
 
 extern "C" int w4a16_lin_forward_glu_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
                                                    uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols,
-                                                   uint64_t y_f16_dev) {
+                                                   uint64_t y_f16_dev, int act) {
     W4Lin* L = nullptr;
     W4_TRY(w4_find_lin(ctx, name, &L));
     if (!x_dev || !y_f16_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_glu_deferred_norm %s: null operand or t=0", name);
@@ -536,6 +548,7 @@ extern "C" int w4a16_lin_forward_glu_deferred_norm(w4a16_ctx* ctx, const char* n
     nm.stats_in = stats_in_dev;
     nm.n_stats_in = n_stats_in;
     nm.in_cols = in_cols;
+    nm.act = act;
     return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t, &nm);
 }
 

@@ -57,7 +57,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                             int kt_per_slice, int kt_per_wave, int ldx,
                                             const float* __restrict__ stats_in, int n_stats_in, float inv_cols_in,
                                             float* __restrict__ stats_out, int stat_rows, float* __restrict__ resid,
-                                            const float* __restrict__ nw) {
+                                            const float* __restrict__ nw, int act_kind) {
     extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K, then [W][2][AUXB] scale slots
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
     constexpr int AUXB = RB * DEPTH * GPT * 32;      // bytes of scales one ring round needs: [rb][tile][group][16 rows]
@@ -355,7 +355,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const float gt = acc[0][i], up = acc[RB - 1][i];
-            float v = (gt / (1.0f + expf(-gt))) * up;
+            float v = w4_act_mul(gt, up, act_kind);
             asm volatile("" : "+v"(v));  // the product is rounded to f32 before the f16 conversion, as in the separate kernel
             o[i] = (_Float16)v;
         }
@@ -411,10 +411,10 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                                                         const float* stats_in, int n_stats_in,       \
                                                                         float inv_cols_in, float* stats_out,         \
                                                                         int stat_rows, float* resid,                 \
-                                                                        const float* nw) {                           \
+                                                                        const float* nw, int act_kind) {             \
         decode_body<G, SBF, RB, DECODE_DEPTH(BUDGET, G, RB, XL), XL>(                                                \
             qt, st, x, y, row_blocks, k, n, t, out_f16, ws, tickets, waves, nks, kt_per_slice, kt_per_wave, ldx,     \
-            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw);                                     \
+            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw, act_kind);                           \
     }
 #define DECODE_GLU_KERNEL_X(NAME, G, SBF, XL, BUDGET, ATTR)                                                           \
     extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
@@ -425,10 +425,10 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                                                         const float* stats_in, int n_stats_in,       \
                                                                         float inv_cols_in, float* stats_out,         \
                                                                         int stat_rows, float* resid,                 \
-                                                                        const float* nw) {                           \
+                                                                        const float* nw, int act_kind) {             \
         decode_body<G, SBF, 2, DECODE_DEPTH(BUDGET, G, 2, XL), XL, true>(                                            \
             qt, st, x, y, row_blocks, k, n, t, out_f16, ws, tickets, waves, nks, kt_per_slice, kt_per_wave, ldx,     \
-            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw);                                     \
+            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw, act_kind);                           \
     }
 #define DECODE_HI __attribute__((amdgpu_waves_per_eu(6, 6)))
 #define DECODE_MID __attribute__((amdgpu_waves_per_eu(5, 5)))

@@ -116,7 +116,7 @@ extern "C" __global__ __launch_bounds__(1024) void w4a16_norm_resid(float* __res
 // out[r][c] = f16((g / (1 + exp(-g))) * u),  g = gu[r][c], u = gu[r][n_ff + c], all in f32 (assets/ew.cu:19-30).
 // Four columns per thread when n_ff % 4 == 0.
 extern "C" __global__ __launch_bounds__(256) void w4a16_silu_mul_f16(const float* __restrict__ gu, int n_ff, int t,
-                                                                    uint16_t* __restrict__ out) {
+                                                                    uint16_t* __restrict__ out, int act_kind) {
     if ((n_ff & 3) == 0) {
         const size_t total = (size_t)t * n_ff / 4;
         for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
@@ -125,7 +125,7 @@ extern "C" __global__ __launch_bounds__(256) void w4a16_silu_mul_f16(const float
             const f4_t u = *reinterpret_cast<const f4_t*>(gu + r * 2 * n_ff + n_ff + c);
             h4_t o;
 #pragma unroll
-            for (int j = 0; j < 4; j++) o[j] = glue_round_f16((g[j] / (1.0f + expf(-g[j]))) * u[j]);
+            for (int j = 0; j < 4; j++) o[j] = glue_round_f16(w4_act_mul(g[j], u[j], act_kind));
             *reinterpret_cast<h4_t*>(reinterpret_cast<_Float16*>(out) + i * 4) = o;
         }
         return;
@@ -134,8 +134,7 @@ extern "C" __global__ __launch_bounds__(256) void w4a16_silu_mul_f16(const float
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t r = i / n_ff, c = i % n_ff;
         const float g = gu[r * 2 * n_ff + c], u = gu[r * 2 * n_ff + n_ff + c];
-        const float e = expf(-g);
-        reinterpret_cast<_Float16*>(out)[i] = glue_round_f16((g / (1.0f + e)) * u);
+        reinterpret_cast<_Float16*>(out)[i] = glue_round_f16(w4_act_mul(g, u, act_kind));
     }
 }
 

@@ -72,12 +72,7 @@ __device__ __forceinline__ void moe_store(f4_t a0, f4_t a1, int slot, int q, int
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const float g = moe_round_f16(a0[i]), up = moe_round_f16(a1[i]);
-            if (act_kind == 1) {  // uniform
-                const float x3 = g * g * g;
-                o[i] = (_Float16)((0.5f * g * (1.0f + tanhf(0.7978846f * (g + 0.044715f * x3)))) * up);
-            } else {
-                o[i] = (_Float16)((g / (1.0f + expf(-g))) * up);
-            }
+            o[i] = (_Float16)w4_act_mul(g, up, act_kind);
         }
         *reinterpret_cast<h4_t*>(reinterpret_cast<_Float16*>(y) + (size_t)slot * n_ff + u * 16 + 4 * q) = o;
     } else {

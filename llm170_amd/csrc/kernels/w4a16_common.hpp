@@ -107,3 +107,15 @@ __device__ __forceinline__ f4_t w4_fma4(f4_t a, f4_t b, f4_t c) {
     for (int i = 0; i < 4; i++) r[i] = __builtin_fmaf(a[i], b[i], c[i]);
     return r;
 }
+
+// act(gate) * up in f32, the element-wise step between a gated FFN's projections: kind 0 = silu (assets/ew.cu:9-32,
+// w4a16_moe_act_silu_f16), kind 1 = the tanh form of gelu (assets/ew.cu:34-57, w4a16_moe_act_gelu_f16,
+// assets/moe.cu:1635-1647), in the reference's order of operations.  One definition for every kernel that applies it,
+// so that fused epilogues give the bits of the separate kernel.  `kind` is uniform.
+__device__ __forceinline__ float w4_act_mul(float g, float u, int kind) {
+    if (kind == 1) {
+        const float x3 = g * g * g;
+        return (0.5f * g * (1.0f + tanhf(0.7978846f * (g + 0.044715f * x3)))) * u;
+    }
+    return (g / (1.0f + expf(-g))) * u;
+}

@@ -49,11 +49,12 @@ _SIGS = {
                                  C.POINTER(C.c_size_t), C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "w4a16_lin_forward": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_size_t, C.c_int, C.c_int]),
     "w4a16_lin_forward_glu": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_size_t]),
+    "w4a16_lin_forward_glu_act": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_size_t, C.c_int]),
     "w4a16_lin_forward_deferred_norm": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64,
                                                   C.c_size_t, C.c_size_t, C.c_uint64, C.c_int, C.c_uint64, C.c_size_t,
                                                   C.POINTER(C.c_size_t), C.c_uint64, C.c_uint64]),
     "w4a16_lin_forward_glu_deferred_norm": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_size_t, C.c_size_t,
-                                                      C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64]),
+                                                      C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64, C.c_int]),
     "w4a16_lin_forward_host": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int]),
     "w4a16_dequant_dump": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int, C.c_uint64]),
     "w4a16_lin_untile": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64]),
@@ -88,6 +89,7 @@ _SIGS = {
     "w4a16_norm_resid": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64,
                                    C.c_size_t, C.c_size_t, C.c_size_t]),
     "w4a16_silu_mul_f16": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64]),
+    "w4a16_act_mul_f16": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64, C.c_int]),
     "w4a16_chain_forward": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64]),
     "w4a16_chain_forward_fused": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64]),
     "w4a16_bench_chain": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t,

@@ -190,9 +190,13 @@ class W4a16Dec:
     def lin_forward(self, name, x_dev, dst_dev, t, out_f16=False, path=PATH_AUTO):
         ffi.check(self.cc.lib.w4a16_lin_forward(self.cc.h, name.encode(), x_dev, dst_dev, t, int(out_f16), path))
 
-    def lin_forward_glu(self, name, x_dev, y_f16_dev, t):
-        """Fused gate|up projection with the SiLU*up epilogue: y f16 [t][n/2]."""
-        ffi.check(self.cc.lib.w4a16_lin_forward_glu(self.cc.h, name.encode(), x_dev, y_f16_dev, t))
+    def lin_forward_glu(self, name, x_dev, y_f16_dev, t, gelu=False):
+        """Fused gate|up projection with the act(gate)*up epilogue (silu, or the tanh form of gelu): y f16 [t][n/2]."""
+        if gelu:
+            ffi.check(self.cc.lib.w4a16_lin_forward_glu_act(self.cc.h, name.encode(), x_dev, y_f16_dev, t,
+                                                            ffi.ACT_GELU_TANH))
+        else:
+            ffi.check(self.cc.lib.w4a16_lin_forward_glu(self.cc.h, name.encode(), x_dev, y_f16_dev, t))
 
     def lin_forward_deferred_norm(self, name, x_dev, t, y_dev, out_f16=False, ldx=0, stats_in=0, n_stats_in=0, in_cols=0,
                                   stats_out=0, stat_rows=0, resid=0, nw=0):
@@ -204,9 +208,11 @@ class W4a16Dec:
                                                               C.byref(n_out), resid, nw))
         return n_out.value
 
-    def lin_forward_glu_deferred_norm(self, name, x_dev, t, y_f16_dev, ldx=0, stats_in=0, n_stats_in=0, in_cols=0):
+    def lin_forward_glu_deferred_norm(self, name, x_dev, t, y_f16_dev, ldx=0, stats_in=0, n_stats_in=0, in_cols=0,
+                                      gelu=False):
         ffi.check(self.cc.lib.w4a16_lin_forward_glu_deferred_norm(self.cc.h, name.encode(), x_dev, ldx, t, stats_in,
-                                                                  n_stats_in, in_cols, y_f16_dev))
+                                                                  n_stats_in, in_cols, y_f16_dev,
+                                                                  ffi.ACT_GELU_TANH if gelu else ffi.ACT_SILU))
 
     def gemv_host(self, name, x, t=1, out_f16=False, path=PATH_AUTO):
         """Host operands in, host result out: y [t][n] (f32, or f16 bit patterns when out_f16)."""
@@ -354,6 +360,10 @@ class W4a16Dec:
 
     def silu_mul_f16(self, gu_dev, n_ff, t, out_dev):
         ffi.check(self.cc.lib.w4a16_silu_mul_f16(self.cc.h, gu_dev, n_ff, t, out_dev))
+
+    def act_mul_f16(self, gu_dev, n_ff, t, out_dev, gelu=False):
+        ffi.check(self.cc.lib.w4a16_act_mul_f16(self.cc.h, gu_dev, n_ff, t, out_dev,
+                                                ffi.ACT_GELU_TANH if gelu else ffi.ACT_SILU))
 
     def chain_forward(self, prefix, layer0, n_layers, x_dev, t, y_dev):
         """chain_device_body (w4a16_dec/chains.rs:195-304) reduced to its linears and glue."""

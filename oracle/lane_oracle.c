@@ -30,6 +30,7 @@
  *   orc_rms_rescale_f16 ... float64 v / sqrt(mean(v^2) + 1e-6) within one f16 step, >= 99.9 % identical; constant rows;
  *                           invariance of the output under scaling the row by a power of two
  *   orc_silu_mul_f16_rows . float64 evaluation within one f16 step; layout (gate | up) by a crafted row
+ *   orc_gelu_mul_f16_rows . float64 evaluation of the tanh form within one f16 step; swapped operands fail
  *   orc_norm_resid ........ numpy float32 restatement whose fused multiply-add is built from exact f64 products and a
  *                           round-to-odd sum (independent of libm's fmaf); float64 v/sqrt(mean v^2 + 1e-6)*w to a few f32
  *                           ulp; x + ab exact; an un-fused sum of squares and a sequential (non-tree) sum are shown to
@@ -488,4 +489,11 @@ void orc_silu_mul_f16_rows(const float* gu, size_t n_ff, size_t t, uint16_t* out
     for (size_t r = 0; r < t; r++)
         for (size_t c = 0; c < n_ff; c++)
             out[r * n_ff + c] = orc_silu_mul_f16(gu[r * 2 * n_ff + c], gu[r * 2 * n_ff + n_ff + c]);
+}
+
+/* ---- ew_gelu (assets/ew.cu:34-57) on the same rows: the tanh form of gelu on the gate, times up. ---- */
+void orc_gelu_mul_f16_rows(const float* gu, size_t n_ff, size_t t, uint16_t* out) {
+    for (size_t r = 0; r < t; r++)
+        for (size_t c = 0; c < n_ff; c++)
+            out[r * n_ff + c] = orc_gelu_mul_f16(gu[r * 2 * n_ff + c], gu[r * 2 * n_ff + n_ff + c]);
 }

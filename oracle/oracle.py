@@ -56,6 +56,7 @@ def lib():
         L.orc_f32_to_f16_array.argtypes, L.orc_f32_to_f16_array.restype = [f32p, sz, u16p], None
         L.orc_rms_rescale_f16.argtypes, L.orc_rms_rescale_f16.restype = [f32p, sz, sz, sz, u16p], None
         L.orc_silu_mul_f16_rows.argtypes, L.orc_silu_mul_f16_rows.restype = [f32p, sz, sz, u16p], None
+        L.orc_gelu_mul_f16_rows.argtypes, L.orc_gelu_mul_f16_rows.restype = [f32p, sz, sz, u16p], None
         L.orc_norm_resid.argtypes, L.orc_norm_resid.restype = [f32p, f32p, f32p, f32p, f32p, u16p, sz, sz, sz], None
         i32p = C.POINTER(C.c_int32)
         L.orc_moe_act_silu_f16.argtypes, L.orc_moe_act_silu_f16.restype = [u16p, sz, sz, u16p], None
@@ -302,6 +303,15 @@ def silu_mul_f16_rows(gu):
     t, two = gu.shape
     out = np.empty((t, two // 2), np.uint16)
     lib().orc_silu_mul_f16_rows(_p(gu, C.c_float), two // 2, t, _p(out, C.c_uint16))
+    return out
+
+
+def gelu_mul_f16_rows(gu):
+    """ew_gelu (assets/ew.cu:34-57): f32 [t][2*n_ff] = (gate | up) -> f16 bits [t][n_ff]."""
+    gu = _c(gu, np.float32)
+    t, two = gu.shape
+    out = np.empty((t, two // 2), np.uint16)
+    lib().orc_gelu_mul_f16_rows(_p(gu, C.c_float), two // 2, t, _p(out, C.c_uint16))
     return out
 
 

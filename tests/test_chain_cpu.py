@@ -57,6 +57,26 @@ def test_silu_mul_rows_against_float64(orc):
     assert np.mean(np.abs(got - swapped) > _step(want)) > 0.9
 
 
+def test_gelu_mul_rows_against_float64(orc):
+    rng = np.random.default_rng(16)
+    gu = (rng.standard_normal((3, 2 * 512)) * 3).astype(np.float32)
+    got = _f16(orc.gelu_mul_f16_rows(gu))
+    g, u = gu[:, :512].astype(np.float64), gu[:, 512:].astype(np.float64)
+
+    def gelu(v):
+        return 0.5 * v * (1.0 + np.tanh(0.7978846 * (v + 0.044715 * v ** 3)))
+
+    want = gelu(g) * u
+    # 1 + tanhf cancels in f32 for a gate below about -4 (the reference's arithmetic too): an absolute 1e-6 covers it
+    assert np.all(np.abs(got - want) <= 0.51 * _step(want) + 1e-6)
+    swapped = gelu(u) * g
+    assert np.mean(np.abs(got - swapped) > _step(want)) > 0.8
+    # against the erf form of gelu the tanh form stays within 1e-3 absolute per unit of up
+    from math import erf
+    exact = np.vectorize(lambda v: 0.5 * v * (1.0 + erf(v / np.sqrt(2.0))))(g) * u
+    assert np.max(np.abs(want - exact) / (np.abs(u) + 1e-9)) < 1e-3
+
+
 def test_chain_layer_against_float64(orc):
     hidden, n_qkv, n_ff, g, t = 256, 384, 512, 128, 3
     shapes = [(n_qkv, hidden), (hidden, hidden), (2 * n_ff, hidden), (hidden, n_ff)]

@@ -3,7 +3,7 @@ the C ABI against the CPU oracle."""
 import numpy as np
 import pytest
 
-from llm170_amd import gen, ops
+from llm170_amd import ffi, gen, ops
 from tests import parity
 
 pytestmark = pytest.mark.gpu
@@ -104,6 +104,40 @@ def test_fused_glu_equals_linear_then_silu_mul(dec, orc, n, k, group, bf16, t):
         rms = float(np.sqrt(np.mean(b * b)))
         assert np.all(np.abs(a - b) <= 2 * parity.f16_ulp(np.maximum(np.abs(b), rms / 128)))
         assert np.mean(one == want) > 0.97
+
+
+@pytest.mark.parametrize("n,k,group,t", [(1024, 256, 128, 1), (2048, 512, 32, 5), (1024, 256, 128, 16),
+                                         (34816, 5120, 128, 4)])
+def test_fused_glu_gelu(dec, orc, n, k, group, t):
+    """The gelu choice (ew_gelu beside ew): elementwise launch against the oracle, fused kernel bit-identical to linear +
+    elementwise launch, and different from the silu result."""
+    q, s, x = gen.make_linear(n, k, group, t, seed=72)
+    dec.upload_lin_g("glu", q, s, n, k, group, False)
+    cc = dec.cc
+    px, pg, pa, pb = cc.to_device(x), cc.alloc(t * n * 4), cc.alloc(t * (n // 2) * 2), cc.alloc(t * (n // 2) * 2)
+    dec.set_decode_shape(32, 4 if t > 8 or n >= 16384 else 8)
+    try:
+        dec.lin_forward("glu", px, pg, t, path=ops.PATH_DECODE)
+    finally:
+        dec.set_decode_shape(0, 0)
+    dec.act_mul_f16(pg, n // 2, t, pa, gelu=True)
+    dec.lin_forward_glu("glu", px, pb, t, gelu=True)
+    gu = cc.d2h(pg, (t, n), np.float32)
+    two, one = cc.d2h(pa, (t, n // 2), np.uint16), cc.d2h(pb, (t, n // 2), np.uint16)
+    dec.lin_forward_glu("glu", px, pb, t)
+    silu = cc.d2h(pb, (t, n // 2), np.uint16)
+    for p in (px, pg, pa, pb):
+        cc.free(p)
+    assert np.array_equal(one, two)
+    assert np.mean(one != silu) > 0.5
+    want = orc.gelu_mul_f16_rows(gu)  # the device's own f32 GEMM result through the oracle's elementwise step
+    a, b = _f16(two).astype(np.float64), _f16(want).astype(np.float64)
+    assert np.all(np.abs(a - b) <= parity.f16_ulp(b))  # tanhf from two libraries: last f32 bit ahead of the rounding
+    assert np.mean(two == want) > 0.99
+    with pytest.raises(ops.W4a16Error):  # an activation that does not exist
+        ffi.check(dec.cc.lib.w4a16_act_mul_f16(dec.cc.h, 1, 8, 1, 1, 7))
+    with pytest.raises(ops.W4a16Error):
+        ffi.check(dec.cc.lib.w4a16_lin_forward_glu_act(dec.cc.h, b"glu", 1, 1, 1, 7))
 
 
 def test_fused_glu_errors(dec):
