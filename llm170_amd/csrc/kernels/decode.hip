@@ -390,9 +390,10 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
 }
 
 // Two register regimes, chosen per instantiation.  Measured on MI355X: what the streaming rate needs is many resident
-// waves with a short ring each, not a deep ring in few waves — with <= 80 VGPRs six waves per SIMD are resident, the
-// whole grid of the 27B layer shapes is on the chip at once, every wave gets its share of HBM and all finish together
-// (a deep-ring build at three waves per SIMD ran the grid in two uneven generations: 4.6 -> 5.0 TB/s at M = 1).
+// waves with a short ring each, not a deep ring in few waves — with <= 80 VGPRs six waves per SIMD are resident (6144
+// on the chip: the whole grid of the 27B layer shapes at two row blocks per wave, 70 % of the gate+up grid at one),
+// every wave gets its share of HBM and the generations are even (a deep-ring build at three waves per SIMD ran the
+// grid in two uneven generations: 4.6 -> 5.0 TB/s at M = 1).
 //   HI: ring sized for 24 VGPRs of load buffers, amdgpu_waves_per_eu(6,6)   — variants that fit 80 VGPRs unspilled
 //   MID: the same ring at five waves per SIMD (<= 102 VGPRs)
 //   LO: occupancy left to the compiler — the wide variants (4 row blocks, 4 x loads) and group size 32; their ring
