@@ -340,10 +340,12 @@ def test_prefill_block_tiles_agree(dec, orc, n, k, group, t):
         dec.set_prefill_tile(96)
 
 
-@pytest.mark.parametrize("n,k,t", [(34816, 5120, 512), (5120, 17408, 512), (34816, 5120, 4096)])
+@pytest.mark.parametrize("n,k,t", [(34816, 5120, 512), (5120, 17408, 512), (34816, 5120, 4096), (34816, 5120, 1024),
+                                   (5120, 17408, 4096), (34816, 5120, 1000)])
 def test_prefill_full_shapes_against_device_twin_and_sampled_oracle(dec, orc, n, k, t):
     """Layer shapes: every output against the bit-exact device twin (itself pinned to the CPU oracle above and on a
-    seeded sample here), because the CPU needs ~1e12 scalar MACs for the full matrix."""
+    seeded sample here), because the CPU needs ~1e12 scalar MACs for the full matrix.  The shapes cover both block
+    tiles, ragged last tiles (t = 1000) and the automatic k slices of the narrow output."""
     say("prefill full", n, k, t)
     group = 128
     q, s, x = gen.make_linear(n, k, group, t, seed=5)
@@ -356,6 +358,16 @@ def test_prefill_full_shapes_against_device_twin_and_sampled_oracle(dec, orc, n,
     assert np.array_equal(_bits(twin[toks, rows]), _bits(smp))
     m = parity.assert_close(got, twin, "prefill full n%d k%d t%d" % (n, k, t))
     say("   ", {a: m[a] for a in ("rel_l2", "max_ulp", "max_ulp_strict", "strict_pass_frac", "clamped")})
+    # the same launch again (same bits) and with the k slices switched off
+    again = _device_forward(dec, "pfull", x, t, ops.PATH_PREFILL)
+    assert np.array_equal(_bits(again), _bits(got))
+    dec.set_prefill_ksplit(-1)
+    try:
+        whole = _device_forward(dec, "pfull", x, t, ops.PATH_PREFILL)
+    finally:
+        dec.set_prefill_ksplit(0)
+    parity.assert_close(whole, twin, "prefill full unsplit n%d k%d t%d" % (n, k, t))
+    parity.assert_close(got, whole, "prefill full split vs unsplit n%d k%d t%d" % (n, k, t))
 
 
 @pytest.mark.parametrize("n,k,group,t,ksplit", [(512, 4096, 128, 100, 2), (512, 4096, 128, 100, 3), (512, 4096, 128, 100, 8),
