@@ -203,6 +203,8 @@ def main():
         sys.exit(2)
 
     from llm170_amd import gen, ops
+    from llm170_amd import build as pkg_build
+    pkg_build.ensure_built()
     dec = ops.W4a16Dec()
     cc = dec.cc
 

@@ -67,6 +67,16 @@ def build_all(verbose=True):
     return outs, lib
 
 
+def ensure_built(verbose=False):
+    """Build only when nothing is built yet (a fresh checkout): tests, the smoke run and the benchmark load what is
+    there.  The library itself never builds or falls back: loading it without these files raises."""
+    missing = not os.path.exists(LIB_PATH) or any(
+        not os.path.exists(os.path.join(ASSET_DIR, n + ".hsaco")) for n in kernel_sources())
+    if missing:
+        build_all(verbose=verbose)
+    return missing
+
+
 if __name__ == "__main__":
     build_all()
     sys.exit(0)

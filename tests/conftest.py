@@ -12,6 +12,13 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+def pytest_sessionstart(session):
+    """A fresh checkout has no code objects and no host library: build them once (hipcc cross-compiles without a
+    GPU).  What is already built is loaded as it is."""
+    from llm170_amd import build
+    build.ensure_built()
+
+
 @pytest.fixture(scope="session")
 def orc():
     from oracle import oracle
