@@ -235,7 +235,7 @@ def main():
 
     # parity of what was just timed, against the CPU oracle (checker only)
     from oracle import oracle
-    from tests import parity
+    from llm170_amd import parity
     cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
     y16 = dec.gemv_host(names[0], x[:1], t=1, out_f16=True, path=ops.PATH_DECODE)
     t0 = time.perf_counter()

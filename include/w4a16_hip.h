@@ -30,6 +30,7 @@ extern "C" {
 
 typedef struct w4a16_ctx w4a16_ctx;
 typedef struct w4a16_event w4a16_event;
+typedef struct w4a16_graph w4a16_graph;
 
 enum {
     W4A16_OK = 0,
@@ -86,6 +87,21 @@ int w4a16_event_create(w4a16_ctx* ctx, w4a16_event** out);
 int w4a16_event_record(w4a16_ctx* ctx, w4a16_event* ev);
 int w4a16_event_elapsed_ms(w4a16_ctx* ctx, w4a16_event* start, w4a16_event* stop, float* ms); /* waits for stop */
 void w4a16_event_destroy(w4a16_ctx* ctx, w4a16_event* ev);
+
+/* Capture of the launch stream into a graph and its replay (CudaCtx::capture_begin / capture_end / graph_instantiate /
+ * graph_upload / graph_launch / graph_destroy, ctx/graph.rs:4-85).  Between w4a16_capture_begin and w4a16_capture_end every
+ * launching entry point of this library (w4a16_launch, w4a16_lin_forward*, w4a16_moe_ffn*, w4a16_chain_forward*,
+ * w4a16_memset0, w4a16_d2d, ...) records a node instead of running.  Nothing may allocate, free, wait or copy to or from
+ * the host in between: w4a16_alloc, w4a16_free, w4a16_sync, w4a16_h2d, w4a16_d2h and any call whose scratch buffer would
+ * have to grow return W4A16_ERR_ARG (and invalidate nothing) — run the sequence once before capturing it, as the
+ * reference does (warm_for_capture, w4a16_dec/graphs.rs:55).  w4a16_capture_end ends the capture, instantiates and
+ * uploads the graph.  A graph replays the recorded launches with the recorded arguments: same buffers, same shapes.
+ * Replays are ordered on the launch stream like any other launch.  w4a16_graph_destroy waits for the launch stream. */
+int w4a16_capture_begin(w4a16_ctx* ctx);
+int w4a16_capture_end(w4a16_ctx* ctx, w4a16_graph** out);
+int w4a16_graph_launch(w4a16_ctx* ctx, w4a16_graph* graph);
+size_t w4a16_graph_nodes(const w4a16_graph* graph); /* kernel and copy nodes recorded */
+void w4a16_graph_destroy(w4a16_ctx* ctx, w4a16_graph* graph);
 
 /* Names in the built-in asset manifest (assets.rs:276-334): returns the number of assets; when `asset` is in range
  * stores its name and NULL-terminated symbol list. */
@@ -341,6 +357,14 @@ int w4a16_chain_forward(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_
  * linears instead of before the roundings to f16 (results agree to those roundings). */
 int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers, uint64_t x_dev,
                               size_t t, uint64_t y_dev);
+/* ensure_graph (w4a16_dec/graphs.rs:41-134): one decode step of the chain as a replayable graph.  Runs the chain once
+ * eagerly (which sizes every scratch buffer and leaves its result in y_dev), then captures the same call —
+ * w4a16_chain_forward, or w4a16_chain_forward_fused when fused != 0 — and returns the instantiated graph.  Each
+ * w4a16_graph_launch recomputes y_dev from whatever x_dev holds at that moment; the reference keeps one such graph
+ * per slot and replays it every token. */
+int w4a16_chain_graph_create(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers, uint64_t x_dev, size_t t,
+                             uint64_t y_dev, int fused, w4a16_graph** out);
+
 /* Timed chain passes (decode_bench, w4a16_dec/probe.rs:1123-1289): `warmup` untimed then `reps` timed passes over
  * layers 0..n_layers-1.  use_graph != 0 captures one pass into a HIP graph and times graph launches
  * (forward_graph, w4a16_dec/graphs.rs); fused != 0 times w4a16_chain_forward_fused. */

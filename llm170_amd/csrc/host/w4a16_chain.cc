@@ -185,34 +185,46 @@ extern "C" int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, siz
     return 0;
 }
 
+extern "C" int w4a16_chain_graph_create(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers, uint64_t x_dev,
+                                        size_t t, uint64_t y_dev, int fused, w4a16_graph** out) {
+    if (!ctx || !prefix || !out) return w4_fail(W4A16_ERR_ARG, "chain_graph_create: null argument");
+    *out = nullptr;
+    auto pass = [&]() {
+        return fused ? w4a16_chain_forward_fused(ctx, prefix, layer0, n_layers, x_dev, t, y_dev)
+                     : w4a16_chain_forward(ctx, prefix, layer0, n_layers, x_dev, t, y_dev);
+    };
+    W4_TRY(pass());  // sizes the scratch (a capture cannot allocate) and checks the arguments
+    W4_TRY(w4a16_capture_begin(ctx));
+    const int frc = pass();
+    const std::string keep = w4_err_save();
+    w4a16_graph* g = nullptr;
+    const int erc = w4a16_capture_end(ctx, &g);
+    if (frc) {  // the failing step's message, not the one of ending the capture
+        if (g) w4a16_graph_destroy(ctx, g);
+        w4_err_restore(keep);
+        return frc;
+    }
+    W4_TRY(erc);
+    *out = g;
+    return 0;
+}
+
 extern "C" int w4a16_bench_chain(w4a16_ctx* ctx, const char* prefix, size_t n_layers, uint64_t x_dev, size_t t,
                                  uint64_t y_dev, size_t warmup, size_t reps, int use_graph, int fused, float* ms_events,
                                  double* ms_wall) {
     if (!ctx || !prefix || reps == 0) return w4_fail(W4A16_ERR_ARG, "bench_chain: null argument");
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
-    // one untimed pass always runs first: it sizes the scratch, which must not happen while capturing
     auto pass = [&]() {
         return fused ? w4a16_chain_forward_fused(ctx, prefix, 0, n_layers, x_dev, t, y_dev)
                      : w4a16_chain_forward(ctx, prefix, 0, n_layers, x_dev, t, y_dev);
     };
     for (size_t i = 0; i < std::max<size_t>(warmup, 1); i++) W4_TRY(pass());
     W4_TRY(w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"));
-    hipGraph_t graph = nullptr;
-    hipGraphExec_t exec = nullptr;
+    w4a16_graph* graph = nullptr;
     int rc = 0;
     if (use_graph) {
-        rc = w4_hip(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
-        if (!rc) {
-            int frc = pass();
-            const std::string keep = w4_err_save();
-            rc = w4_hip(hipStreamEndCapture(ctx->stream, &graph), "hipStreamEndCapture");
-            if (frc) {
-                w4_err_restore(keep);
-                rc = frc;
-            }
-        }
-        if (!rc) rc = w4_hip(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
-        if (!rc) rc = w4_hip(hipGraphLaunch(exec, ctx->stream), "hipGraphLaunch");  // one untimed replay
+        rc = w4a16_chain_graph_create(ctx, prefix, 0, n_layers, x_dev, t, y_dev, fused, &graph);
+        if (!rc) rc = w4a16_graph_launch(ctx, graph);  // one untimed replay
         if (!rc) rc = w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
     }
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -220,8 +232,7 @@ extern "C" int w4a16_bench_chain(w4a16_ctx* ctx, const char* prefix, size_t n_la
     if (!rc) rc = w4_hip(hipEventCreate(&e1), "hipEventCreate");
     auto w0 = std::chrono::steady_clock::now();
     if (!rc) rc = w4_hip(hipEventRecord(e0, ctx->stream), "hipEventRecord");
-    for (size_t i = 0; i < reps && !rc; i++)
-        rc = use_graph ? w4_hip(hipGraphLaunch(exec, ctx->stream), "hipGraphLaunch") : pass();
+    for (size_t i = 0; i < reps && !rc; i++) rc = use_graph ? w4a16_graph_launch(ctx, graph) : pass();
     if (!rc) rc = w4_hip(hipEventRecord(e1, ctx->stream), "hipEventRecord");
     if (!rc) rc = w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
     auto w1 = std::chrono::steady_clock::now();
@@ -232,8 +243,7 @@ extern "C" int w4a16_bench_chain(w4a16_ctx* ctx, const char* prefix, size_t n_la
     const std::string keep = w4_err_save();
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
-    if (exec) (void)hipGraphExecDestroy(exec);
-    if (graph) (void)hipGraphDestroy(graph);
+    if (graph) w4a16_graph_destroy(ctx, graph);
     if (rc) w4_err_restore(keep);
     return rc;
 }

@@ -214,6 +214,12 @@ extern "C" int w4a16_ctx_create(int device_ordinal, const char* asset_dir, w4a16
 extern "C" void w4a16_ctx_destroy(w4a16_ctx* ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
+    if (ctx->capturing) {  // a capture left open: end it and drop what it recorded
+        hipGraph_t dangling = nullptr;
+        (void)hipStreamEndCapture(ctx->stream, &dangling);
+        if (dangling) (void)hipGraphDestroy(dangling);
+        ctx->capturing = false;
+    }
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->stream2) (void)hipStreamSynchronize(ctx->stream2);
     for (auto& a : ctx->allocs) (void)hipFree((void*)a.first);
@@ -264,6 +270,8 @@ extern "C" int w4a16_alloc(w4a16_ctx* ctx, size_t bytes, uint64_t* dptr) {
     if (!ctx || !dptr) return w4_fail(W4A16_ERR_ARG, "alloc: null argument");
     *dptr = 0;
     if (bytes == 0) return w4_fail(W4A16_ERR_ARG, "alloc: zero bytes");
+    if (ctx->capturing)
+        return w4_fail(W4A16_ERR_ARG, "alloc(%zu) while the launch stream is capturing: run the sequence once before the capture so that every scratch buffer has its size", bytes);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     void* p = nullptr;
     hipError_t e = hipMalloc(&p, bytes);
@@ -280,6 +288,7 @@ extern "C" int w4a16_free(w4a16_ctx* ctx, uint64_t dptr) {
     auto it = ctx->allocs.find(dptr);
     if (it == ctx->allocs.end()) return w4_fail(W4A16_ERR_ARG, "free: %#llx was not allocated by this context",
                                                 (unsigned long long)dptr);
+    if (ctx->capturing) return w4_fail(W4A16_ERR_ARG, "free while the launch stream is capturing");
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     // work queued on the launch stream may still use the buffer
     W4_TRY(w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"));
@@ -293,6 +302,7 @@ extern "C" size_t w4a16_allocated_bytes(w4a16_ctx* ctx) { return ctx ? ctx->allo
 extern "C" int w4a16_h2d(w4a16_ctx* ctx, uint64_t dst, const void* src, size_t bytes) {
     if (!ctx || !dst || !src) return w4_fail(W4A16_ERR_ARG, "h2d: null argument");
     if (bytes == 0) return 0;
+    if (ctx->capturing) return w4_fail(W4A16_ERR_ARG, "h2d while the launch stream is capturing");
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     W4_TRY(w4_hip(hipMemcpyAsync((void*)dst, src, bytes, hipMemcpyHostToDevice, ctx->stream), "hipMemcpyAsync(h2d)"));
     return w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
@@ -301,6 +311,7 @@ extern "C" int w4a16_h2d(w4a16_ctx* ctx, uint64_t dst, const void* src, size_t b
 extern "C" int w4a16_d2h(w4a16_ctx* ctx, void* dst, uint64_t src, size_t bytes) {
     if (!ctx || !dst || !src) return w4_fail(W4A16_ERR_ARG, "d2h: null argument");
     if (bytes == 0) return 0;
+    if (ctx->capturing) return w4_fail(W4A16_ERR_ARG, "d2h while the launch stream is capturing");
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     W4_TRY(w4_hip(hipMemcpyAsync(dst, (const void*)src, bytes, hipMemcpyDeviceToHost, ctx->stream), "hipMemcpyAsync(d2h)"));
     return w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
@@ -328,8 +339,66 @@ extern "C" int w4a16_memset0(w4a16_ctx* ctx, uint64_t dst, size_t bytes) {
 
 extern "C" int w4a16_sync(w4a16_ctx* ctx) {
     if (!ctx) return w4_fail(W4A16_ERR_ARG, "sync: null context");
+    if (ctx->capturing) return w4_fail(W4A16_ERR_ARG, "sync while the launch stream is capturing");
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     return w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+// ------------------------------------------------------------------------------------------------ graphs
+// Capture of the launch stream into a HIP graph (reference: CudaCtx::capture_begin / capture_end / graph_instantiate /
+// graph_upload / graph_launch / graph_destroy, ctx/graph.rs:4-85).  Between begin and end every launch entry point of
+// this library records a kernel node instead of running; nothing may allocate, free, copy to or from the host or wait
+// (the entry points that would refuse).  Clearing memory inside a capture goes through the fill kernel of
+// w4a16_memset0, never a memset node.
+extern "C" int w4a16_capture_begin(w4a16_ctx* ctx) {
+    if (!ctx) return w4_fail(W4A16_ERR_ARG, "capture_begin: null context");
+    if (ctx->capturing) return w4_fail(W4A16_ERR_ARG, "capture_begin: the launch stream is capturing already");
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    W4_TRY(w4_hip(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"));
+    W4_TRY(w4_hip(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture"));
+    ctx->capturing = true;
+    return 0;
+}
+
+extern "C" int w4a16_capture_end(w4a16_ctx* ctx, w4a16_graph** out) {
+    if (!ctx || !out) return w4_fail(W4A16_ERR_ARG, "capture_end: null argument");
+    *out = nullptr;
+    if (!ctx->capturing) return w4_fail(W4A16_ERR_ARG, "capture_end: the launch stream is not capturing");
+    ctx->capturing = false;
+    w4a16_graph* g = new w4a16_graph();
+    int rc = w4_hip(hipStreamEndCapture(ctx->stream, &g->graph), "hipStreamEndCapture");
+    if (!rc && !g->graph) rc = w4_fail(W4A16_ERR_ARG, "capture_end: the capture was invalidated");
+    if (!rc) rc = w4_hip(hipGraphGetNodes(g->graph, nullptr, &g->nodes), "hipGraphGetNodes");
+    if (!rc && g->nodes == 0) rc = w4_fail(W4A16_ERR_ARG, "capture_end: nothing was launched between begin and end");
+    if (!rc) rc = w4_hip(hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0), "hipGraphInstantiate");
+    if (!rc) rc = w4_hip(hipGraphUpload(g->exec, ctx->stream), "hipGraphUpload");
+    if (rc) {
+        const std::string keep = w4_err_save();
+        w4a16_graph_destroy(ctx, g);
+        w4_err_restore(keep);
+        return rc;
+    }
+    *out = g;
+    return 0;
+}
+
+extern "C" int w4a16_graph_launch(w4a16_ctx* ctx, w4a16_graph* g) {
+    if (!ctx || !g || !g->exec) return w4_fail(W4A16_ERR_ARG, "graph_launch: null argument");
+    if (ctx->capturing) return w4_fail(W4A16_ERR_ARG, "graph_launch while the launch stream is capturing");
+    return w4_hip(hipGraphLaunch(g->exec, ctx->stream), "hipGraphLaunch");
+}
+
+extern "C" size_t w4a16_graph_nodes(const w4a16_graph* g) { return g ? g->nodes : 0; }
+
+extern "C" void w4a16_graph_destroy(w4a16_ctx* ctx, w4a16_graph* g) {
+    if (!g) return;
+    if (ctx) {
+        (void)hipSetDevice(ctx->device);
+        if (ctx->stream && !ctx->capturing) (void)hipStreamSynchronize(ctx->stream);  // a replay may still be running
+    }
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    delete g;
 }
 
 // ------------------------------------------------------------------------------------------------ events

@@ -57,6 +57,14 @@ struct w4a16_event {
     hipEvent_t ev;
 };
 
+// A captured and instantiated sequence of launches (reference: GraphEntry {exec, handle}, w4a16_dec/mod.rs; the pair
+// ctx/graph.rs hands to graph_destroy).
+struct w4a16_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    size_t nodes = 0;
+};
+
 struct w4a16_ctx {
     int device = 0;
     hipStream_t stream = nullptr;   // launch stream (reference: CudaCtx.stream)
@@ -80,6 +88,7 @@ struct w4a16_ctx {
     uint64_t prefill_ws = 0;                                    // f32 partials of a split-K prefill launch
     size_t prefill_ws_cap = 0;
     int cu_count = 0;
+    bool capturing = false;  // between w4a16_capture_begin and w4a16_capture_end: nothing may allocate, free or wait
 };
 
 // Launch constants that mirror #defines of the kernel sources (a CPU test reads both texts and compares the values):

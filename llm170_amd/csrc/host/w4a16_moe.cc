@@ -188,6 +188,8 @@ extern "C" int w4a16_moe_align(w4a16_ctx* ctx, uint64_t idx_dev, size_t ns, size
 // ------------------------------------------------------------------------------------------------ FFN
 int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes) {
     if (bytes <= *cap) return 0;
+    if (ctx->capturing)
+        return w4_fail(W4A16_ERR_ARG, "a scratch buffer would grow to %zu bytes while the launch stream is capturing: run the sequence once before the capture", bytes);
     if (*buf) W4_TRY(w4a16_sync(ctx));  // earlier launches may still read the old buffer
     (void)w4a16_free(ctx, *buf);
     *buf = 0;

@@ -29,6 +29,9 @@
 #include "w4a16_common.hpp"
 
 #define W4_DECODE_MAX_KSPLIT 8  // k slices across workgroups; the host clamps to this
+#ifndef W4_TICKET_ORDER
+#define W4_TICKET_ORDER __ATOMIC_RELAXED  // see the hand-over in decode_body
+#endif
 
 // One pipeline stage = the loads of one k tile: RB weight tiles, their scales, and XL loads of x.
 template <int RB, int XL>
@@ -264,26 +267,37 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
         }
     }
     if (nks > 1) {  // wave 0 only from here
-        // Partial tiles and tickets travel as device-scope accesses (write-through stores, cache-bypassing loads), so
-        // no cache write-back or invalidate is needed: a device-scope release fence writes back the whole L2 of the
-        // XCD and costs more per workgroup than the slice itself.
+        // Hand-over of the partial tiles between workgroups (possibly on different XCDs, each with its own L2).
+        // Every access to the workspace is a device-scope access: stores with sc1 are written through to memory, loads
+        // with sc1 are served from memory — the instruction forms the compiler itself emits for agent-scope atomic
+        // stores and loads — so no line of the workspace is ever valid in a non-coherent cache.  Order: the producer
+        // waits until its stores have completed (s_waitcnt vmcnt(0): a write-through store is acknowledged by memory)
+        // before it draws the ticket; the ticket is an agent-scope atomic; the consumer issues its loads only after
+        // the atomic has returned the last ticket, behind an agent-scope acquire fence (buffer_inv sc1: nothing
+        // fetched earlier can satisfy them).  A release fence on the producer side would write back the XCD's whole
+        // L2 (buffer_wbl2) and cost more per workgroup than the slice itself; with write-through stores there is
+        // nothing of this hand-over left in the L2 to write back.
         const __amdgpu_buffer_rsrc_t wr = w4_make_rsrc(ws, (unsigned)gridDim.x * (unsigned)nks * (RB * 1024u));
-        const unsigned mine = ((unsigned)blockIdx.x * RB * 64u + (unsigned)lane) * 16u;
         const unsigned slice = (unsigned)gridDim.x * (RB * 1024u);  // bytes per k slice
+        const unsigned mine = ((unsigned)blockIdx.x * RB * 64u + (unsigned)lane) * 16u;
         constexpr int DEV = 16;                                     // cache policy: device scope (sc1)
+        // The slice offset travels in the vector offset and the scalar offset is the constant 0: for a store of more
+        // than 8 bytes per lane the hardware reads its data registers after issue, and the compiler inserts the wait
+        // state that a following write to them needs only for this form (with a register scalar offset it does not,
+        // and its next instruction, v_mov_b32 of the first data register, gave one wrong dword in lanes 12..15 of every
+        // 16).  The tiles are also kept live until the stores have completed.
+        const unsigned park = mine + (unsigned)ky * slice;
 #pragma unroll
         for (int rb = 0; rb < RB; rb++)
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, acc[rb]), wr, mine + rb * 1024u, ky * slice, DEV);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, acc[rb]), wr, park + rb * 1024u, 0, DEV);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores have reached memory before the ticket is drawn
-        // ... and the tiles stay in their registers until then: a 16-byte buffer store with a register scalar offset
-        // reads its data after issue, and the compiler models no hazard for that form
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) asm volatile("" ::"v"(acc[rb]));
         int ticket = 0;
-        if (lane == 0) ticket = __hip_atomic_fetch_add(tickets + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) ticket = __hip_atomic_fetch_add(tickets + blockIdx.x, 1, W4_TICKET_ORDER, __HIP_MEMORY_SCOPE_AGENT);
         ticket = __builtin_amdgcn_readfirstlane(ticket);
         if (ticket != nks - 1) return;
-        asm volatile("" ::: "memory");
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
             f4_t part[W4_DECODE_MAX_KSPLIT];

@@ -581,22 +581,24 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     if (!active) return;
     if (KS && nks > 1) {
         // every wave on its own: park the partial tiles (device-scope stores), draw the (block, wave) ticket, and the
-        // wave that draws the last one adds the slices in slice order and stores (see the dense decode kernel)
+        // wave that draws the last one adds the slices in slice order and stores.  The hand-over is the one of the
+        // dense decode kernel (decode.hip): write-through stores completed before the agent-scope ticket atomic,
+        // cache-bypassing loads behind an agent-scope acquire fence in the wave that drew the last ticket; the slice
+        // offset travels in the vector offset (scalar offset 0) so that the compiler inserts the wait state a write to
+        // the data registers of a 16-byte store needs, and the tiles stay live until the stores have completed.
         constexpr unsigned PER_WAVE = 2u * TT * 1024u;
         const unsigned per_slice = gridDim.x * (unsigned)W * PER_WAVE;
         const __amdgpu_buffer_rsrc_t wr = w4_make_rsrc(ws, per_slice * (unsigned)nks);
         const unsigned mine = (blockIdx.x * (unsigned)W + (unsigned)wave) * PER_WAVE + (unsigned)lane * 16u;
+        const unsigned park = mine + (unsigned)ky * per_slice;
         constexpr int DEV = 16;  // cache policy: device scope
 #pragma unroll
         for (int rb = 0; rb < 2; rb++)
 #pragma unroll
             for (int tt = 0; tt < TT; tt++)
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, acc[rb][tt]), wr,
-                                                       mine + (unsigned)(rb * TT + tt) * 1024u, ky * per_slice, DEV);
+                                                       park + (unsigned)(rb * TT + tt) * 1024u, 0, DEV);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        // The tiles stay in their registers until the stores have completed: a 16-byte buffer store with a register
-        // scalar offset reads its data after issue, and the compiler, which models no hazard for that form, otherwise
-        // reuses the first data register in the very next instruction (seen as one wrong dword in the last lanes).
 #pragma unroll
         for (int rb = 0; rb < 2; rb++)
 #pragma unroll
@@ -606,7 +608,7 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
         if (lane == 0) ticket = __hip_atomic_fetch_add(tk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         ticket = __builtin_amdgcn_readfirstlane(ticket);
         if (ticket != nks - 1) return;
-        asm volatile("" ::: "memory");
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 #pragma unroll
         for (int rb = 0; rb < 2; rb++)
 #pragma unroll

@@ -37,6 +37,11 @@ _SIGS = {
     "w4a16_event_record": (C.c_int, [C.c_void_p, C.c_void_p]),
     "w4a16_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "w4a16_event_destroy": (None, [C.c_void_p, C.c_void_p]),
+    "w4a16_capture_begin": (C.c_int, [C.c_void_p]),
+    "w4a16_capture_end": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "w4a16_graph_launch": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "w4a16_graph_nodes": (C.c_size_t, [C.c_void_p]),
+    "w4a16_graph_destroy": (None, [C.c_void_p, C.c_void_p]),
     "w4a16_manifest": (C.c_size_t, [C.c_size_t, C.POINTER(C.c_char_p), C.POINTER(C.POINTER(C.c_char_p))]),
     "w4a16_check_shapes": (C.c_int, [C.c_size_t] * 7),
     "w4a16_kernel_sym": (C.c_char_p, [C.c_int, C.c_int]),
@@ -92,6 +97,8 @@ _SIGS = {
     "w4a16_act_mul_f16": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64, C.c_int]),
     "w4a16_chain_forward": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64]),
     "w4a16_chain_forward_fused": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64]),
+    "w4a16_chain_graph_create": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_size_t, C.c_uint64, C.c_size_t,
+                                           C.c_uint64, C.c_int, C.POINTER(C.c_void_p)]),
     "w4a16_bench_chain": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t,
                                     C.c_size_t, C.c_int, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_double)]),
     "w4a16_bench_moe": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.c_size_t, C.c_uint64, C.c_uint64, C.c_uint64,

@@ -56,6 +56,25 @@ class Event:
             self.h = None
 
 
+class Graph:
+    """A captured sequence of launches (GraphEntry of the reference: exec + handle)."""
+
+    def __init__(self, ctx, handle):
+        self.ctx, self.h = ctx, handle
+
+    def launch(self):
+        ffi.check(self.ctx.lib.w4a16_graph_launch(self.ctx.h, self.h))
+
+    @property
+    def nodes(self):
+        return self.ctx.lib.w4a16_graph_nodes(self.h)
+
+    def destroy(self):
+        if self.h and self.ctx.h:
+            self.ctx.lib.w4a16_graph_destroy(self.ctx.h, self.h)
+        self.h = None
+
+
 class Ctx:
     """Device context: launch stream, loaded gfx950 code objects, tracked allocations."""
 
@@ -133,6 +152,15 @@ class Ctx:
 
     def event(self):
         return Event(self)
+
+    # ---- CudaCtx::capture_begin / capture_end + graph_instantiate + graph_upload (ctx/graph.rs:4-85)
+    def capture_begin(self):
+        ffi.check(self.lib.w4a16_capture_begin(self.h))
+
+    def capture_end(self):
+        g = C.c_void_p()
+        ffi.check(self.lib.w4a16_capture_end(self.h, C.byref(g)))
+        return Graph(self, g)
 
 
 class Gptq4:
@@ -372,6 +400,13 @@ class W4a16Dec:
     def chain_forward_fused(self, prefix, layer0, n_layers, x_dev, t, y_dev):
         """The chain with its normalisations deferred across the linears: four launches per layer, t <= 16."""
         ffi.check(self.cc.lib.w4a16_chain_forward_fused(self.cc.h, prefix.encode(), layer0, n_layers, x_dev, t, y_dev))
+
+    def chain_graph(self, prefix, layer0, n_layers, x_dev, t, y_dev, fused=False):
+        """ensure_graph (w4a16_dec/graphs.rs:41-134): one chain step captured for replay."""
+        g = C.c_void_p()
+        ffi.check(self.cc.lib.w4a16_chain_graph_create(self.cc.h, prefix.encode(), layer0, n_layers, x_dev, t, y_dev,
+                                                       int(fused), C.byref(g)))
+        return Graph(self.cc, g)
 
     def bench_chain(self, prefix, n_layers, x_dev, t, y_dev, reps, warmup=1, use_graph=False, fused=False):
         ms, wall = C.c_float(), C.c_double()

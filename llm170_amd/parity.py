@@ -1,0 +1,96 @@
+"""Parity measures shared by the GPU tests, smoke() and bench.py (arithmetic on arrays only; no kernel, no oracle).
+
+Contract (floating-point outputs of the fast kernels against the lane-order f32 reference):
+  * relative L2 error  ||y - y_ref|| / ||y_ref||  <= 1e-3
+  * max |y - y_ref| <= 4 f16 ulp of the output's magnitude, on at least 99.99 % of the outputs with the magnitude
+    taken as it is ("strict"), and on all of them with the magnitude clamped from below at rms(y_ref)/512.
+    Why a floor at all: an output that is small only because thousands of O(rms) terms cancelled carries the f32
+    rounding noise of the *reference's own* summation.  Measured against the compensated f64 dot
+    (crates/core/src/quant/exact.rs:27-53) the lane-order reference itself sits up to 4.3 strict f16 ulp from the
+    exact value on the 27B gate+up shape (1 output in 35 000 beyond 4) and up to 2.7e-6 / 1.0e-5 absolute on the
+    gate+up / down shapes, so no kernel with another summation order can meet 4 ulp of a near-zero magnitude.
+    Where the floor comes from: rms/512 is the largest power-of-two divisor at which 4 f16 ulp of the floor still
+    covers twice the reference's own worst distance from exact on both 27B layer shapes (a kernel that is as
+    accurate as the reference differs from it by at most the sum of the two errors); tests/test_parity_floor.py
+    recomputes that on the CPU, and the GPU tests show per shape that the kernels are as close to the exact value as
+    the reference is (exact_evidence below).  The reference's own gate uses an absolute 1e-5 for its non-bit-exact
+    kernel (crates/server/src/probes/w4a16/gates.rs:134-138).
+"""
+import math
+
+import numpy as np
+
+REL_L2_TOL = 1e-3
+ULP_TOL = 4.0
+CLAMP_DIV = 512.0
+STRICT_PASS_MIN = 0.9999
+
+
+def f16_ulp(mag):
+    """Spacing of binary16 at magnitude `mag` (2^-24 in the subnormal range)."""
+    mag = np.abs(np.asarray(mag, dtype=np.float64))
+    e = np.floor(np.log2(np.maximum(mag, 2.0 ** -14)))
+    return np.ldexp(1.0, (e - 10).astype(np.int64))
+
+
+def compare(y, y_ref):
+    """Returns a dict of error measures; y and y_ref are float arrays of the same shape."""
+    y = np.asarray(y, dtype=np.float64).ravel()
+    r = np.asarray(y_ref, dtype=np.float64).ravel()
+    d = np.abs(y - r)
+    rms = float(np.sqrt(np.mean(r * r))) if r.size else 0.0
+    rel_l2 = float(np.sqrt(np.sum(d * d)) / max(np.sqrt(np.sum(r * r)), 1e-300))
+    strict = d / f16_ulp(r)
+    clamped_mag = np.maximum(np.abs(r), rms / CLAMP_DIV)
+    ulps = d / f16_ulp(clamped_mag)
+    return {
+        "rel_l2": rel_l2,
+        "max_abs": float(d.max()) if d.size else 0.0,
+        "max_ulp": float(ulps.max()) if d.size else 0.0,
+        "max_ulp_strict": float(strict.max()) if d.size else 0.0,
+        "strict_pass_frac": float(np.mean(strict <= ULP_TOL)) if d.size else 1.0,
+        "strict_fail": int(np.sum(strict > ULP_TOL)),
+        "clamped": int(np.sum(np.abs(r) < rms / CLAMP_DIV)),
+        "count": int(d.size),
+        "rms_ref": rms,
+        "ulp_hist": np.histogram(ulps, bins=[0, 0.25, 0.5, 1, 2, 4, np.inf])[0].tolist(),
+    }
+
+
+def strict_ok(m):
+    """At least 99.99 % of the outputs within 4 f16 ulp of their own magnitude; a small array may hold two that are
+    not (one near-zero output of a few hundred would otherwise fail the fraction by itself)."""
+    allowed = max(2, int(math.floor((1.0 - STRICT_PASS_MIN) * m["count"])))
+    return m["strict_fail"] <= allowed
+
+
+def ok(m):
+    return bool(np.isfinite(m["rel_l2"]) and m["rel_l2"] <= REL_L2_TOL and m["max_ulp"] <= ULP_TOL and strict_ok(m))
+
+
+def assert_close(y, y_ref, what=""):
+    m = compare(y, y_ref)
+    assert ok(m), "%s parity: %r" % (what, m)
+    return m
+
+
+def exact_evidence(y, y_ref, y_exact):
+    """Distances of a kernel's outputs and of the lane-order reference's from the compensated f64 dot of the same
+    operands: absolute rms and max, and in strict f16 ulp of the exact value's magnitude.  A kernel passes when it is
+    as close to the exact value as the reference is (within 3x on both measures: the two are different f32 summation
+    orders of the same exact products, neither is privileged)."""
+    y = np.asarray(y, dtype=np.float64).ravel()
+    r = np.asarray(y_ref, dtype=np.float64).ravel()
+    e = np.asarray(y_exact, dtype=np.float64).ravel()
+    dk, dl = np.abs(y - e), np.abs(r - e)
+    u = f16_ulp(e)
+    out = {
+        "kernel_rms_err": float(np.sqrt(np.mean(dk * dk))), "lane_rms_err": float(np.sqrt(np.mean(dl * dl))),
+        "kernel_max_err": float(dk.max()), "lane_max_err": float(dl.max()),
+        "kernel_max_strict_ulp": float((dk / u).max()), "lane_max_strict_ulp": float((dl / u).max()),
+        "kernel_beyond_4ulp": int(np.sum(dk / u > ULP_TOL)), "lane_beyond_4ulp": int(np.sum(dl / u > ULP_TOL)),
+        "count": int(e.size),
+    }
+    out["ok"] = bool(out["kernel_rms_err"] <= 3.0 * out["lane_rms_err"] + 1e-12 and
+                     out["kernel_max_err"] <= 3.0 * out["lane_max_err"] + 1e-12)
+    return out

@@ -21,6 +21,7 @@
  *   orc_tree64 ............ math.fsum on exactly-summable inputs + a pairing-order vector that distinguishes orders
  *   orc_moe_topk .......... KATs qwen35/stages/moe.rs:135-155
  *   orc_exact_dot ......... exact-rational brute force (quant/exact.rs:77-135 precedent)
+ *   orc_exact_dot_sample .. the row function above, call for call; plain f64 dot of the dequantised row
  *   orc_moe_act_silu_f16 .. float64 evaluation of g/(1+exp(-g))*u within one f16 step; special cases g = 0, u = 0,
  *                           large |g| (silu -> g, -> 0)
  *   orc_moe_act_gelu_f16 .. float64 evaluation of 0.5 g (1 + tanh(0.7978846 (g + 0.044715 g^3))) u within one f16 step;
@@ -313,6 +314,24 @@ int orc_gemm_lane_sample(const uint16_t* x, const uint32_t* q, const uint16_t* s
     free(z8);
     free(sf);
     return rc;
+}
+
+/* Sampled outputs of the compensated f64 dot (orc_exact_dot, quant/exact.rs:27-53), activations widened from f16
+ * exactly: out[j] = exact(row rows[j], x row toks[j]).  The yardstick that tells summation-order noise of the f32
+ * lane sum from a kernel's own error. */
+int orc_exact_dot_sample(const uint16_t* x, const uint32_t* q, const uint16_t* s, size_t k, size_t group,
+                         int scale_bf16, const uint32_t* rows, const uint32_t* toks, size_t count, double* out) {
+    if ((group != 128 && group != 32) || k % group != 0) return -1;
+    size_t ng = k / group;
+    float* xf = (float*)malloc(k * sizeof(float));
+    for (size_t j = 0; j < count; j++) {
+        const uint16_t* xr = x + (size_t)toks[j] * k;
+        for (size_t i = 0; i < k; i++) xf[i] = orc_half_to_f32(xr[i]);
+        out[j] = orc_exact_dot((const uint8_t*)(q + (size_t)rows[j] * (k / 8)), (const uint8_t*)(s + (size_t)rows[j] * ng),
+                               xf, k, group, scale_bf16);
+    }
+    free(xf);
+    return 0;
 }
 
 /* ---- crates/backend-gpu/src/rawcuda/w4a16_dec/mod.rs:168-185 (moe_topk) ≡ qwen35/stages/moe.rs:8-31:

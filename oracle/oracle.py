@@ -51,6 +51,8 @@ def lib():
         L.orc_gemm_lane.restype = C.c_int
         L.orc_gemm_lane_sample.argtypes = [u16p, u32p, u16p, sz, sz, C.c_int, u32p, u32p, sz, f32p]
         L.orc_gemm_lane_sample.restype = C.c_int
+        L.orc_exact_dot_sample.argtypes = [u16p, u32p, u16p, sz, sz, C.c_int, u32p, u32p, sz, f64p]
+        L.orc_exact_dot_sample.restype = C.c_int
         L.orc_moe_topk.argtypes, L.orc_moe_topk.restype = [f32p, sz, sz, u32p, f32p], None
         L.orc_silu_mul_f16.argtypes, L.orc_silu_mul_f16.restype = [C.c_float, C.c_float], C.c_uint16
         L.orc_f32_to_f16_array.argtypes, L.orc_f32_to_f16_array.restype = [f32p, sz, u16p], None
@@ -183,6 +185,19 @@ def gemm_lane_sample(x, q, s, k, group, rows, toks, scale_bf16=False):
                                     _p(out, C.c_float))
     if rc != 0:
         raise ValueError("gemm_lane_sample: shape contract violated")
+    return out
+
+
+def exact_dot_sample(x, q, s, k, group, rows, toks, scale_bf16=False):
+    """f64 [count]: the compensated f64 dot (quant/exact.rs:27-53) of row rows[j] with x row toks[j]."""
+    x, q, s = _c(x, np.uint16).ravel(), _c(q, np.uint32).ravel(), _c(s, np.uint16).ravel()
+    rows, toks = _c(rows, np.uint32), _c(toks, np.uint32)
+    out = np.empty(rows.size, np.float64)
+    rc = lib().orc_exact_dot_sample(_p(x, C.c_uint16), _p(q, C.c_uint32), _p(s, C.c_uint16), k, group,
+                                    int(scale_bf16), _p(rows, C.c_uint32), _p(toks, C.c_uint32), rows.size,
+                                    _p(out, C.c_double))
+    if rc != 0:
+        raise ValueError("exact_dot_sample: shape contract violated")
     return out
 
 

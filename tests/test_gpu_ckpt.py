@@ -5,7 +5,7 @@ import pytest
 
 from llm170_amd import ckpt, gen, ops
 from tests import ckpt_fixture as fx
-from tests import parity
+from llm170_amd import parity
 
 pytestmark = pytest.mark.gpu
 
@@ -85,7 +85,7 @@ def test_fused_projections_from_a_checkpoint(tmp_path, orc):
         ref_act = orc.silu_mul_f16_rows(gu)
         a, b = gen.f16_bits_to_f32(act).astype(np.float64), gen.f16_bits_to_f32(ref_act).astype(np.float64)
         rms = float(np.sqrt(np.mean(b * b)))
-        assert np.all(np.abs(a - b) <= 2 * parity.f16_ulp(np.maximum(np.abs(b), rms / 128)))
+        assert np.all(np.abs(a - b) <= 2 * parity.f16_ulp(np.maximum(np.abs(b), rms / parity.CLAMP_DIV)))
         assert np.mean(act == ref_act) > 0.97
     finally:
         cc.close()

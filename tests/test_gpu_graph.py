@@ -1,0 +1,155 @@
+"""Capture and replay of the launch stream through the C ABI (w4a16_capture_begin / _end, w4a16_graph_launch,
+w4a16_chain_graph_create): replays give the bits of eager passes, follow the contents of their input buffer, and
+nothing that allocates, frees or waits is accepted while capturing.  Each graph is replayed several times with eager
+work and synchronisations of the same context in between."""
+import numpy as np
+import pytest
+
+from llm170_amd import ffi, gen, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def dec():
+    d = ops.W4a16Dec()
+    yield d
+    d.cc.close()
+
+
+def test_capture_of_plain_abi_calls_replays_eager_bits(dec, orc):
+    """A caller's own sequence: two linears (the second split over k across workgroups, so its tickets must be back
+    at zero after every replay) and a fill, captured once, replayed five times with other launches in between."""
+    cc = dec.cc
+    n1, k1, n2, g, t = 2048, 512, 256, 128, 4
+    q1, s1, x = gen.make_linear(n1, k1, g, t, seed=3)
+    q2, s2, _ = gen.make_linear(n2, n1, g, 1, seed=4)
+    dec.upload_lin_g("g1", q1, s1, n1, k1, g, False)
+    dec.upload_lin_g("g2", q2, s2, n2, n1, g, False)
+    px, ph, py = cc.to_device(x), cc.alloc(t * n1 * 2), cc.alloc(t * n2 * 4)
+    dec.set_decode_ksplit(4)
+    try:
+        def step():
+            cc.memset0(py, t * n2 * 4)
+            dec.lin_forward("g1", px, ph, t, out_f16=True, path=ops.PATH_DECODE)
+            dec.lin_forward("g2", ph, py, t, path=ops.PATH_DECODE)
+        step()  # sizes the split workspace
+        eager = cc.d2h(py, (t, n2), np.uint32)
+        cc.capture_begin()
+        step()
+        graph = cc.capture_end()
+        assert graph.nodes == 3
+        for i in range(5):
+            cc.memset0(py, t * n2 * 4)
+            graph.launch()
+            assert np.array_equal(cc.d2h(py, (t, n2), np.uint32), eager), "replay %d" % i
+            dec.lin_forward("g1", px, ph, t, out_f16=True, path=ops.PATH_DECODE)  # eager work between replays
+            cc.sync()
+        # a replay reads its input buffer when it runs: new x, new result, equal to an eager pass on it
+        x2 = gen.normal_f16(99, (t, k1))
+        cc.h2d(px, x2)
+        graph.launch()
+        got = cc.d2h(py, (t, n2), np.uint32)
+        step()
+        assert np.array_equal(got, cc.d2h(py, (t, n2), np.uint32)) and not np.array_equal(got, eager)
+        graph.destroy()
+    finally:
+        dec.set_decode_ksplit(0)
+        for p in (px, ph, py):
+            cc.free(p)
+
+
+def test_capture_refuses_what_cannot_be_recorded(dec):
+    cc = dec.cc
+    q, s, x = gen.make_linear(64, 256, 128, 2, seed=8)
+    dec.upload_lin_g("cap", q, s, 64, 256, 128, False)
+    px, py = cc.to_device(x), cc.alloc(2 * 64 * 4)
+    cc.capture_begin()
+    try:
+        for call in (lambda: cc.alloc(64), lambda: cc.free(py), cc.sync, lambda: cc.h2d(px, x),
+                     lambda: cc.d2h(py, (2, 64), np.float32), cc.capture_begin,
+                     lambda: dec.gemv_host("cap", x, t=2)):
+            with pytest.raises(ops.W4a16Error) as e:
+                call()
+            assert e.value.code == ffi.ERR_ARG and "captur" in str(e.value)
+        dec.lin_forward("cap", px, py, 2, path=ops.PATH_DECODE)
+    finally:
+        graph = cc.capture_end()
+    assert graph.nodes == 1
+    graph.launch()
+    want = dec.gemv_host("cap", x, t=2, path=ops.PATH_DECODE)
+    assert np.array_equal(cc.d2h(py, (2, 64), np.float32).view(np.uint32), want.view(np.uint32))
+    graph.destroy()
+    with pytest.raises(ops.W4a16Error):  # nothing to end
+        cc.capture_end()
+    cc.capture_begin()
+    with pytest.raises(ops.W4a16Error):  # an empty capture
+        cc.capture_end()
+    cc.free(px)
+    cc.free(py)
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_chain_graph_small(dec, orc, fused):
+    layers, hidden, n_qkv, n_ff, t = 3, 256, 384, 512, 4
+    cc = dec.cc
+    dec.upload_chain_synth("gsmall", layers, hidden, n_qkv, n_ff, 128)
+    x = gen.normal_f16(12, (t, hidden))
+    px, py = cc.to_device(x), cc.alloc(t * hidden * 2)
+    run = dec.chain_forward_fused if fused else dec.chain_forward
+    run("gsmall", 0, layers, px, t, py)
+    eager = cc.d2h(py, (t, hidden), np.uint16)
+    graph = dec.chain_graph("gsmall", 0, layers, px, t, py, fused=fused)
+    assert graph.nodes == layers * (4 if fused else 7) + (1 if fused else 0)
+    for i in range(4):
+        cc.memset0(py, t * hidden * 2)
+        graph.launch()
+        assert np.array_equal(cc.d2h(py, (t, hidden), np.uint16), eager), "replay %d" % i
+        run("gsmall", 1, 1, px, t, py)  # eager work between replays, same scratch
+        cc.sync()
+    graph.destroy()
+    cc.free(px)
+    cc.free(py)
+
+
+def test_chain_graph_64_layers_at_27b_shapes(dec):
+    """The chain the benchmark times: 64 layers of QKV 5120->7168, O 5120->5120, gate|up 5120->34816, down
+    17408->5120 at M = 4 (10.9 GB of device-generated weights).  Output finite, of unit mean square, the same bits
+    from eager passes and graph replays, for both statements of the chain; the two statements agree to the f16
+    roundings they place differently."""
+    layers, hidden, n_qkv, n_ff, t = 64, 5120, 7168, 17408, 4
+    cc = dec.cc
+    say("chain 64: generating")
+    dec.upload_chain_synth("c64", layers, hidden, n_qkv, n_ff, 128)
+    for l in range(layers):
+        for role in ops.W4a16Dec.CHAIN_ROLES:
+            dec.drop_raw("c64.%d.%s" % (l, role))
+    px, py = cc.to_device(gen.normal_f16(404, (t, hidden))), cc.alloc(t * hidden * 2)
+    out = {}
+    for fused in (False, True):
+        run = dec.chain_forward_fused if fused else dec.chain_forward
+        run("c64", 0, layers, px, t, py)
+        eager = cc.d2h(py, (t, hidden), np.uint16)
+        v = gen.f16_bits_to_f32(eager).astype(np.float64)
+        assert np.all(np.isfinite(v))
+        assert np.allclose(np.mean(v * v, axis=1), 1.0, atol=2e-3)
+        run("c64", 0, layers, px, t, py)
+        assert np.array_equal(cc.d2h(py, (t, hidden), np.uint16), eager)  # eager passes repeat bit for bit
+        say("chain 64: capturing, fused =", fused)
+        graph = dec.chain_graph("c64", 0, layers, px, t, py, fused=fused)
+        assert graph.nodes == layers * (4 if fused else 7) + (1 if fused else 0)
+        for i in range(3):
+            cc.memset0(py, t * hidden * 2)
+            graph.launch()
+            assert np.array_equal(cc.d2h(py, (t, hidden), np.uint16), eager), "replay %d fused %d" % (i, fused)
+        graph.destroy()
+        out[fused] = v
+    rel = np.sqrt(np.sum((out[True] - out[False]) ** 2) / np.sum(out[False] ** 2))
+    say("chain 64: fused vs unfused rel-L2", rel)
+    assert rel < 0.05  # 64 layers of re-normalised random projections amplify the f16 rounding differences
+    cc.free(px)
+    cc.free(py)

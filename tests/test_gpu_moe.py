@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 
 from llm170_amd import gen, ops
-from tests import parity
+from llm170_amd import parity
 
 pytestmark = pytest.mark.gpu
 
@@ -134,7 +134,7 @@ def _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf
     # (about 1e-6 absolute here), so a few round to the neighbouring f16 before the activation, and a sum that
     # cancelled to almost nothing moves by many of its own tiny f16 steps.  Tolerance: the device value must lie
     # inside the envelope of silu(g')*u' over g', u' within ONE f16 step of the oracle's gate/up — the step taken at
-    # a magnitude clamped from below at rms/128, the rule of tests/parity.py — widened by 1.5 f16 steps of the
+    # a magnitude clamped from below as in llm170_amd/parity.py — widened by 1.5 f16 steps of the
     # result (final rounding, exp implementation); and nearly all elements must be identical.
     g0 = full["c13"][:, :n_ff].view(np.float16).astype(np.float64)
     u0 = full["c13"][:, n_ff:].view(np.float16).astype(np.float64)
