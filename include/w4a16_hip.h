@@ -69,6 +69,11 @@ int w4a16_has_symbol(w4a16_ctx* ctx, const char* symbol);
 int w4a16_launch(w4a16_ctx* ctx, const char* symbol, unsigned gx, unsigned gy, unsigned block, unsigned shmem,
                  void** params);
 
+/* Name of the kernel the most recent launch of this context used ("" before the first), whichever entry point made
+ * it: what a profile is matched against (the reference resolves the launched function's name per launch for its
+ * profile report, prof_mark, ctx/prof.rs:56-72).  Valid until the context is destroyed. */
+const char* w4a16_last_launch_symbol(w4a16_ctx* ctx);
+
 /* CudaCtx::alloc / free / h2d / d2h / d2d / memset (ctx/mem.rs:4-44, 164-336).  Copies and the fill are ordered on
  * the launch stream; h2d and d2h return after the data has moved. */
 int w4a16_alloc(w4a16_ctx* ctx, size_t bytes, uint64_t* dptr);
@@ -188,7 +193,12 @@ int w4a16_lin_forward_glu_act(w4a16_ctx* ctx, const char* name, uint64_t x_dev, 
  *              those of v, and v is what continues;
  *   nw_dev     f32 [n], the norm weight of the output rows (norm.cu:19-23): y_dev receives v * nw.
  * The consumer's output is then 1/rms(v) * W2 (v * nw), the reference's W2 (v * 1/rms(v) * nw) with the f16 rounding
- * of the activations taken before the 1/rms factor instead of after it. */
+ * of the activations taken before the 1/rms factor instead of after it.
+ * RANGE PRECONDITION: the activations travel between the two launches as f16 WITHOUT their 1/rms factor, so every
+ * element of v (of v * nw with a norm weight) must lie inside the f16 range: beyond 65504 it becomes Inf (and the
+ * consumer's output NaN) where norm_resid, which normalises in f32 first, stays finite; rows whose elements fall below
+ * 6e-5 lose relative precision to f16 subnormals.  Nothing is detected at run time.  Residual streams of trained
+ * models sit well inside; the synthetic 64-layer chain of random projections does not (see w4a16_chain_forward_fused). */
 int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
                                     uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_dev,
                                     int out_f16, uint64_t stats_out_dev, size_t stat_rows, size_t* n_stats_out,
@@ -354,7 +364,11 @@ int w4a16_chain_forward(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_
  *     gu = r(v2) * ffn_gate_up(b)            c = silu_mul_f16(gu)
  *     v4 = ffn_down(c)                       x[l+1] = f16(v4), s[l+1] = r(v4)
  * and y = rms_f16(v4) after the last layer: the function of w4a16_chain_forward with the factors applied after the
- * linears instead of before the roundings to f16 (results agree to those roundings). */
+ * linears instead of before the roundings to f16 (results agree to those roundings) — as long as v4, which crosses
+ * the layer boundary as f16 without its factor, stays inside the f16 range (the precondition of
+ * w4a16_lin_forward_deferred_norm).  With random weights of mean -0.5 and no residual stream the rows of v4 drift
+ * apart by orders of magnitude within three layers (rows aligned with the weights' mean direction switch the gated
+ * unit fully on or off), so deep synthetic chains must use w4a16_chain_forward. */
 int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers, uint64_t x_dev,
                               size_t t, uint64_t y_dev);
 /* ensure_graph (w4a16_dec/graphs.rs:41-134): one decode step of the chain as a replayable graph.  Runs the chain once

@@ -66,8 +66,7 @@ static const char* const kDecodeSyms[] = {
 static const char* const kPrefillSyms[] = {"w4a16_prefill_g128_f16", "w4a16_prefill_g128_bf16", "w4a16_prefill_g32_f16",
                                            "w4a16_prefill_g32_bf16", "w4a16_prefill_g128_f16_m64", "w4a16_prefill_g128_bf16_m64", "w4a16_prefill_g32_f16_m64",
                                            "w4a16_prefill_g32_bf16_m64", "w4a16_prefill_splitk_sum", nullptr};
-static const char* const kUtilSyms[] = {"w4a16_fill0_u32", "w4a16_copy_u4", "w4a16_read_u4", "w4a16_mfma_peak_f16",
-                                         nullptr};
+static const char* const kUtilSyms[] = {"w4a16_fill0_u32", nullptr};
 static const char* const kGlueSyms[] = {"w4a16_rms_rescale_f16", "w4a16_silu_mul_f16", "w4a16_synth_q", "w4a16_synth_s",
                                         "w4a16_norm_resid", nullptr};
 #define W4_MOE_FAMILY(P)                                                                                      \
@@ -231,14 +230,14 @@ extern "C" void w4a16_ctx_destroy(w4a16_ctx* ctx) {
 
 extern "C" int w4a16_has_symbol(w4a16_ctx* ctx, const char* symbol) {
     if (!ctx || !symbol) return w4_fail(W4A16_ERR_ARG, "has_symbol: null argument");
-    if (ctx->functions.find(symbol) == ctx->functions.end())
+    if (ctx->functions.find(std::string_view(symbol)) == ctx->functions.end())
         return w4_fail(W4A16_ERR_SYMBOL, "function: symbol %s is not loaded", symbol);
     return 0;
 }
 
 int w4_launch(w4a16_ctx* ctx, const char* symbol, unsigned gx, unsigned gy, unsigned block, unsigned shmem,
               void** params) {
-    auto it = ctx->functions.find(symbol);
+    auto it = ctx->functions.find(std::string_view(symbol));
     if (it == ctx->functions.end()) return w4_fail(W4A16_ERR_SYMBOL, "function: symbol %s is not loaded", symbol);
     if (gx == 0 || gy == 0 || block == 0 || block > 1024)
         return w4_fail(W4A16_ERR_ARG, "launch %s: grid %ux%u block %u", symbol, gx, gy, block);
@@ -251,12 +250,15 @@ int w4_launch(w4a16_ctx* ctx, const char* symbol, unsigned gx, unsigned gy, unsi
             return w4_fail((int)e, "hipFuncSetAttribute(%s, dynamic LDS %u): %s (%d)", symbol, shmem, hipGetErrorString(e),
                            (int)e);
     }
+    ctx->last_symbol = it->first.c_str();
     e = hipModuleLaunchKernel(it->second, gx, gy, 1, block, 1, 1, shmem, ctx->stream, params, nullptr);
     if (e != hipSuccess)
         return w4_fail((int)e, "hipModuleLaunchKernel(%s grid %ux%u block %u shmem %u): %s (%d)", symbol, gx, gy, block,
                        shmem, hipGetErrorString(e), (int)e);
     return 0;
 }
+
+extern "C" const char* w4a16_last_launch_symbol(w4a16_ctx* ctx) { return ctx ? ctx->last_symbol : ""; }
 
 extern "C" int w4a16_launch(w4a16_ctx* ctx, const char* symbol, unsigned gx, unsigned gy, unsigned block,
                             unsigned shmem, void** params) {

@@ -6,6 +6,7 @@
 #include <cstdint>
 #include <map>
 #include <string>
+#include <string_view>
 #include <unordered_map>
 #include <vector>
 
@@ -70,11 +71,11 @@ struct w4a16_ctx {
     hipStream_t stream = nullptr;   // launch stream (reference: CudaCtx.stream)
     hipStream_t stream2 = nullptr;  // second stream (reference: CudaCtx.stream2); copies that must not serialise
     std::vector<hipModule_t> modules;
-    std::unordered_map<std::string, hipFunction_t> functions;
+    std::map<std::string, hipFunction_t, std::less<>> functions;  // looked up by string_view: a launch allocates nothing
     std::unordered_map<uint64_t, size_t> allocs;
     size_t allocated = 0;
-    std::map<std::string, W4Lin> lins;
-    std::map<std::string, W4Experts> experts;
+    std::map<std::string, W4Lin, std::less<>> lins;
+    std::map<std::string, W4Experts, std::less<>> experts;
     W4MoeScratch moe;
     W4ChainScratch chain;
     int moe_block = 0, moe_waves = 0;  // 0 = automatic
@@ -88,6 +89,7 @@ struct w4a16_ctx {
     uint64_t prefill_ws = 0;                                    // f32 partials of a split-K prefill launch
     size_t prefill_ws_cap = 0;
     int cu_count = 0;
+    const char* last_symbol = "";  // kernel of the most recent launch (a key of `functions`: stable storage)
     bool capturing = false;  // between w4a16_capture_begin and w4a16_capture_end: nothing may allocate, free or wait
 };
 

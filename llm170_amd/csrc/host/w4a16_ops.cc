@@ -63,9 +63,17 @@ static int pick_decode_shape(const w4a16_ctx* ctx, const W4Lin& L, size_t t, int
     return 0;
 }
 
-// k slices across workgroups for a decode launch of `blocks` workgroups, and the workspace they need.  The tickets are
-// zeroed when (re)allocated; every launch leaves them zero.
-static int decode_split(w4a16_ctx* ctx, const W4Lin& L, size_t t, size_t blocks, int rb, int* waves, int* nks_out) {
+// k slices across workgroups for a decode launch of `blocks` workgroups, and the workspace they need: partial tiles and
+// one ticket per workgroup of a slice.  The tickets are zero when (re)allocated and every launch leaves them zero.
+// With `fixed` the workspace is the caller's (a buffer of stated size that cannot grow): a launch that needs more is
+// refused, nothing is allocated.
+struct DecodeWorkspace {
+    uint64_t ws = 0, tickets = 0;
+    size_t ws_cap = 0, tickets_cap = 0;  // bytes
+};
+
+static int decode_split(w4a16_ctx* ctx, const W4Lin& L, size_t t, size_t blocks, int rb, int* waves, int* nks_out,
+                        DecodeWorkspace* out, const DecodeWorkspace* fixed) {
     const int kt_n = (int)(L.k / 128);
     int nks = 1;
     if (ctx->decode_ksplit > 0) {
@@ -80,11 +88,24 @@ static int decode_split(w4a16_ctx* ctx, const W4Lin& L, size_t t, size_t blocks,
     nks = std::max(1, std::min(nks, kt_n / 2));
     if (nks > 1) {
         *waves = std::max(1, std::min(*waves, kt_n / nks));
-        W4_TRY(w4_ensure(ctx, &ctx->decode_ws, &ctx->decode_ws_cap, blocks * (size_t)rb * 1024 * (size_t)nks));
-        if (blocks * 4 > ctx->decode_tickets_cap) {
-            W4_TRY(w4_ensure(ctx, &ctx->decode_tickets, &ctx->decode_tickets_cap, std::max<size_t>(blocks * 4, 16384)));
-            W4_TRY(w4a16_memset0(ctx, ctx->decode_tickets, ctx->decode_tickets_cap));
+        const size_t ws_need = blocks * (size_t)rb * 1024 * (size_t)nks, tk_need = blocks * 4;
+        if (fixed) {
+            if (ws_need > fixed->ws_cap || tk_need > fixed->tickets_cap)
+                return w4_fail(W4A16_ERR_SHAPE, "decode: the split over k needs %zu bytes of partial tiles and %zu of tickets, the fixed workspace holds %zu and %zu",
+                               ws_need, tk_need, fixed->ws_cap, fixed->tickets_cap);
+        } else {
+            W4_TRY(w4_ensure(ctx, &ctx->decode_ws, &ctx->decode_ws_cap, ws_need));
+            if (tk_need > ctx->decode_tickets_cap) {
+                W4_TRY(w4_ensure(ctx, &ctx->decode_tickets, &ctx->decode_tickets_cap, std::max<size_t>(tk_need, 16384)));
+                W4_TRY(w4a16_memset0(ctx, ctx->decode_tickets, ctx->decode_tickets_cap));
+            }
         }
+    }
+    if (fixed) {
+        *out = *fixed;
+    } else {
+        out->ws = ctx->decode_ws;
+        out->tickets = ctx->decode_tickets;
     }
     *nks_out = nks;
     return 0;
@@ -120,7 +141,7 @@ static int check_decode_norm(const W4Lin& L, size_t t, const DecodeNorm& nm) {
 }
 
 static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16,
-                         DecodeNorm* norm = nullptr) {
+                         DecodeNorm* norm = nullptr, const DecodeWorkspace* fixed_ws = nullptr) {
     if (t == 0 || t > 16) return w4_fail(W4A16_ERR_SHAPE, "decode: t=%zu outside 1..16", t);
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode: linear has no tiled copy (needs k %% 128 == 0)");
     int rb = 0, waves = 0;
@@ -135,8 +156,9 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
     const size_t blocks = ceil_div(L.row_blocks, (size_t)rb);
     int nks = 1;
-    W4_TRY(decode_split(ctx, L, t, blocks, rb, &waves, &nks));
-    uint64_t ws = ctx->decode_ws, tk = ctx->decode_tickets;
+    DecodeWorkspace W;
+    W4_TRY(decode_split(ctx, L, t, blocks, rb, &waves, &nks, &W, fixed_ws));
+    uint64_t ws = W.ws, tk = W.tickets;
     // launch geometry as kernel arguments (the kernel reads nothing from the dispatch packet): k tiles per slice and
     // per wave, both rounded up
     int kt_per_slice = (int)ceil_div(L.k / 128, (size_t)nks), kt_per_wave = (kt_per_slice + waves - 1) / waves;
@@ -175,8 +197,9 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = 1;
     const size_t blocks = L.row_blocks / 2;
     int nks = 1;
-    W4_TRY(decode_split(ctx, L, t, blocks, 2, &waves, &nks));
-    uint64_t ws = ctx->decode_ws, tk = ctx->decode_tickets;
+    DecodeWorkspace W;
+    W4_TRY(decode_split(ctx, L, t, blocks, 2, &waves, &nks, &W, nullptr));
+    uint64_t ws = W.ws, tk = W.tickets;
     int kt_per_slice = (kt_n + nks - 1) / nks, kt_per_wave = (kt_per_slice + waves - 1) / waves;
     DecodeNorm none;
     DecodeNorm& nm = norm ? *norm : none;
@@ -323,10 +346,20 @@ extern "C" int w4a16_upload_lin(w4a16_ctx* ctx, const char* name, const void* q,
     {
         const uint16_t* sp = static_cast<const uint16_t*>(s);
         const size_t ns = slen_bytes / 2;
+        // "regular": what the MFMA prefill kernel can carry as a running unit (it multiplies its accumulators by
+        // s_prev / s_cur at every group boundary and holds sum / s_cur) — finite, non-zero, and for bf16 scales inside
+        // [2^-60, 2^60], so that neither a quotient of two scales nor an accumulator expressed in the smallest one
+        // leaves the f32 range (f16 scales span 2^-24 .. 2^16 and always qualify; a bf16 subnormal or 1e-38 does not).
+        // Other linears are served by the streaming kernels, which only ever multiply by a scale.
         const unsigned expmask = scale_bf16 ? 0x7F80u : 0x7C00u;
         for (size_t i = 0; i < ns; i++) {
             const unsigned b = sp[i];
-            if ((b & 0x7FFFu) == 0 || (b & expmask) == expmask) {
+            bool bad = (b & 0x7FFFu) == 0 || (b & expmask) == expmask;
+            if (!bad && scale_bf16) {
+                const unsigned e = (b >> 7) & 0xFFu;  // biased exponent, 127 = 2^0
+                bad = e < 127u - 60u || e > 127u + 60u;
+            }
+            if (bad) {
                 L.scales_regular = false;
                 break;
             }
@@ -433,7 +466,7 @@ int w4_register_lin(w4a16_ctx* ctx, const char* name, W4Lin& L) {
 
 int w4_find_lin(w4a16_ctx* ctx, const char* name, W4Lin** out) {
     if (!ctx || !name) return w4_fail(W4A16_ERR_ARG, "lin: null argument");
-    auto it = ctx->lins.find(name);
+    auto it = ctx->lins.find(std::string_view(name));  // transparent comparator: no std::string is built
     if (it == ctx->lins.end()) return w4_fail(W4A16_ERR_NOT_FOUND, "lin %s: not registered", name);
     *out = &it->second;
     return 0;

@@ -369,7 +369,13 @@ __device__ __forceinline__ void moe_down_sum_body(const char* __restrict__ qa, c
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) acc[rb][i] = moe_round_f16(acc[rb][i] * wgt);
+        for (int i = 0; i < 4; i++) {
+            // the product is rounded to f32 first, as where c2 is materialised (the compiler would otherwise fold the
+            // multiply into the conversion, v_fma_mixlo_f16: one rounding of the exact product instead of two)
+            float p = acc[rb][i] * wgt;
+            asm volatile("" : "+v"(p));
+            acc[rb][i] = moe_round_f16(p);
+        }
         red[(wave * RB + rb) * 64 + lane] = acc[rb];
     }
     __syncthreads();

@@ -25,6 +25,7 @@ _SIGS = {
     "w4a16_module_load": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_char_p), C.c_size_t]),
     "w4a16_has_symbol": (C.c_int, [C.c_void_p, C.c_char_p]),
     "w4a16_launch": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint, C.c_uint, C.c_uint, C.c_uint, C.POINTER(C.c_void_p)]),
+    "w4a16_last_launch_symbol": (C.c_char_p, [C.c_void_p]),
     "w4a16_alloc": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_uint64)]),
     "w4a16_free": (C.c_int, [C.c_void_p, C.c_uint64]),
     "w4a16_h2d": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_size_t]),

@@ -153,6 +153,14 @@ class Ctx:
     def event(self):
         return Event(self)
 
+    def last_launch_symbol(self):
+        return self.lib.w4a16_last_launch_symbol(self.h).decode()
+
+    def module_load(self, key, image, symbols):
+        """CudaCtx::load_fatbin: a gfx950 code object image and the symbols to resolve from it."""
+        arr = (C.c_char_p * len(symbols))(*[s.encode() for s in symbols])
+        ffi.check(self.lib.w4a16_module_load(self.h, key.encode(), image, len(image), arr, len(symbols)))
+
     # ---- CudaCtx::capture_begin / capture_end + graph_instantiate + graph_upload (ctx/graph.rs:4-85)
     def capture_begin(self):
         ffi.check(self.lib.w4a16_capture_begin(self.h))

@@ -410,3 +410,40 @@ def test_prefill_refuses_irregular_scales_and_auto_falls_back(dec, orc):
     x_long = np.concatenate([x, x, x, x, x])[:170]  # beyond 64 rows the fallback is the streaming kernel as well
     parity.assert_close(_device_forward(dec, "irr", x_long, 170, ops.PATH_AUTO),
                         orc.gemm_lane(x_long, 170, q, s, n, k, group, threads=8), "auto fallback, 170 rows")
+
+
+def test_bf16_scales_of_extreme_range_take_the_streaming_path(dec, orc):
+    """A bf16 row whose scales span the f32 range (1.0 next to 1e-38, and a subnormal): the running-unit rescale of
+    the MFMA kernel would overflow, so such a linear is refused there and AUTO serves it with the streaming kernel;
+    the result is finite and meets the contract like any other."""
+    n, k, group, t = 64, 512, 128, 100
+    q, s, x = gen.make_linear(n, k, group, t, seed=10)
+    s = (gen.f16_bits_to_f32(s).view(np.uint32) >> 16).astype(np.uint16)
+    s[5] = [0x3F80, 0x006D, 0x3F80, 0x006D]   # 1.0, 1e-38, 1.0, 1e-38
+    s[9, 2] = 0x0001                          # a bf16 subnormal
+    s[11] = [0x5F00, 0x1E80, 0x5F00, 0x1E80]   # 2^63 next to 2^-66
+    dec.upload_lin_g("wild", q, s, n, k, group, True)
+    with pytest.raises(ops.W4a16Error) as e:
+        _device_forward(dec, "wild", x, t, ops.PATH_PREFILL)
+    assert e.value.code == ffi.ERR_UNSUPPORTED
+    got = _device_forward(dec, "wild", x, t, ops.PATH_AUTO)
+    assert np.all(np.isfinite(got))
+    want = orc.gemm_lane(x, t, q, s, n, k, group, scale_bf16=True, threads=8)
+    # rows 5, 9 and 11 have their own magnitudes: compare them and the ordinary rows separately
+    special = np.zeros(n, bool)
+    special[[5, 9, 11]] = True
+    parity.assert_close(got[:, ~special], want[:, ~special], "wild scales, ordinary rows")
+    for r in (5, 9, 11):
+        assert np.allclose(got[:, r], want[:, r], rtol=1e-4, atol=0), r
+    # one notch inside the bound the MFMA kernel still serves the linear
+    s2 = s.copy()
+    s2[5] = [0x3F80, 0x2180, 0x3F80, 0x2180]  # 1.0 next to 2^-60
+    s2[9, 2] = 0x3F80
+    s2[11] = [0x5D00, 0x2180, 0x5D00, 0x2180]  # 2^59 next to 2^-60
+    dec.upload_lin_g("tame", q, s2, n, k, group, True)
+    got2 = _device_forward(dec, "tame", x, t, ops.PATH_PREFILL)
+    want2 = orc.gemm_lane(x, t, q, s2, n, k, group, scale_bf16=True, threads=8)
+    assert np.all(np.isfinite(got2))
+    parity.assert_close(got2[:, ~special], want2[:, ~special], "tame scales, ordinary rows")
+    for r in (5, 11):
+        assert np.allclose(got2[:, r], want2[:, r], rtol=1e-4, atol=0), r

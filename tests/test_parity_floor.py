@@ -65,6 +65,8 @@ def test_compare_counts_strict_failures():
     y[2::4] += 3e-7  # a quarter of the outputs: the strict fraction fails although every clamped distance is tiny
     m = parity.compare(y, ref)
     assert m["max_ulp"] < 0.5 and not parity.ok(m)
-    e = parity.exact_evidence(ref + 1e-6, ref + 2e-6, ref)
+    big = np.array([1.0, 2.0, 3.0, 4.0] * 2500)
+    e = parity.exact_evidence(big + 1e-6, big + 2e-6, big)
     assert e["ok"] and e["kernel_max_err"] < e["lane_max_err"]
-    assert not parity.exact_evidence(ref + 1e-5, ref + 2e-6, ref)["ok"]
+    assert not parity.exact_evidence(big + 2e-5, big + 2e-6, big)["ok"]  # ten times the reference's distance
+    assert not parity.exact_evidence(ref + 1e-6, ref + 2e-6, ref)["ok"]  # the contract against the exact value fails
