@@ -164,6 +164,21 @@ enum {
 int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16,
                       int path);
 
+/* w4a16_lin_forward for callers that cannot allocate.  NO COUNTERPART IN THE REFERENCE: it exists for code under HIP graph
+ * capture, tight serving loops and harnesses that forbid hipMalloc.  w4a16_lin_forward's decode launch, when it splits k
+ * across workgroups (the 27B down projection does), parks partial tiles and tickets in a workspace that the context
+ * grows on demand; this entry point runs the same launch with that workspace in a fixed array in the library's own
+ * device image (8 MiB of partial tiles + 64 KiB of tickets per GPU, held until the process ends) and calls no
+ * hipMalloc, hipFree or any other allocating routine.  Decode regime only: t <= 16 (W4A16_ERR_SHAPE beyond), a linear
+ * with a tiled copy.  A launch whose split needs more than the array holds — workgroups x row blocks per wave x 1 KiB x
+ * k slices > w4a16_noalloc_workspace_bytes(), or more than 16384 workgroups per slice — is refused with W4A16_ERR_SHAPE
+ * and a message that gives both sizes.  Same results, bit for bit, as w4a16_lin_forward(..., W4A16_PATH_DECODE) under
+ * the same w4a16_set_decode_* settings.  Every context on a GPU shares that GPU's array: two calls that overlap on
+ * one GPU (two contexts, or one call still running when the next is issued on another stream) race; calls on one
+ * launch stream are ordered and safe. */
+int w4a16_lin_forward_noalloc(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16);
+size_t w4a16_noalloc_workspace_bytes(void);
+
 /* The gate|up projection of a dense FFN with the elementwise kernel that follows it folded in
  * (gemv_multi_dev of the gate/up group + ew_dev_fused, w4a16_dec/chains.rs:271-287, assets/ew.cu:9-32):
  * y[r][c] = f16(silu(g) * u), g = (W x)[r][c], u = (W x)[r][n/2 + c], f32 arithmetic, for a linear whose rows 0..n/2 are

@@ -200,6 +200,7 @@ extern "C" int w4a16_ctx_create(int device_ordinal, const char* asset_dir, w4a16
         while (kAssets[a].syms[nsym]) nsym++;
         rc = w4a16_module_load(ctx, kAssets[a].name, image.data(), image.size(), kAssets[a].syms, nsym);
     }
+    if (!rc) rc = w4_noalloc_init(ctx);
     if (rc) {
         const std::string keep = w4_err_save();
         w4a16_ctx_destroy(ctx);

@@ -90,6 +90,7 @@ struct w4a16_ctx {
     size_t prefill_ws_cap = 0;
     int cu_count = 0;
     const char* last_symbol = "";  // kernel of the most recent launch (a key of `functions`: stable storage)
+    uint64_t fixed_scratch = 0;  // this device's copy of the static scratch array of w4a16_noalloc.hip (device address)
     bool capturing = false;  // between w4a16_capture_begin and w4a16_capture_end: nothing may allocate, free or wait
 };
 
@@ -119,6 +120,10 @@ int w4_register_lin(w4a16_ctx* ctx, const char* name, W4Lin& L);
 int w4_find_lin(w4a16_ctx* ctx, const char* name, W4Lin** out);
 int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes);
 int w4_dense_grouped(w4a16_ctx* ctx, const W4Lin& L, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16);
+int w4_lin_forward_fixed_ws(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16,
+                            uint64_t ws, size_t ws_bytes, uint64_t tickets, size_t ticket_bytes);
+// per-device fixed scratch of the allocation-free entry point (w4a16_noalloc.hip)
+int w4_noalloc_init(w4a16_ctx* ctx);
 
 #define W4_TRY(expr)          \
     do {                      \

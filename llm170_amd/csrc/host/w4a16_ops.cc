@@ -531,6 +531,24 @@ extern "C" int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_de
     }
 }
 
+// Decode-regime lin_forward whose split-K workspace is the fixed per-device buffer of w4a16_noalloc.hip: no allocation
+// on any path (the linear and the kernel are looked up without building a std::string).
+int w4_lin_forward_fixed_ws(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16,
+                            uint64_t ws, size_t ws_bytes, uint64_t tickets, size_t ticket_bytes) {
+    W4Lin* L = nullptr;
+    W4_TRY(w4_find_lin(ctx, name, &L));
+    if (!x_dev || !y_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_noalloc %s: null operand or t=0", name);
+    if (t > 16)
+        return w4_fail(W4A16_ERR_SHAPE, "lin_forward_noalloc %s: t=%zu, the entry point serves the decode regime (1..16 rows)", name, t);
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    DecodeWorkspace W;
+    W.ws = ws;
+    W.ws_cap = ws_bytes;
+    W.tickets = tickets;
+    W.tickets_cap = ticket_bytes;
+    return launch_decode(ctx, *L, x_dev, y_dev, t, out_f16, nullptr, &W);
+}
+
 extern "C" int w4a16_lin_forward_glu(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_f16_dev, size_t t) {
     return w4a16_lin_forward_glu_act(ctx, name, x_dev, y_f16_dev, t, W4A16_ACT_SILU);
 }

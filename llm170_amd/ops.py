@@ -226,6 +226,10 @@ class W4a16Dec:
     def lin_forward(self, name, x_dev, dst_dev, t, out_f16=False, path=PATH_AUTO):
         ffi.check(self.cc.lib.w4a16_lin_forward(self.cc.h, name.encode(), x_dev, dst_dev, t, int(out_f16), path))
 
+    def lin_forward_noalloc(self, name, x_dev, dst_dev, t, out_f16=False):
+        """lin_forward (decode regime) with the split-K workspace in the library's fixed device array: no allocation."""
+        ffi.check(self.cc.lib.w4a16_lin_forward_noalloc(self.cc.h, name.encode(), x_dev, dst_dev, t, int(out_f16)))
+
     def lin_forward_glu(self, name, x_dev, y_f16_dev, t, gelu=False):
         """Fused gate|up projection with the act(gate)*up epilogue (silu, or the tanh form of gelu): y f16 [t][n/2]."""
         if gelu:
