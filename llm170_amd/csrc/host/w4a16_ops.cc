@@ -126,6 +126,11 @@ struct DecodeNorm {
     int act = 0;             // gated projection only: W4A16_ACT_*
 };
 
+// LDS bytes of one wave's staged scales (kernels/decode.hip, AUX_PW)
+static unsigned decode_scale_lds(const W4Lin& L, int rb, int kt_per_wave) {
+    return ((unsigned)(rb * kt_per_wave * (128 / (int)L.group) * 32) + 1023u) / 1024u * 1024u;
+}
+
 static unsigned decode_stats_lds(const DecodeNorm& nm) {
     return nm.stats_in ? (unsigned)std::min<size_t>((nm.n_stats_in + 63) / 64, 8) * 1024u : 0u;
 }
@@ -172,11 +177,12 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     nm.n_stats_out = s_out ? std::min(blocks, (size_t)ceil_div((size_t)stat_rows, (size_t)rb * 16)) : 0;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
                       &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind};
-    // LDS: the split-K partial tiles [waves][rb][1 KiB], then two scale slots per wave; a slot holds the scales of
-    // one ring round (rb x depth x groups-per-tile x 32 bytes, ring never deeper than 8 tiles) rounded up to 512
-    const unsigned slot = ((unsigned)(rb * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
-    // ... then the staging area of the input statistics: 1 KiB per 64 entries, at most 8
-    const unsigned shmem = (unsigned)(waves * rb * 1024) + (unsigned)waves * 2u * slot + decode_stats_lds(nm);
+    // LDS: the split-K partial tiles [waves][rb][1 KiB]; then per wave the scales of its whole k slice (rb x tiles per
+    // wave x groups per tile x 32 bytes, in whole 1 KiB DMA instructions); then the staging area of the input
+    // statistics: 1 KiB per 64 entries, at most 8
+    const unsigned shmem = (unsigned)(waves * rb * 1024) + (unsigned)waves * decode_scale_lds(L, rb, kt_per_wave) + decode_stats_lds(nm);
+    if (shmem > 160u * 1024u)
+        return w4_fail(W4A16_ERR_SHAPE, "decode: k=%zu needs %u bytes of LDS for the staged scales (limit 160 KiB): split k over more workgroups (w4a16_set_decode_ksplit) or waves", L.k, shmem);
     return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);
 }
 
@@ -214,8 +220,7 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
     int act_kind = nm.act;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
                       &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind};
-    const unsigned slot = ((unsigned)(2 * 8 * (128 / L.group) * 32) + 511u) / 512u * 512u;
-    const unsigned shmem = (unsigned)(waves * 2 * 1024) + (unsigned)waves * 2u * slot + decode_stats_lds(nm);
+    const unsigned shmem = (unsigned)(waves * 2 * 1024) + (unsigned)waves * decode_scale_lds(L, 2, kt_per_wave) + decode_stats_lds(nm);
     return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);
 }
 

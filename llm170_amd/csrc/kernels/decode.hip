@@ -16,9 +16,11 @@
 //   * each wave keeps DEPTH k-tiles of loads in flight (register ring, software pipelined);
 //   * scales: a per-row-block scale load per k tile is a vector-memory instruction that moves 32 distinct bytes; with
 //     the x load they cost more address-unit time than the weight stream itself (measured: without them the same
-//     load structure runs 13 % faster).  So ONE 8-byte-per-lane load per ring round fetches the scales of all RB row
-//     blocks x DEPTH k tiles of the next round into a wave-private LDS slot (double buffered, no barrier: LDS
-//     operations of one wave execute in order) and each MFMA group reads its four scales back with ds_read_b64;
+//     load structure runs 13 % faster).  So the scales of a wave's WHOLE k slice (its row blocks x its tiles x groups
+//     x 16 rows, contiguous per row block in the tiled scale array) are staged once, ahead of the first weight load,
+//     into a wave-private LDS area by LDS DMA (buffer_load ... lds: no registers, no ds_write) and each MFMA group reads
+//     its four scales back with ds_read_b64.  (One 8-byte load per ring round into a double-buffered slot was 0.2-0.8 us
+//     per launch slower on the 27B shapes: the small loads sit on every round's critical path.)
 //   * split-K lives inside the workgroup: the W waves of a block take consecutive k-tile slices of the same RB row
 //     blocks and wave 0 folds the partial tiles through LDS in fixed order (deterministic, no atomics, no second
 //     launch).  The host picks RB and W;
@@ -61,11 +63,8 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                             const float* __restrict__ stats_in, int n_stats_in, float inv_cols_in,
                                             float* __restrict__ stats_out, int stat_rows, float* __restrict__ resid,
                                             const float* __restrict__ nw, int act_kind) {
-    extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K, then [W][2][AUXB] scale slots
+    extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K, then the waves' staged scales
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
-    constexpr int AUXB = RB * DEPTH * GPT * 32;      // bytes of scales one ring round needs: [rb][tile][group][16 rows]
-    constexpr int AUXN = (AUXB + 511) / 512;         // 8-byte-per-lane loads that fetch them
-    constexpr int SLOT = AUXN * 512;                 // LDS bytes of one slot: every lane of every load has a place
     constexpr int C = 4 / XL;           // 32-k chunks (MFMAs) served by one x load
     constexpr int TPL = 16 / C;         // token columns served by one x load
     // The launch geometry (W waves per block, nks k slices over blockIdx.y, tiles per slice and per wave) arrives as
@@ -99,28 +98,25 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
         const unsigned nb = (unsigned)row_block(rb);  // a tail block re-reads the last row block
         qoff[rb] = nb * (unsigned)kt_n * 1024u + (unsigned)lane * 16u;
     }
-    // scale fetch: byte o = lane*8 + a*512 of the round's slot belongs to row block o / (DEPTH*GPT*32); the rest of o
-    // is the offset inside that row block's run of DEPTH tiles, contiguous in the tiled scale array as well
-    char* const aux_lds = reinterpret_cast<char*>(red) + W * RB * 1024 + wave * (2 * SLOT);
-    unsigned aoff[AUXN];
-#pragma unroll
-    for (int a = 0; a < AUXN; a++) {
-        const int o = lane * 8 + a * 512;
-        const int rb = o / (DEPTH * GPT * 32), rem = o % (DEPTH * GPT * 32);
-        const unsigned nb = (unsigned)row_block(rb);
-        aoff[a] = o < AUXB ? nb * (unsigned)kg_n * 32u + (unsigned)rem : W4_OOB;
+    // Scales of the wave's k slice, staged once: the wave's LDS area holds [row block][tile of the slice][group][16 rows],
+    // aux_rb_bytes per row block (the stride is that of a full slice, so a shorter last slice leaves a gap); byte
+    // o = lane*16 + a*1024 is fetched by lane `lane` of DMA instruction a (a lane past the slice fetches out of range:
+    // zeros, no traffic).  AUX_PW bytes per wave, whole DMA instructions.
+    const int aux_rb_bytes = kt_per_wave * (GPT * 32);
+    const int AUX_PW = (RB * aux_rb_bytes + 1023) & ~1023;
+    char* const aux_lds = reinterpret_cast<char*>(red) + W * RB * 1024 + wave * AUX_PW;
+    {
+        const __amdgpu_buffer_rsrc_t sr_ = w4_make_rsrc(st, s_bytes);
+        const int slice_bytes = (kt1 - kt0) * (GPT * 32);
+        for (int a = 0; a * 1024 < RB * aux_rb_bytes; a++) {
+            const int o = lane * 16 + a * 1024;
+            const int rb = o / aux_rb_bytes, rem = o - rb * aux_rb_bytes;
+            const unsigned nb = (unsigned)row_block(min(rb, RB - 1));
+            const unsigned off = (rb < RB && rem < slice_bytes) ? nb * (unsigned)kg_n * 32u + (unsigned)(kt0 * (GPT * 32) + rem) : W4_OOB;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(sr_, (__attribute__((address_space(3))) void*)(aux_lds + a * 1024), 16, off, 0,
+                                                     0, 0);
+        }
     }
-    u2_t aux[AUXN];
-    auto load_aux = [&](int kt) {  // scales of tiles kt .. kt+DEPTH-1 (a run past the wave's slice is never used)
-        const __amdgpu_buffer_rsrc_t sr_ = w4_make_rsrc(st, kt < kt1 ? s_bytes : 0u);
-#pragma unroll
-        for (int a = 0; a < AUXN; a++) aux[a] = __builtin_amdgcn_raw_buffer_load_b64(sr_, aoff[a], kt * (GPT * 32), 0);
-    };
-    auto store_aux = [&](int buf) {  // all lanes store (lanes past AUXB hold zeros): no divergence, nothing for the
-                                     // compiler to sink the loads into
-#pragma unroll
-        for (int a = 0; a < AUXN; a++) *reinterpret_cast<u2_t*>(aux_lds + buf * SLOT + lane * 8 + a * 512) = aux[a];
-    };
 
     // Per-tile addressing costs no vector ALU work: the lane part of every offset is loop invariant, the k-tile part
     // travels in the scalar offset operand, and a tile past the wave's range is switched off by a zero-length
@@ -137,8 +133,8 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
         for (int l = 0; l < XL; l++)
             s_.x[l] = __builtin_amdgcn_raw_buffer_load_b128(xr_, xoff + (unsigned)(l * C * 32) * 2u, kt * (W4_TILE_K * 2), 0);
     };
-    // sc = this lane's view of the round's scale slot: rows 4g..4g+3 of (row block rb, tile d, group gi) are the 8
-    // bytes at sc + ((rb*DEPTH + d)*GPT + gi)*32
+    // sc = this lane's view of the scales of the round's first tile: rows 4g..4g+3 of (row block rb, tile d of the round,
+    // group gi) are the 8 bytes at sc + rb*aux_rb_bytes + (d*GPT + gi)*32
     auto compute = [&](const DecodeStage<RB, XL>& s_, const char* sc, int d) {
         // B operand of MFMA w = chunk w of x for token column m: held by lane (m + (w % C) * TPL) of load w / C
         u4_t xb[4];
@@ -159,7 +155,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                 for (int w = 0; w < 4; w++)
                     part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
                                                                   __builtin_bit_cast(h8_t, xb[w]), part, 0, 0, 0);
-                const u2_t sv = *reinterpret_cast<const u2_t*>(sc + (rb * DEPTH + d) * GPT * 32);
+                const u2_t sv = *reinterpret_cast<const u2_t*>(sc + rb * aux_rb_bytes + d * GPT * 32);
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     acc[rb][i] = __builtin_fmaf(w4_scale_fast<SBF>((sv[i >> 1] >> (16 * (i & 1))) & 0xFFFFu), part[i], acc[rb][i]);
@@ -169,7 +165,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                     f4_t part = {0.f, 0.f, 0.f, 0.f};
                     part = __builtin_amdgcn_mfma_f32_16x16x32_f16(w4_deq8(s_.q[rb][w]),
                                                                   __builtin_bit_cast(h8_t, xb[w]), part, 0, 0, 0);
-                    const u2_t sv = *reinterpret_cast<const u2_t*>(sc + ((rb * DEPTH + d) * GPT + w % GPT) * 32);
+                    const u2_t sv = *reinterpret_cast<const u2_t*>(sc + rb * aux_rb_bytes + (d * GPT + w % GPT) * 32);
 #pragma unroll
                     for (int i = 0; i < 4; i++)
                         acc[rb][i] = __builtin_fmaf(w4_scale_fast<SBF>((sv[i >> 1] >> (16 * (i & 1))) & 0xFFFFu), part[i], acc[rb][i]);
@@ -187,7 +183,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     // in-block reduction never writes.  The epilogue multiplies the sums by it.  Further token quads and entries
     // beyond the staging area (8 x 64) repeat the fetch inside input_scale.
     typedef __attribute__((address_space(3))) char lds_char_t;
-    lds_char_t* const stage_lds = (lds_char_t*)(reinterpret_cast<char*>(red) + W * RB * 1024 + W * (2 * SLOT));
+    lds_char_t* const stage_lds = (lds_char_t*)(reinterpret_cast<char*>(red) + W * RB * 1024 + W * AUX_PW);
     const int stat_chunks = min((n_stats_in + 63) >> 6, 8);
     auto fetch_stats = [&](int c0, int qd) {
         const __amdgpu_buffer_rsrc_t sr_in = w4_make_rsrc(stats_in, (unsigned)n_stats_in * 64u);
@@ -197,7 +193,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     };
     if (stats_in != nullptr && wave == 0) fetch_stats(0, 0);
     auto input_scale = [&]() {
-        const f4_t* const staged = reinterpret_cast<const f4_t*>(reinterpret_cast<char*>(red) + W * RB * 1024 + W * (2 * SLOT));
+        const f4_t* const staged = reinterpret_cast<const f4_t*>(reinterpret_cast<char*>(red) + W * RB * 1024 + W * AUX_PW);
         float mine = 0.f;
         for (int qd = 0; qd * 4 < t; qd++) {  // a quad of token columns at a time
             f4_t sum = {0.f, 0.f, 0.f, 0.f};
@@ -206,8 +202,8 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                     fetch_stats(c0, qd);
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 } else {
-                    // the first fetch is older than the fill's loads (scales, then DEPTH stages): wait for it alone
-                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AUXN + DEPTH * (RB + XL) < 63 ? AUXN + DEPTH * (RB + XL) : 63) : "memory");
+                    // the first fetch is older than the ring fill's loads (DEPTH stages): wait for it alone
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DEPTH * (RB + XL) < 63 ? DEPTH * (RB + XL) : 63) : "memory");
                 }
                 for (int c = 0; c < stat_chunks; c++) sum += staged[c * 64 + lane];
             }
@@ -230,12 +226,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     const int rounds = tiles / DEPTH;
     const char* const sc0 = aux_lds + g * 8;
     for (int r = -1; r < rounds; r++) {
-        // scales of round r+1 travel with this round's ring loads and are parked in LDS slot (r+1)&1 once this
-        // round's computes (which read slot r&1) are issued; they are older than every ring load issued below, so
-        // waiting for them leaves the whole ring in flight
-        load_aux(kt0 + (r + 1) * DEPTH);
-        __builtin_amdgcn_sched_barrier(0);
-        const char* sc = sc0 + (r & 1) * SLOT;
+        const char* sc = sc0 + r * (DEPTH * GPT * 32);  // the staged scales are older than every ring load: no wait of their own
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
             if (r >= 0) compute(stage[d], sc, d);
@@ -243,12 +234,10 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
             load(stage[d], kt0 + (r + 1) * DEPTH + d);
             __builtin_amdgcn_sched_barrier(0);
         }
-        store_aux((r + 1) & 1);
-        __builtin_amdgcn_sched_barrier(0);
         if (r == -1 && stats_in != nullptr && wave == 0) input_scale();  // behind the first ring loads, once
     }
     {
-        const char* sc = sc0 + (rounds & 1) * SLOT;
+        const char* sc = sc0 + rounds * (DEPTH * GPT * 32);
 #pragma unroll
         for (int d = 0; d < DEPTH - 1; d++)
             if (rounds * DEPTH + d < tiles) compute(stage[d], sc, d);
