@@ -176,11 +176,11 @@ def bench_moe(dec, gen, ops, args):
 def bench_chain(dec, gen, ops, args):
     """64 dense decoder layers of linears at M = 4 (QKV 5120->7168, O 5120->5120, gate+up 5120->34816, down
     17408->5120, group 128) with the RMS-rescale / SiLU*up glue, independent device-generated weights (10.9 GB).
-    What is reported is w4a16_chain_forward (seven launches per layer: every activation is normalised in f32 before it
-    is rounded to f16), eager and as graph replays; its output is checked finite, of unit mean square and equal
-    between the two.  The statement with the normalisations deferred across the linears (four launches per layer)
-    carries the un-normalised down-projection output in f16 and overflows on these synthetic weights from the third
-    layer on, so it is timed on the side and flagged, never reported as this configuration's figure."""
+    Two statements of the same chain are timed, eager and as graph replays: w4a16_chain_forward (seven launches per
+    layer: every activation is normalised in f32 by a launch of its own before it is rounded to f16) and
+    w4a16_chain_forward_fused (four launches per layer: the normalisations deferred across the linears, hand-overs with
+    power-of-two factors).  A variant counts only if its output is finite, of unit mean square and the same bits from
+    graph replays as from eager passes; the configuration's figure is the faster valid one."""
     cc = dec.cc
     layers, hidden, n_qkv, n_ff, g, t = 64, 5120, 7168, 17408, 128, 4
     dec.upload_chain_synth("c4", layers, hidden, n_qkv, n_ff, g)
@@ -188,33 +188,38 @@ def bench_chain(dec, gen, ops, args):
               "ffn_down": (hidden, n_ff)}
     for l in range(layers):
         for role in ops.W4a16Dec.CHAIN_ROLES:
+            dec.row_norm_max("c4.%d.%s" % (l, role))  # needs nothing but the tiled copy; kept with the linear
             dec.drop_raw("c4.%d.%s" % (l, role))
     px, py = cc.to_device(gen.normal_f16(404, (t, hidden))), cc.alloc(t * hidden * 2)
     reps = max(3, args.steps // 80)
-
-    def timed(use_graph, fused):
-        return [dec.bench_chain("c4", layers, px, t, py, reps, warmup=1, use_graph=use_graph, fused=fused)[0] / reps
-                for _ in range(ROUNDS)]
-
-    def output():
-        return cc.d2h(py, (t, hidden), np.uint16)
-
-    eager = timed(False, False)
-    y_eager = output()
-    v = gen.f16_bits_to_f32(y_eager).astype(np.float64)
-    finite = bool(np.all(np.isfinite(v)))
-    unit_ms = bool(finite and np.allclose(np.mean(v * v, axis=1), 1.0, atol=2e-3))
-    if args.no_graph:  # eager passes only (a tracer that cannot follow graph replays)
-        graph, same = eager, None
-    else:
-        graph = timed(True, False)
-        same = bool(np.array_equal(output(), y_eager))
-    if not finite or not unit_ms or same is False:
-        raise RuntimeError("chain: output finite %r, unit mean square %r, graph == eager %r" % (finite, unit_ms, same))
-    fused = timed(False, True)
-    fused_finite = bool(np.all(np.isfinite(gen.f16_bits_to_f32(output()))))
     total = sum(algorithmic_bytes(t, kk, nn, g) for (nn, kk) in shapes.values()) * layers
-    best = min(sorted(eager)[ROUNDS // 2], sorted(graph)[ROUNDS // 2])
+
+    def variant(fused):
+        def timed(use_graph):
+            return [dec.bench_chain("c4", layers, px, t, py, reps, warmup=1, use_graph=use_graph, fused=fused)[0] / reps
+                    for _ in range(ROUNDS)]
+        eager = timed(False)
+        y_eager = cc.d2h(py, (t, hidden), np.uint16)
+        v = gen.f16_bits_to_f32(y_eager).astype(np.float64)
+        finite = bool(np.all(np.isfinite(v)))
+        unit_ms = bool(finite and np.allclose(np.mean(v * v, axis=1), 1.0, atol=2e-3))
+        if args.no_graph:  # eager passes only (a tracer that cannot follow graph replays)
+            graph, same = eager, None
+        else:
+            graph = timed(True)
+            same = bool(np.array_equal(cc.d2h(py, (t, hidden), np.uint16), y_eager))
+        best = min(sorted(eager)[ROUNDS // 2], sorted(graph)[ROUNDS // 2])
+        return {"launches_per_layer": 4 if fused else 7, "ms_per_pass_eager": spread(eager, 1.0, 4),
+                "ms_per_pass_graph": spread(graph, 1.0, 4), "ms_per_pass": round(best, 4),
+                "output_finite": finite, "output_unit_mean_square": unit_ms, "graph_equals_eager_bits": same,
+                "valid": bool(finite and unit_ms and same is not False)}
+
+    kept, deferred = variant(False), variant(True)
+    valid = [v for v in (kept, deferred) if v["valid"]]
+    if not valid:
+        raise RuntimeError("chain: no valid variant: %r / %r" % (kept, deferred))
+    fig = min(valid, key=lambda v: v["ms_per_pass"])
+    best = fig["ms_per_pass"]
     per_gemm = []
     xw, yw = cc.alloc(t * n_ff * 2), cc.alloc(t * 2 * n_ff * 4)
     cc.memset0(xw, t * n_ff * 2)
@@ -227,16 +232,10 @@ def bench_chain(dec, gen, ops, args):
                          "GBps": round(b / (ms * 1e-3) / 1e9, 1)})
     for p_ in (px, py, xw, yw):
         cc.free(p_)
-    return {"layers": layers, "M": t, "launches_per_layer": 7, "ms_per_pass_eager": spread(eager, 1.0, 4),
-            "ms_per_pass_graph": spread(graph, 1.0, 4), "us_per_token": round(best * 1e3 / t, 2),
-            "GBps_end_to_end": round(total / (best * 1e-3) / 1e9, 1),
+    return {"layers": layers, "M": t, "launches_per_layer": fig["launches_per_layer"], "ms_per_pass": best,
+            "us_per_token": round(best * 1e3 / t, 2), "GBps_end_to_end": round(total / (best * 1e-3) / 1e9, 1),
             "hbm_frac_end_to_end": round(total / (best * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-            "output_finite": finite, "output_unit_mean_square": unit_ms, "graph_equals_eager_bits": same,
-            "deferred_normalisation_variant": {
-                "launches_per_layer": 4, "ms_per_pass_eager": spread(fused, 1.0, 4), "output_finite": fused_finite,
-                "note": "not this configuration's figure: its f16 hand-over of the un-normalised down projection "
-                        "leaves the f16 range on these synthetic weights"},
-            "per_gemm": per_gemm}
+            "normalisation_launches_kept": kept, "normalisations_deferred": deferred, "per_gemm": per_gemm}
 
 
 def main():

@@ -213,7 +213,8 @@ int w4a16_lin_forward_glu_act(w4a16_ctx* ctx, const char* name, uint64_t x_dev, 
  * element of v (of v * nw with a norm weight) must lie inside the f16 range: beyond 65504 it becomes Inf (and the
  * consumer's output NaN) where norm_resid, which normalises in f32 first, stays finite; rows whose elements fall below
  * 6e-5 lose relative precision to f16 subnormals.  Nothing is detected at run time.  Residual streams of trained
- * models sit well inside; the synthetic 64-layer chain of random projections does not (see w4a16_chain_forward_fused). */
+ * models sit well inside; the synthetic 64-layer chain of random projections does not: the _scaled forms below lift the
+ * precondition. */
 int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
                                     uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_dev,
                                     int out_f16, uint64_t stats_out_dev, size_t stat_rows, size_t* n_stats_out,
@@ -223,6 +224,25 @@ int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x
 int w4a16_lin_forward_glu_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
                                         uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_f16_dev,
                                         int act);
+/* Both with a power-of-two factor on each hand-over, which lifts the range precondition above when the exponents come
+ * from a bound on the values: x_dev holds the true activations times 2^-in_exp and y_dev receives the true output
+ * times 2^-out_exp (for the gated form: the true silu(g)*u times 2^-out_exp).  The statistics, the residual stream and
+ * the norm weight see true values.  Both factors are exact in f32, so wherever the un-scaled hand-over stays inside
+ * the normal f16 range the results are the same numbers.  Exponents in -120..120; 0, 0 is the un-scaled call.
+ * A bound for the output of a linear fed rows of unit root mean square: w4a16_lin_row_norm_max(W) * sqrt(k)
+ * (norm_resid of the reference hands over normalised values and needs none of this, assets/norm.cu:4-48). */
+int w4a16_lin_forward_deferred_norm_scaled(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
+                                           uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, int in_exp,
+                                           uint64_t y_dev, int out_f16, int out_exp, uint64_t stats_out_dev,
+                                           size_t stat_rows, size_t* n_stats_out, uint64_t resid_dev, uint64_t nw_dev);
+int w4a16_lin_forward_glu_deferred_norm_scaled(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
+                                               uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, int in_exp,
+                                               uint64_t y_f16_dev, int out_exp, int act);
+/* max over rows r of sqrt(sum_c ((nibble - 8) * scale)^2) of a registered linear's dequantised weights (the values of
+ * dequant_row_w4a16_split, crates/core/src/matmul/cpu.rs:167-194), f32 arithmetic on the device.  By Cauchy-Schwarz no
+ * element of W x exceeds it times the Euclidean norm of x.  Computed on the first request (a launch and a 4-byte
+ * read-back, so not while capturing) and kept with the linear.  Needs the tiled copy (k % 128 == 0). */
+int w4a16_lin_row_norm_max(w4a16_ctx* ctx, const char* name, float* out);
 
 /* gemv_host (w4a16_dec/mod.rs, host-operand convenience used by probes): lin_forward with host x / y. */
 int w4a16_lin_forward_host(w4a16_ctx* ctx, const char* name, const uint16_t* x_f16, void* y, size_t t, int out_f16,
@@ -379,11 +399,14 @@ int w4a16_chain_forward(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_
  *     gu = r(v2) * ffn_gate_up(b)            c = silu_mul_f16(gu)
  *     v4 = ffn_down(c)                       x[l+1] = f16(v4), s[l+1] = r(v4)
  * and y = rms_f16(v4) after the last layer: the function of w4a16_chain_forward with the factors applied after the
- * linears instead of before the roundings to f16 (results agree to those roundings) — as long as v4, which crosses
- * the layer boundary as f16 without its factor, stays inside the f16 range (the precondition of
- * w4a16_lin_forward_deferred_norm).  With random weights of mean -0.5 and no residual stream the rows of v4 drift
- * apart by orders of magnitude within three layers (rows aligned with the weights' mean direction switch the gated
- * unit fully on or off), so deep synthetic chains must use w4a16_chain_forward. */
+ * linears instead of before the roundings to f16 (results agree to those roundings).  a, b, c and x[l+1] cross from
+ * launch to launch without their 1/rms factor; each crossing carries a power-of-two factor 2^-e
+ * (w4a16_lin_forward_deferred_norm_scaled) with e the smallest exponent that brings a bound on the values under 32768:
+ * row_norm_max(W) * sqrt(k) for a linear fed unit-rms rows, the square of that for the gated product, and for the down
+ * projection row_norm_max * sqrt(n_ff) * the bound of c.  So nothing leaves the f16 range whatever the weights (random
+ * weights of mean -0.5 with no residual stream push v4 beyond 65504 within three layers), and wherever the un-scaled
+ * values stay in range the result is the same.  The first call on a set of linears computes their row norms (a small
+ * launch and read-back each): call it once before capturing it in a graph. */
 int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers, uint64_t x_dev,
                               size_t t, uint64_t y_dev);
 /* ensure_graph (w4a16_dec/graphs.rs:41-134): one decode step of the chain as a replayable graph.  Runs the chain once

@@ -134,8 +134,21 @@ extern "C" int w4a16_chain_forward(w4a16_ctx* ctx, const char* prefix, size_t la
     return 0;
 }
 
+// Smallest e >= 0 with bound * 2^-e <= 32768 (half the f16 range), for a bound on the magnitude of what is handed over.
+static int handover_exp(double bound) {
+    int e = 0;
+    while (e < 120 && std::ldexp(bound, -e) > 32768.0) e++;
+    return e;
+}
+
 // The same chain with the three normalisations inside a layer deferred across the linears that follow them
-// (w4a16_lin_forward_deferred_norm): four launches per layer instead of seven.
+// (w4a16_lin_forward_deferred_norm_scaled): four launches per layer instead of seven.  The activations cross from launch
+// to launch as f16 WITHOUT their 1/rms factor, so each hand-over carries a power-of-two factor that keeps it inside
+// the f16 range whatever the input: a linear fed rows of unit root mean square over k columns gives no element above
+// (largest row norm of W) x sqrt(k) (Cauchy-Schwarz; w4a16_lin_row_norm_max), the gated product none above the square
+// of that, and the down projection none above its own row-norm bound times sqrt(n_ff) times the bound of its input.
+// The producer multiplies by 2^-e before rounding to f16 and the consumer by 2^e after its MFMA sums, both exact, so the
+// values are those of the un-scaled statement wherever that one stays in range.
 extern "C" int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers,
                                          uint64_t x_dev, size_t t, uint64_t y_dev) {
     if (!ctx || !prefix || !x_dev || !y_dev) return w4_fail(W4A16_ERR_ARG, "chain_forward_fused: null argument");
@@ -144,6 +157,7 @@ extern "C" int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, siz
     W4ChainScratch& S = ctx->chain;
     uint64_t cur = x_dev;
     size_t n_prev = 0;  // partial sums the previous layer's down projection left in S.stats[2]
+    int e_prev = 0;     // and the exponent of its hand-over
     for (size_t l = layer0; l < layer0 + n_layers; l++) {
         char nm[4][160];
         const char* role[4] = {"attn_qkv", "attn_output", "ffn_gate_up", "ffn_down"};
@@ -166,20 +180,30 @@ extern "C" int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, siz
             W4_TRY(w4_ensure(ctx, &S.stats[i], &S.stats_cap[i], ((std::max(n_qkv, hidden) + 15) / 16) * 64));
         const bool last = l + 1 == layer0 + n_layers;
         size_t n_a = 0, n_b = 0, n_d = 0;
-        // a = qkv(x)[:, :hidden], its statistics over those columns only
-        W4_TRY(w4a16_lin_forward_deferred_norm(ctx, nm[0], cur, 0, t, n_prev ? S.stats[2] : 0, n_prev, hidden, S.a16, 1,
-                                               S.stats[0], hidden, &n_a, 0, 0));
-        W4_TRY(w4a16_lin_forward_deferred_norm(ctx, nm[1], S.a16, n_qkv, t, S.stats[0], n_a, hidden, S.h16a, 1, S.stats[1],
-                                               hidden, &n_b, 0, 0));
-        W4_TRY(w4a16_lin_forward_glu_deferred_norm(ctx, nm[2], S.h16a, 0, t, S.stats[1], n_b, hidden, S.h16b, W4A16_ACT_SILU));
+        float rn[4];
+        for (int i = 0; i < 4; i++) W4_TRY(w4a16_lin_row_norm_max(ctx, nm[i], &rn[i]));
+        const double b_qkv = (double)rn[0] * std::sqrt((double)hidden), b_o = (double)rn[1] * std::sqrt((double)hidden),
+                     b_gu = (double)rn[2] * std::sqrt((double)hidden), b_act = b_gu * b_gu,
+                     b_down = (double)rn[3] * std::sqrt((double)n_ff) * b_act;
+        const int e_a = handover_exp(b_qkv), e_b = handover_exp(b_o), e_c = handover_exp(b_act), e_d = handover_exp(b_down);
+        // a = qkv(x)[:, :hidden], its statistics over those columns only.  The chain's own input is taken as given
+        // (e_prev = 0); the previous layer's down projection handed over 2^-e_prev times its output
+        W4_TRY(w4a16_lin_forward_deferred_norm_scaled(ctx, nm[0], cur, 0, t, n_prev ? S.stats[2] : 0, n_prev, hidden, e_prev,
+                                                      S.a16, 1, e_a, S.stats[0], hidden, &n_a, 0, 0));
+        W4_TRY(w4a16_lin_forward_deferred_norm_scaled(ctx, nm[1], S.a16, n_qkv, t, S.stats[0], n_a, hidden, e_a, S.h16a, 1,
+                                                      e_b, S.stats[1], hidden, &n_b, 0, 0));
+        W4_TRY(w4a16_lin_forward_glu_deferred_norm_scaled(ctx, nm[2], S.h16a, 0, t, S.stats[1], n_b, hidden, e_b, S.h16b, e_c,
+                                                          W4A16_ACT_SILU));
         if (last) {
             // the chain's output is normalised: one launch per call, not per layer
-            W4_TRY(w4a16_lin_forward(ctx, nm[3], S.h16b, S.y32, t, 0, W4A16_PATH_DECODE));
+            W4_TRY(w4a16_lin_forward_deferred_norm_scaled(ctx, nm[3], S.h16b, 0, t, 0, 0, 0, e_c, S.y32, 0, 0, 0, 0, nullptr, 0, 0));
             W4_TRY(w4a16_rms_rescale_f16(ctx, S.y32, hidden, hidden, t, y_dev));
         } else {
-            W4_TRY(w4a16_lin_forward_deferred_norm(ctx, nm[3], S.h16b, 0, t, 0, 0, 0, S.ping[0], 1, S.stats[2], hidden, &n_d, 0, 0));
+            W4_TRY(w4a16_lin_forward_deferred_norm_scaled(ctx, nm[3], S.h16b, 0, t, 0, 0, 0, e_c, S.ping[0], 1, e_d, S.stats[2],
+                                                          hidden, &n_d, 0, 0));
             cur = S.ping[0];
             n_prev = n_d;
+            e_prev = e_d;
         }
     }
     return 0;

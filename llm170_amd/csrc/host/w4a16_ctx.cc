@@ -44,7 +44,8 @@ static const char* const kLaneSyms[] = {"w4a16_lane_g128_f16", "w4a16_lane_g128_
                                         "w4a16_lane_g32_bf16", nullptr};
 static const char* const kLayoutSyms[] = {"w4a16_tile_q",         "w4a16_tile_s",          "w4a16_untile_q",
                                           "w4a16_untile_s",       "w4a16_dump_tiled_f16",  "w4a16_dump_tiled_bf16",
-                                          "w4a16_dump_raw_f16",   "w4a16_dump_raw_bf16",   nullptr};
+                                          "w4a16_dump_raw_f16",   "w4a16_dump_raw_bf16",   "w4a16_row_norm_max_f16",
+                                          "w4a16_row_norm_max_bf16", nullptr};
 static const char* const kDecodeSyms[] = {
     "w4a16_decode_g128_f16_rb1_x1", "w4a16_decode_g128_f16_rb1_x2", "w4a16_decode_g128_f16_rb1_x4",
     "w4a16_decode_g128_f16_rb2_x1", "w4a16_decode_g128_f16_rb2_x2", "w4a16_decode_g128_f16_rb2_x4",

@@ -22,6 +22,7 @@ struct W4Lin {
     int scale_bf16 = 0;
     size_t row_blocks = 0;
     bool scales_regular = true;  // every scale finite and non-zero (the MFMA prefill kernel divides by them)
+    float row_norm_max = -1.0f;  // largest row norm of the dequantised weights, computed on first request (< 0: not yet)
 };
 
 // The experts of one MoE layer: two arenas in the tiled layout, experts at a fixed stride
@@ -81,6 +82,8 @@ struct w4a16_ctx {
     int moe_block = 0, moe_waves = 0;  // 0 = automatic
     int moe_act_kind = 0;              // activation of the expert FFN call in progress (W4A16_ACT_*)
     int decode_rows_per_wave = 0, decode_waves_per_block = 0;  // 0 = automatic
+    uint64_t norm_word = 0;  // one device word for w4a16_lin_row_norm_max
+    size_t norm_word_cap = 0;
     int decode_ksplit = 0;                                      // 0 = automatic, -1 = never, n = exactly n k slices
     uint64_t decode_ws = 0, decode_tickets = 0;                 // partial tiles and per-block tickets of a split launch
     size_t decode_ws_cap = 0, decode_tickets_cap = 0;

@@ -4,6 +4,7 @@
 // kernels/gemv.rs:112-187, kernels/gemm.rs:4-51).
 #include <algorithm>
 #include <chrono>
+#include <cmath>
 #include <cstring>
 
 #include "w4a16_internal.h"
@@ -124,6 +125,7 @@ struct DecodeNorm {
     uint64_t resid = 0;      // f32 [t][n] residual stream, takes the output: v = resid + y, written back
     uint64_t nw = 0;         // f32 [n] norm weight of the output rows, multiplies what y_dev receives
     int act = 0;             // gated projection only: W4A16_ACT_*
+    int in_exp = 0, out_exp = 0;  // x holds its true value times 2^-in_exp, y receives its true value times 2^-out_exp
 };
 
 // LDS bytes of one wave's staged scales (kernels/decode.hip, AUX_PW)
@@ -142,6 +144,8 @@ static int check_decode_norm(const W4Lin& L, size_t t, const DecodeNorm& nm) {
     if (nm.stats_in && (nm.n_stats_in == 0 || nm.n_stats_in > 0x7fffffffu / 16 || nm.in_cols == 0))
         return w4_fail(W4A16_ERR_ARG, "decode: input statistics need n_stats_in and in_cols (got %zu, %zu)", nm.n_stats_in, nm.in_cols);
     if (nm.stats_out && nm.stat_rows == 0) return w4_fail(W4A16_ERR_ARG, "decode: output statistics over zero rows");
+    if (nm.in_exp < -120 || nm.in_exp > 120 || nm.out_exp < -120 || nm.out_exp > 120)
+        return w4_fail(W4A16_ERR_ARG, "decode: hand-over exponents %d, %d outside -120..120", nm.in_exp, nm.out_exp);
     return 0;
 }
 
@@ -174,9 +178,10 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     float inv_cols = nm.in_cols ? 1.0f / (float)nm.in_cols : 0.0f;
     uint64_t s_in = nm.stats_in, s_out = nm.stats_out, resid = nm.resid, nw = nm.nw;
     int act_kind = 0;  // no activation in the plain linear
+    float in_scale = std::ldexp(1.0f, nm.in_exp), out_scale = std::ldexp(1.0f, -nm.out_exp);
     nm.n_stats_out = s_out ? std::min(blocks, (size_t)ceil_div((size_t)stat_rows, (size_t)rb * 16)) : 0;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
-                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind};
+                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind, &in_scale, &out_scale};
     // LDS: the split-K partial tiles [waves][rb][1 KiB]; then per wave the scales of its whole k slice (rb x tiles per
     // wave x groups per tile x 32 bytes, in whole 1 KiB DMA instructions); then the staging area of the input
     // statistics: 1 KiB per 64 entries, at most 8
@@ -218,8 +223,9 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
     if (nm.act != W4A16_ACT_SILU && nm.act != W4A16_ACT_GELU_TANH)
         return w4_fail(W4A16_ERR_ARG, "decode glu: activation %d (0 = silu, 1 = gelu, tanh form)", nm.act);
     int act_kind = nm.act;
+    float in_scale = std::ldexp(1.0f, nm.in_exp), out_scale = std::ldexp(1.0f, -nm.out_exp);
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
-                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind};
+                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind, &in_scale, &out_scale};
     const unsigned shmem = (unsigned)(waves * 2 * 1024) + (unsigned)waves * decode_scale_lds(L, 2, kt_per_wave) + decode_stats_lds(nm);
     return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);
 }
@@ -569,10 +575,45 @@ extern "C" int w4a16_lin_forward_glu_act(w4a16_ctx* ctx, const char* name, uint6
     return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t, &nm);
 }
 
+// Largest row norm of the dequantised weights (kernels/layout.hip, w4a16_row_norm_max_*), computed on the first request
+// and kept with the linear.  The one device word it is reduced into belongs to the context.
+extern "C" int w4a16_lin_row_norm_max(w4a16_ctx* ctx, const char* name, float* out) {
+    W4Lin* L = nullptr;
+    W4_TRY(w4_find_lin(ctx, name, &L));
+    if (!out) return w4_fail(W4A16_ERR_ARG, "lin_row_norm_max %s: null output", name);
+    if (L->row_norm_max < 0.0f) {
+        if (!L->q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "lin_row_norm_max %s: linear has no tiled copy (needs k %% 128 == 0)", name);
+        if (ctx->capturing)
+            return w4_fail(W4A16_ERR_ARG, "lin_row_norm_max %s: first request while the launch stream is capturing (it reads a word back): ask once before the capture", name);
+        W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+        W4_TRY(w4_ensure(ctx, &ctx->norm_word, &ctx->norm_word_cap, 256));
+        W4_TRY(w4a16_memset0(ctx, ctx->norm_word, 256));
+        int rbi = (int)L->row_blocks, kt_n = (int)(L->k / 128), gi = (int)L->group;
+        void* p[] = {&L->q_tiled, &L->s_tiled, &ctx->norm_word, &rbi, &kt_n, &gi};
+        W4_TRY(w4_launch(ctx, L->scale_bf16 ? "w4a16_row_norm_max_bf16" : "w4a16_row_norm_max_f16",
+                         ceil_div(L->row_blocks, 4), 1, 256, 0, p));
+        float v = 0.0f;
+        W4_TRY(w4a16_d2h(ctx, &v, ctx->norm_word, 4));
+        if (!std::isfinite(v)) return w4_fail(W4A16_ERR_UNSUPPORTED, "lin_row_norm_max %s: a scale is not finite", name);
+        L->row_norm_max = v;
+    }
+    *out = L->row_norm_max;
+    return 0;
+}
+
 extern "C" int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
                                                uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_dev,
                                                int out_f16, uint64_t stats_out_dev, size_t stat_rows,
                                                size_t* n_stats_out, uint64_t resid_dev, uint64_t nw_dev) {
+    return w4a16_lin_forward_deferred_norm_scaled(ctx, name, x_dev, ldx, t, stats_in_dev, n_stats_in, in_cols, 0, y_dev,
+                                                  out_f16, 0, stats_out_dev, stat_rows, n_stats_out, resid_dev, nw_dev);
+}
+
+extern "C" int w4a16_lin_forward_deferred_norm_scaled(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx,
+                                                      size_t t, uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols,
+                                                      int in_exp, uint64_t y_dev, int out_f16, int out_exp,
+                                                      uint64_t stats_out_dev, size_t stat_rows, size_t* n_stats_out,
+                                                      uint64_t resid_dev, uint64_t nw_dev) {
     W4Lin* L = nullptr;
     W4_TRY(w4_find_lin(ctx, name, &L));
     if (!x_dev || !y_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_deferred_norm %s: null operand or t=0", name);
@@ -587,6 +628,8 @@ extern "C" int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name,
     nm.stat_rows = stat_rows;
     nm.resid = resid_dev;
     nm.nw = nw_dev;
+    nm.in_exp = in_exp;
+    nm.out_exp = out_exp;
     W4_TRY(launch_decode(ctx, *L, x_dev, y_dev, t, out_f16, &nm));
     if (n_stats_out) *n_stats_out = nm.n_stats_out;
     return 0;
@@ -595,6 +638,14 @@ extern "C" int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name,
 extern "C" int w4a16_lin_forward_glu_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
                                                    uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols,
                                                    uint64_t y_f16_dev, int act) {
+    return w4a16_lin_forward_glu_deferred_norm_scaled(ctx, name, x_dev, ldx, t, stats_in_dev, n_stats_in, in_cols, 0,
+                                                      y_f16_dev, 0, act);
+}
+
+extern "C" int w4a16_lin_forward_glu_deferred_norm_scaled(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx,
+                                                          size_t t, uint64_t stats_in_dev, size_t n_stats_in,
+                                                          size_t in_cols, int in_exp, uint64_t y_f16_dev, int out_exp,
+                                                          int act) {
     W4Lin* L = nullptr;
     W4_TRY(w4_find_lin(ctx, name, &L));
     if (!x_dev || !y_f16_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_glu_deferred_norm %s: null operand or t=0", name);
@@ -605,6 +656,8 @@ extern "C" int w4a16_lin_forward_glu_deferred_norm(w4a16_ctx* ctx, const char* n
     nm.n_stats_in = n_stats_in;
     nm.in_cols = in_cols;
     nm.act = act;
+    nm.in_exp = in_exp;
+    nm.out_exp = out_exp;
     return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t, &nm);
 }
 

@@ -62,7 +62,7 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                             int kt_per_slice, int kt_per_wave, int ldx,
                                             const float* __restrict__ stats_in, int n_stats_in, float inv_cols_in,
                                             float* __restrict__ stats_out, int stat_rows, float* __restrict__ resid,
-                                            const float* __restrict__ nw, int act_kind) {
+                                            const float* __restrict__ nw, int act_kind, float in_scale, float out_scale) {
     extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K, then the waves' staged scales
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
     constexpr int C = 4 / XL;           // 32-k chunks (MFMAs) served by one x load
@@ -301,8 +301,11 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
         }
         if (lane == 0) __hip_atomic_store(tickets + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
     }
-    if (stats_in != nullptr) {
-        const float inv = reinterpret_cast<const float*>(red)[lane];
+    // Power-of-two factors of an f16 hand-over that could leave the f16 range otherwise: x arrives as its true value
+    // times 1/in_scale, y leaves as its true value times out_scale (both exact; 1 = none).  in_scale joins the input's
+    // 1/rms ahead of everything that looks at the values (statistics, residual, activation); out_scale is applied last.
+    if (stats_in != nullptr || in_scale != 1.0f) {
+        const float inv = (stats_in != nullptr ? reinterpret_cast<const float*>(red)[lane] : 1.0f) * in_scale;
 #pragma unroll
         for (int rb = 0; rb < RB; rb++)
 #pragma unroll
@@ -360,10 +363,21 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
             const float gt = acc[0][i], up = acc[RB - 1][i];
             float v = w4_act_mul(gt, up, act_kind);
             asm volatile("" : "+v"(v));  // the product is rounded to f32 before the f16 conversion, as in the separate kernel
+            v *= out_scale;
+            asm volatile("" : "+v"(v));
             o[i] = (_Float16)v;
         }
         *reinterpret_cast<h4_t*>(reinterpret_cast<_Float16*>(y) + (size_t)m * n_ff + blockIdx.x * 16 + 4 * g) = o;
         return;
+    }
+    if (out_scale != 1.0f) {
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                acc[rb][i] *= out_scale;
+                asm volatile("" : "+v"(acc[rb][i]));  // rounded to f32 on its own, not fused into the f16 conversion
+            }
     }
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
@@ -415,10 +429,11 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                                                         const float* stats_in, int n_stats_in,       \
                                                                         float inv_cols_in, float* stats_out,         \
                                                                         int stat_rows, float* resid,                 \
-                                                                        const float* nw, int act_kind) {             \
+                                                                        const float* nw, int act_kind,               \
+                                                                        float in_scale, float out_scale) {           \
         decode_body<G, SBF, RB, DECODE_DEPTH(BUDGET, G, RB, XL), XL>(                                                \
             qt, st, x, y, row_blocks, k, n, t, out_f16, ws, tickets, waves, nks, kt_per_slice, kt_per_wave, ldx,     \
-            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw, act_kind);                           \
+            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw, act_kind, in_scale, out_scale);                           \
     }
 #define DECODE_GLU_KERNEL_X(NAME, G, SBF, XL, BUDGET, ATTR)                                                           \
     extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
@@ -429,10 +444,11 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                                                         const float* stats_in, int n_stats_in,       \
                                                                         float inv_cols_in, float* stats_out,         \
                                                                         int stat_rows, float* resid,                 \
-                                                                        const float* nw, int act_kind) {             \
+                                                                        const float* nw, int act_kind,               \
+                                                                        float in_scale, float out_scale) {           \
         decode_body<G, SBF, 2, DECODE_DEPTH(BUDGET, G, 2, XL), XL, true>(                                            \
             qt, st, x, y, row_blocks, k, n, t, out_f16, ws, tickets, waves, nks, kt_per_slice, kt_per_wave, ldx,     \
-            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw, act_kind);                           \
+            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw, act_kind, in_scale, out_scale);                           \
     }
 #define DECODE_HI __attribute__((amdgpu_waves_per_eu(6, 6)))
 #define DECODE_MID __attribute__((amdgpu_waves_per_eu(5, 5)))

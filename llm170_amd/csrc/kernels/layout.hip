@@ -121,3 +121,45 @@ extern "C" __global__ __launch_bounds__(256) void w4a16_dump_raw_bf16(const uint
                                                                       float* out, int n, int k, int group) {
     dump_raw_body<true>(q, s, out, n, k, group);
 }
+
+// Largest row norm of the dequantised weights, max over rows of sqrt(sum_k ((nib - 8) * scale)^2): with an input of
+// unit root mean square over k columns no output element exceeds it times sqrt(k) (Cauchy-Schwarz), which sizes the
+// power-of-two factor of an f16 hand-over.  One wave per row block of the tiled copy; lanes of a row add their shares,
+// the 16 rows take the maximum, and the waves join through an integer maximum on the bits of the non-negative f32
+// (unsigned order = float order; a maximum does not depend on the order of its operands).  *out starts at zero.
+template <bool SBF>
+__device__ __forceinline__ void row_norm_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
+                                              unsigned* __restrict__ out, int row_blocks, int kt_n, int group) {
+    const int wave = (int)(((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6), lane = threadIdx.x & 63;
+    if (wave >= row_blocks) return;
+    const int r = lane & 15, gpt = W4_TILE_K / group, kg_n = kt_n * gpt;
+    float ss = 0.f;
+    for (int kt = 0; kt < kt_n; kt++) {
+        const u4_t d = qt[((size_t)wave * kt_n + kt) * 64 + lane];
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            int isum = 0;
+#pragma unroll
+            for (int p = 0; p < 8; p++) {
+                const int v = (int)((d[w] >> (4 * p)) & 0xFu) - 8;
+                isum += v * v;
+            }
+            const float sc = w4_scale_to_f32<SBF>(st[((size_t)wave * kg_n + kt * gpt + (w * 32) / group) * 16 + r]);
+            ss += (float)isum * (sc * sc);
+        }
+    }
+    ss += __shfl_xor(ss, 16);
+    ss += __shfl_xor(ss, 32);
+    float nrm = sqrtf(ss);
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) nrm = fmaxf(nrm, __shfl_xor(nrm, off));
+    if (lane == 0) atomicMax(out, __builtin_bit_cast(unsigned, nrm));
+}
+extern "C" __global__ __launch_bounds__(256) void w4a16_row_norm_max_f16(const u4_t* qt, const uint16_t* st, unsigned* out,
+                                                                         int row_blocks, int kt_n, int group) {
+    row_norm_body<false>(qt, st, out, row_blocks, kt_n, group);
+}
+extern "C" __global__ __launch_bounds__(256) void w4a16_row_norm_max_bf16(const u4_t* qt, const uint16_t* st, unsigned* out,
+                                                                          int row_blocks, int kt_n, int group) {
+    row_norm_body<true>(qt, st, out, row_blocks, kt_n, group);
+}

@@ -63,6 +63,14 @@ _SIGS = {
                                                   C.POINTER(C.c_size_t), C.c_uint64, C.c_uint64]),
     "w4a16_lin_forward_glu_deferred_norm": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_size_t, C.c_size_t,
                                                       C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64, C.c_int]),
+    "w4a16_lin_forward_deferred_norm_scaled": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_size_t, C.c_size_t,
+                                                         C.c_uint64, C.c_size_t, C.c_size_t, C.c_int, C.c_uint64, C.c_int,
+                                                         C.c_int, C.c_uint64, C.c_size_t, C.POINTER(C.c_size_t),
+                                                         C.c_uint64, C.c_uint64]),
+    "w4a16_lin_forward_glu_deferred_norm_scaled": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_size_t, C.c_size_t,
+                                                             C.c_uint64, C.c_size_t, C.c_size_t, C.c_int, C.c_uint64,
+                                                             C.c_int, C.c_int]),
+    "w4a16_lin_row_norm_max": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_float)]),
     "w4a16_lin_forward_host": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int]),
     "w4a16_dequant_dump": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int, C.c_uint64]),
     "w4a16_lin_untile": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64]),

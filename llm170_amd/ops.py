@@ -239,20 +239,37 @@ class W4a16Dec:
             ffi.check(self.cc.lib.w4a16_lin_forward_glu(self.cc.h, name.encode(), x_dev, y_f16_dev, t))
 
     def lin_forward_deferred_norm(self, name, x_dev, t, y_dev, out_f16=False, ldx=0, stats_in=0, n_stats_in=0, in_cols=0,
-                                  stats_out=0, stat_rows=0, resid=0, nw=0):
+                                  stats_out=0, stat_rows=0, resid=0, nw=0, in_exp=None, out_exp=None):
         """y = s * (W x) with s = 1/rms of the input from its producer's partial sums; returns the number of partial
-        sums this launch wrote to stats_out (0 without one)."""
+        sums this launch wrote to stats_out (0 without one).  in_exp / out_exp: x holds its true values times
+        2^-in_exp, y receives its true values times 2^-out_exp (the _scaled entry point; None, None = the plain one)."""
         n_out = C.c_size_t(0)
-        ffi.check(self.cc.lib.w4a16_lin_forward_deferred_norm(self.cc.h, name.encode(), x_dev, ldx, t, stats_in, n_stats_in,
-                                                              in_cols, y_dev, int(out_f16), stats_out, stat_rows,
-                                                              C.byref(n_out), resid, nw))
+        if in_exp is None and out_exp is None:
+            ffi.check(self.cc.lib.w4a16_lin_forward_deferred_norm(self.cc.h, name.encode(), x_dev, ldx, t, stats_in,
+                                                                  n_stats_in, in_cols, y_dev, int(out_f16), stats_out,
+                                                                  stat_rows, C.byref(n_out), resid, nw))
+        else:
+            ffi.check(self.cc.lib.w4a16_lin_forward_deferred_norm_scaled(
+                self.cc.h, name.encode(), x_dev, ldx, t, stats_in, n_stats_in, in_cols, in_exp or 0, y_dev, int(out_f16),
+                out_exp or 0, stats_out, stat_rows, C.byref(n_out), resid, nw))
         return n_out.value
 
     def lin_forward_glu_deferred_norm(self, name, x_dev, t, y_f16_dev, ldx=0, stats_in=0, n_stats_in=0, in_cols=0,
-                                      gelu=False):
-        ffi.check(self.cc.lib.w4a16_lin_forward_glu_deferred_norm(self.cc.h, name.encode(), x_dev, ldx, t, stats_in,
-                                                                  n_stats_in, in_cols, y_f16_dev,
-                                                                  ffi.ACT_GELU_TANH if gelu else ffi.ACT_SILU))
+                                      gelu=False, in_exp=None, out_exp=None):
+        act = ffi.ACT_GELU_TANH if gelu else ffi.ACT_SILU
+        if in_exp is None and out_exp is None:
+            ffi.check(self.cc.lib.w4a16_lin_forward_glu_deferred_norm(self.cc.h, name.encode(), x_dev, ldx, t, stats_in,
+                                                                      n_stats_in, in_cols, y_f16_dev, act))
+        else:
+            ffi.check(self.cc.lib.w4a16_lin_forward_glu_deferred_norm_scaled(
+                self.cc.h, name.encode(), x_dev, ldx, t, stats_in, n_stats_in, in_cols, in_exp or 0, y_f16_dev,
+                out_exp or 0, act))
+
+    def row_norm_max(self, name):
+        """Largest row norm of the linear's dequantised weights (f32, device arithmetic)."""
+        v = C.c_float(0)
+        ffi.check(self.cc.lib.w4a16_lin_row_norm_max(self.cc.h, name.encode(), C.byref(v)))
+        return v.value
 
     def gemv_host(self, name, x, t=1, out_f16=False, path=PATH_AUTO):
         """Host operands in, host result out: y [t][n] (f32, or f16 bit patterns when out_f16)."""
@@ -373,7 +390,7 @@ class W4a16Dec:
         gen.scales_f16(seed_s, n, k, group, lo, hi)."""
         ffi.check(self.cc.lib.w4a16_upload_lin_synth(self.cc.h, name.encode(), n, k, group, seed_q, seed_s, lo, hi))
 
-    def upload_chain_synth(self, prefix, n_layers, hidden, n_qkv, n_ff, group=128, seed=None):
+    def upload_chain_synth(self, prefix, n_layers, hidden, n_qkv, n_ff, group=128, seed=None, lo=0.002, hi=0.02):
         """Register n_layers synthetic decoder layers "<prefix>.<l>.<role>" with independent weights; returns the
         (seed_q, seed_s) pairs used, keyed by linear name."""
         from . import gen
@@ -386,7 +403,7 @@ class W4a16Dec:
                 n, k = shapes[role]
                 sq, ss = gen.shape_seed(n, k, seed, 100 + 8 * l + 2 * r), gen.shape_seed(n, k, seed, 101 + 8 * l + 2 * r)
                 name = "%s.%d.%s" % (prefix, l, role)
-                self.upload_lin_synth(name, n, k, group, sq, ss)
+                self.upload_lin_synth(name, n, k, group, sq, ss, lo, hi)
                 seeds[name] = (sq, ss)
         return seeds
 

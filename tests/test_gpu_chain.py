@@ -468,6 +468,111 @@ def test_fused_chain_27b_layer_shapes(dec, orc):
     assert m["rel_l2"] < 3e-3
 
 
+# ------------------------------------------------------------------ hand-overs with a power-of-two factor
+@pytest.mark.parametrize("n,k,group,bf16", [(512, 1024, 128, False), (200, 256, 32, True), (5120, 17408, 128, False)])
+def test_row_norm_max_matches_numpy(dec, orc, n, k, group, bf16):
+    """max_r sqrt(sum_c ((nib-8)*scale)^2) against float64 over the oracle's dequantised weights; a second request
+    returns the kept value."""
+    say("row norm", n, k, group, bf16)
+    q, s, _ = gen.make_linear(n, k, group, 1, seed=61)
+    if bf16:
+        s = (gen.f16_bits_to_f32(s).view(np.uint32) >> 16).astype(np.uint16)
+    dec.upload_lin_g("rn", q, s, n, k, group, bf16)
+    w = orc.dequant_matrix(q, s, n, k, group, scale_bf16=bf16).astype(np.float64)
+    want = float(np.max(np.sqrt(np.sum(w * w, axis=1))))
+    got = dec.row_norm_max("rn")
+    assert abs(got - want) <= 2e-5 * want, (got, want)
+    assert dec.row_norm_max("rn") == got
+
+
+def _pow2(bits16, e):
+    """f16 bit patterns times 2^e, exact (the caller keeps the values inside the normal range)."""
+    return gen.f32_to_f16_bits(np.ldexp(gen.f16_bits_to_f32(bits16), e).astype(np.float32))
+
+
+@pytest.mark.parametrize("e", [-3, 4])
+@pytest.mark.parametrize("t", [1, 4, 11])
+def test_scaled_handover_is_exact(dec, e, t):
+    """A power-of-two factor on a hand-over changes nothing but the exponent: the producer's f16 output with out_exp = e
+    is its un-scaled output times 2^-e bit for bit (statistics unchanged), and a consumer given x * 2^-e with in_exp = e
+    returns the bits it returns for x — plain and gated, with and without input statistics."""
+    say("scaled hand-over", e, t)
+    cc = dec.cc
+    n1, k1, n2 = 1024, 512, 512
+    q1, s1, x = gen.make_linear(n1, k1, 128, t, seed=71)
+    q2, s2, _ = gen.make_linear(n2, n1, 128, 1, seed=72)
+    dec.upload_lin_g("sh1", q1, s1, n1, k1, 128, False)
+    dec.upload_lin_g("sh2", q2, s2, n2, n1, 128, False)
+    px = cc.to_device(x)
+    pa, pb = cc.alloc(t * n1 * 2), cc.alloc(t * n1 * 2)
+    sa, sb = cc.alloc((n1 // 16) * 64), cc.alloc((n1 // 16) * 64)
+    py, pz, pg, ph = cc.alloc(t * n2 * 4), cc.alloc(t * n2 * 4), cc.alloc(t * (n2 // 2) * 2), cc.alloc(t * (n2 // 2) * 2)
+    try:
+        na = dec.lin_forward_deferred_norm("sh1", px, t, pa, out_f16=True, stats_out=sa, stat_rows=n1)
+        nb = dec.lin_forward_deferred_norm("sh1", px, t, pb, out_f16=True, stats_out=sb, stat_rows=n1, in_exp=0, out_exp=e)
+        a, b = cc.d2h(pa, (t, n1), np.uint16), cc.d2h(pb, (t, n1), np.uint16)
+        assert na == nb and np.array_equal(cc.d2h(sa, (na, 16), np.uint32)[:, :t], cc.d2h(sb, (nb, 16), np.uint32)[:, :t])
+        av = np.abs(gen.f16_bits_to_f32(a))
+        normal = (np.ldexp(av, -e) >= 6.2e-5) & (av >= 6.2e-5)  # f16 subnormals round on a different grid
+        assert normal.mean() > 0.99
+        assert np.array_equal(_pow2(a, -e)[normal], b[normal])
+        # consumer: the scaled activations with in_exp = e against the un-scaled ones, statistics in both
+        cc.h2d(pb, _pow2(a, -e))  # exact copies, subnormal elements included in neither comparison
+        a_clean = np.where(normal, a, 0).astype(np.uint16)
+        cc.h2d(pa, a_clean)
+        cc.h2d(pb, _pow2(a_clean, -e))
+        for stats in (0, sa):
+            kw = dict(stats_in=stats, n_stats_in=na if stats else 0, in_cols=n1 if stats else 0)
+            dec.lin_forward_deferred_norm("sh2", pa, t, py, **kw)
+            dec.lin_forward_deferred_norm("sh2", pb, t, pz, in_exp=e, out_exp=0, **kw)
+            assert np.array_equal(cc.d2h(py, (t, n2), np.uint32), cc.d2h(pz, (t, n2), np.uint32))
+            dec.lin_forward_glu_deferred_norm("sh2", pa, t, pg, **kw)
+            dec.lin_forward_glu_deferred_norm("sh2", pb, t, ph, in_exp=e, out_exp=0, **kw)
+            g0 = cc.d2h(pg, (t, n2 // 2), np.uint16)
+            assert np.array_equal(g0, cc.d2h(ph, (t, n2 // 2), np.uint16))
+            dec.lin_forward_glu_deferred_norm("sh2", pb, t, ph, in_exp=e, out_exp=e, **kw)
+            gv = np.abs(gen.f16_bits_to_f32(g0))
+            ok = (np.ldexp(gv, -e) >= 6.2e-5) & (gv >= 6.2e-5) & (np.ldexp(gv, -e) < 6.0e4)
+            assert np.array_equal(_pow2(g0, -e)[ok], cc.d2h(ph, (t, n2 // 2), np.uint16)[ok]) and ok.mean() > 0.9
+        with pytest.raises(ops.W4a16Error):
+            dec.lin_forward_deferred_norm("sh2", pa, t, py, in_exp=121, out_exp=0)
+    finally:
+        for p_ in (px, pa, pb, sa, sb, py, pz, pg, ph):
+            cc.free(p_)
+
+
+def test_fused_chain_keeps_large_outputs_in_range(dec, orc):
+    """Weights thirty times larger than the other chains': the down projection's output passes 65504, so an un-scaled
+    f16 hand-over would carry Inf across the layer boundary.  The chain with the normalisations deferred stays finite
+    and agrees with the chain that normalises in f32 first."""
+    hidden, n_qkv, n_ff, group, layers, t = 256, 384, 512, 128, 3, 4
+    shapes = {"attn_qkv": (n_qkv, hidden), "attn_output": (hidden, hidden), "ffn_gate_up": (2 * n_ff, hidden),
+              "ffn_down": (hidden, n_ff)}
+    seeds = dec.upload_chain_synth("fbig", layers, hidden, n_qkv, n_ff, group, lo=0.06, hi=0.6)
+    x = gen.normal_f16(77, (t, hidden))
+    lins0 = []
+    for role in ops.W4a16Dec.CHAIN_ROLES:
+        n, k = shapes[role]
+        sq, ss = seeds["fbig.0.%s" % role]
+        lins0.append((gen.weights_q(sq, n, k), gen.scales_f16(ss, n, k, group, 0.06, 0.6), n, k))
+    v4 = orc.chain_layer_fused(x, np.ones(t, np.float32), lins0, group, 4)["v4"]
+    say("fused chain, large weights: max |v4| of layer 0 =", float(np.max(np.abs(v4))))
+    assert np.max(np.abs(v4)) > 65504.0
+    cc = dec.cc
+    px, py, pz = cc.to_device(x), cc.alloc(t * hidden * 2), cc.alloc(t * hidden * 2)
+    try:
+        dec.chain_forward_fused("fbig", 0, layers, px, t, py)
+        dec.chain_forward("fbig", 0, layers, px, t, pz)
+        got, want = _f16(cc.d2h(py, (t, hidden), np.uint16)), _f16(cc.d2h(pz, (t, hidden), np.uint16))
+        assert np.all(np.isfinite(got)) and np.all(np.isfinite(want))
+        m = parity.compare(got, want)
+        say("  fused vs unfused rel_l2", m["rel_l2"])
+        assert m["rel_l2"] < 2e-2
+    finally:
+        for p_ in (px, py, pz):
+            cc.free(p_)
+
+
 # ------------------------------------------------------------------ norm_resid (assets/norm.cu:4-48, 97-148)
 @pytest.mark.parametrize("t,hidden,w_off", [(1, 5120, 0), (4, 5120, 5120), (7, 2048, 0), (3, 1000, 24), (2, 8192, 0),
                                             (5, 64, 0)])

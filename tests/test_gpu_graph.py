@@ -118,11 +118,11 @@ def test_chain_graph_small(dec, orc, fused):
 
 def test_chain_graph_64_layers_at_27b_shapes(dec):
     """The chain the benchmark times: 64 layers of QKV 5120->7168, O 5120->5120, gate|up 5120->34816, down
-    17408->5120 at M = 4 (10.9 GB of device-generated weights).  Output finite and of unit mean square, the same bits
-    from eager passes and from graph replays.  The statement with the normalisations deferred across the linears is
-    checked on the first two layers only: it carries the un-normalised down-projection output in f16, and on these
-    synthetic weights (mean -0.5, no residual stream) that output leaves the f16 range from the third layer on — the
-    range precondition stated with w4a16_lin_forward_deferred_norm."""
+    17408->5120 at M = 4 (10.9 GB of device-generated weights), with its normalisation launches and with the
+    normalisations deferred across the linears.  Output finite and of unit mean square, the same bits from eager passes
+    and from graph replays.  On these synthetic weights (mean -0.5, no residual stream) the un-normalised output of the
+    down projection passes the f16 range from the third layer on: the deferred form stays finite only because its
+    hand-overs carry their power-of-two factors."""
     layers, hidden, n_qkv, n_ff, t = 64, 5120, 7168, 17408, 4
     cc = dec.cc
     say("chain 64: generating")
@@ -131,7 +131,7 @@ def test_chain_graph_64_layers_at_27b_shapes(dec):
         for role in ops.W4a16Dec.CHAIN_ROLES:
             dec.drop_raw("c64.%d.%s" % (l, role))
     px, py = cc.to_device(gen.normal_f16(404, (t, hidden))), cc.alloc(t * hidden * 2)
-    for fused, n_l in ((False, layers), (True, 2)):
+    for fused, n_l in ((False, layers), (True, layers)):
         run = dec.chain_forward_fused if fused else dec.chain_forward
         run("c64", 0, n_l, px, t, py)
         eager = cc.d2h(py, (t, hidden), np.uint16)
