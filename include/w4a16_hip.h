@@ -347,6 +347,12 @@ int w4a16_moe_scratch(w4a16_ctx* ctx, int which, uint64_t* dptr, size_t* bytes, 
 /* Launch-shape override for the MoE GEMMs (0 = automatic): block = slots per segment (4, 16, 32, 48, 64; 1 = direct mode);
  * waves = waves per workgroup (k split for segments of <= 16 slots, output-row units otherwise). */
 int w4a16_set_moe_shape(w4a16_ctx* ctx, int block, int waves);
+/* The MFMA-tiled grouped kernels (the role of the reference's grouped Marlin GEMM at prefill sizes, assets/moe.cu:686-759
+ * via kernels/marlin_moe.rs:290-422): workgroup = one 64-slot segment x 256 output columns on 32x32x16 MFMA tiles, the
+ * segment's x rows gathered into LDS, expert weights as the B operand straight from the arena.  0 = automatic (mean run
+ * per expert of at least 96 slots, i.e. t * top_k >= 96 * n_experts, and no segment size forced), -1 = never, 1 =
+ * always (64-slot segments whatever t).  Same results as the streaming kernels up to the order of the f32 sums. */
+int w4a16_set_moe_tiled(w4a16_ctx* ctx, int mode);
 /* Timed back-to-back w4a16_moe_ffn calls (as w4a16_bench_forward); call i uses experts names[i % n_names]. */
 int w4a16_bench_moe(w4a16_ctx* ctx, const char* const* names, size_t n_names, uint64_t x_dev, uint64_t idx_dev,
                     uint64_t wt_dev, size_t t, size_t top_k, uint64_t y_dev, size_t warmup, size_t reps,

@@ -66,7 +66,10 @@ static const char* const kDecodeSyms[] = {
     nullptr};
 static const char* const kPrefillSyms[] = {"w4a16_prefill_g128_f16", "w4a16_prefill_g128_bf16", "w4a16_prefill_g32_f16",
                                            "w4a16_prefill_g32_bf16", "w4a16_prefill_g128_f16_m64", "w4a16_prefill_g128_bf16_m64", "w4a16_prefill_g32_f16_m64",
-                                           "w4a16_prefill_g32_bf16_m64", "w4a16_prefill_splitk_sum", nullptr};
+                                           "w4a16_prefill_g32_bf16_m64", "w4a16_prefill_splitk_sum",
+                                           "w4a16_moe_g128_f16_pf_glu", "w4a16_moe_g128_f16_pf_lin", "w4a16_moe_g128_bf16_pf_glu",
+                                           "w4a16_moe_g128_bf16_pf_lin", "w4a16_moe_g32_f16_pf_glu", "w4a16_moe_g32_f16_pf_lin",
+                                           "w4a16_moe_g32_bf16_pf_glu", "w4a16_moe_g32_bf16_pf_lin", nullptr};
 static const char* const kUtilSyms[] = {"w4a16_fill0_u32", nullptr};
 static const char* const kGlueSyms[] = {"w4a16_rms_rescale_f16", "w4a16_silu_mul_f16", "w4a16_synth_q", "w4a16_synth_s",
                                         "w4a16_norm_resid", nullptr};

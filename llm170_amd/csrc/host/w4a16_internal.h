@@ -80,6 +80,7 @@ struct w4a16_ctx {
     W4MoeScratch moe;
     W4ChainScratch chain;
     int moe_block = 0, moe_waves = 0;  // 0 = automatic
+    int moe_tiled = 0;                 // MFMA-tiled grouped kernel: 0 = automatic (long runs per expert), -1 = never, 1 = always
     int moe_act_kind = 0;              // activation of the expert FFN call in progress (W4A16_ACT_*)
     int decode_rows_per_wave = 0, decode_waves_per_block = 0;  // 0 = automatic
     uint64_t norm_word = 0;  // one device word for w4a16_lin_row_norm_max

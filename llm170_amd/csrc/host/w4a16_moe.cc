@@ -219,7 +219,7 @@ static size_t pick_block(const w4a16_ctx* ctx, size_t t, size_t ns, size_t n_exp
 
 static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_t x, size_t x_rows, size_t x_div,
                            uint64_t y, int y_f16, uint64_t topw, size_t ns, size_t block, size_t max_segs,
-                           uint64_t sorted, uint64_t eids, uint64_t npost, size_t nks = 1) {
+                           uint64_t sorted, uint64_t eids, uint64_t npost, size_t nks = 1, bool tiled = false) {
     const size_t n = glu ? 2 * E.n_ff : E.h, k = glu ? E.h : E.n_ff;
     const size_t row_blocks = (n + 15) / 16, kt_n = k / 128;
     const size_t units = glu ? row_blocks / 2 : (row_blocks + 1) / 2;
@@ -236,6 +236,15 @@ static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_
                  &ws, &tk, &waves, &act_kind};
     char sym[80];
     const char* fam = E.scale_bf16 ? "bf16" : "f16";
+    if (tiled) {
+        // MFMA-tiled grouped kernel (kernels/prefill.hip, MODE 1 / 2): block tile = one 64-slot segment x 256 columns
+        // (gate|up: 128 gate + the 128 matching up columns); LDS = two x stages of 64 rows x 64 k and the slot ids
+        if (block != 64) return w4_fail(W4A16_ERR_ARG, "moe: the tiled grouped kernel needs 64-slot segments (got %zu)", block);
+        if (max_segs > 65535) return w4_fail(W4A16_ERR_SHAPE, "moe: %zu segments exceed the grid", max_segs);
+        const size_t cols = glu ? E.n_ff : n, per_tile = glu ? 128 : 256;
+        snprintf(sym, sizeof sym, "w4a16_moe_g%zu_%s_pf_%s", E.group, fam, glu ? "glu" : "lin");
+        return w4_launch(ctx, sym, (unsigned)((cols + per_tile - 1) / per_tile), (unsigned)max_segs, 256, 2 * 64 * 64 * 2 + 256, p);
+    }
     if (block <= 16) {
         // in-block split-K: each wave needs at least one k tile
         waves = ctx->moe_waves ? ctx->moe_waves : 4;
@@ -382,7 +391,10 @@ extern "C" int w4a16_moe_ffn_act(w4a16_ctx* ctx, const char* name, uint64_t x_de
         return w4_fail(W4A16_ERR_SHAPE, "moe_ffn %s: t=%zu top_k=%zu experts=%zu", name, t, top_k, E->n_exp);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
     const size_t ns = t * top_k;
-    const size_t block = pick_block(ctx, t, ns, E->n_exp, top_k);
+    // From a mean run of 96 slots per expert on, 64-slot segments are mostly full and the MFMA-tiled grouped kernel
+    // (one segment x 256 columns per workgroup, x through LDS, 32x32x16 tiles) takes over from the streaming kernels.
+    const bool tiled = ctx->moe_tiled > 0 || (ctx->moe_tiled == 0 && ctx->moe_block == 0 && ns >= 96 * E->n_exp);
+    const size_t block = tiled ? 64 : pick_block(ctx, t, ns, E->n_exp, top_k);
     if (block != 1 && block != 4 && block != 16 && block != 32 && block != 48 && block != 64)
         return w4_fail(W4A16_ERR_ARG, "moe_ffn %s: segment size %zu not in {1,4,16,32,48,64}", name, block);
     if (block == 1) return moe_ffn_direct(ctx, name, *E, x_dev, idx_dev, wt_dev, t, top_k, y_dev);
@@ -403,10 +415,10 @@ extern "C" int w4a16_moe_ffn_act(w4a16_ctx* ctx, const char* name, uint64_t x_de
     W4_TRY(w4a16_moe_align(ctx, idx_dev, ns, E->n_exp, block, S.sorted, S.expert_ids, S.num_post));
     // gate|up with the SiLU*up epilogue: slot j reads token j / top_k
     W4_TRY(launch_moe_gemm(ctx, *E, true, x_dev, t, top_k, S.act, 1, 0, ns, block, max_segs, S.sorted, S.expert_ids,
-                           S.num_post));
+                           S.num_post, 1, tiled));
     // down, multiplied by the routing weight: slot j reads act row j
     W4_TRY(launch_moe_gemm(ctx, *E, false, S.act, ns, 1, S.c2, 1, wt_dev, ns, block, max_segs, S.sorted, S.expert_ids,
-                           S.num_post));
+                           S.num_post, 1, tiled));
     int ti = (int)t, hi = (int)E->h, ki = (int)top_k;
     void* p[] = {&S.c2, &y_dev, &ti, &hi, &ki};
     return w4_launch(ctx, "w4a16_moe_topk_sum_f16", std::min<unsigned>(ceil_div(t * E->h / (E->h % 8 == 0 ? 8 : 1), 256), 4096), 1, 256, 0, p);
@@ -435,6 +447,13 @@ extern "C" int w4a16_set_moe_shape(w4a16_ctx* ctx, int block, int waves) {
         return w4_fail(W4A16_ERR_ARG, "set_moe_shape: block in {0,1,4,16,32,48,64}, waves in 0..8");
     ctx->moe_block = block;
     ctx->moe_waves = waves;
+    return 0;
+}
+
+extern "C" int w4a16_set_moe_tiled(w4a16_ctx* ctx, int mode) {
+    if (!ctx) return w4_fail(W4A16_ERR_ARG, "set_moe_tiled: null context");
+    if (mode < -1 || mode > 1) return w4_fail(W4A16_ERR_ARG, "set_moe_tiled: -1 = never, 0 = automatic, 1 = always");
+    ctx->moe_tiled = mode;
     return 0;
 }
 

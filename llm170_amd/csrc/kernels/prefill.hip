@@ -40,11 +40,32 @@ __device__ __forceinline__ float pf_ratio(float s_prev, float s_cur) {
 // MI = 32-row MFMA tiles along m per wave: 4 (block tile 128 x 256, 128 accumulator registers, two workgroups per CU) or
 // 2 (64 x 256, 64 registers, three workgroups per CU) for a few dozen to a couple of hundred rows, where 128-row tiles
 // would spend half their MFMAs on padding and leave too few workgroups.
-template <int G, bool SBF, int MI>
+//
+// Grouped form for the expert FFN (MODE 1, 2): the role of the reference's grouped Marlin GEMM at prefill sizes
+// (assets/moe.cu:686-759 via kernels/marlin_moe.rs:290-422).  The rows of a block tile are one 64-slot segment of the
+// alignment pass (sorted_ids, padded with the sentinel ns; expert_ids per segment; num_post = padded slot total), the
+// weights are those of the segment's expert in its arena, x rows are gathered by slot id (slot j reads row j / x_div)
+// straight into the LDS stage by the same DMA, and the epilogue scatters by slot id:
+//   MODE 1 (gate|up, n = 2 n_ff): a wave's two 32-column sub-tiles are gate columns c.. and up columns n_ff + c.., so
+//     the lane that holds a gate sum holds the matching up sum; both are rounded to f16 (the reference materialises
+//     them as f16) and act[slot][c] = f16(act(gate) * up) is written, f16 [ns][n_ff];
+//   MODE 2 (down, n = hidden): y[slot][c] = sum * topw[slot] as f16 or f32 [ns][n].
+template <int MODE>
+struct PfGroup {
+    const int* sorted_ids;
+    const int* expert_ids;
+    const int* num_post;
+    const float* topw;
+    unsigned long long q_stride, s_stride;  // bytes per expert
+    int ns, x_rows, x_div, n_exp, act_kind;
+};
+
+template <int G, bool SBF, int MI, int MODE = 0>
 __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                              const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
-                                             int k, int n, int t, int out_f16, int sup_m, int sup_n) {
-    extern __shared__ _Float16 lds[];  // 2 stages x [PF_BM][PF_LDA]
+                                             int k, int n, int t, int out_f16, int sup_m, int sup_n,
+                                             const PfGroup<MODE> gp = PfGroup<MODE>()) {
+    extern __shared__ _Float16 lds[];  // 2 stages x [PF_BM][PF_LDA]; grouped: then the segment's PF_BM slot ids
     constexpr int GPT = W4_TILE_K / G;
     constexpr int PF_BM = 32 * MI, PF_STAGE_BYTES = PF_BM * PF_LDA * 2;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -56,17 +77,32 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     // blocks of an XCD walk one super-tile of sup_m x sup_n block tiles (m fastest), so the blocks resident on an XCD
     // at a time share x slabs and weight panels through its L2.  Super-tiles are dealt round-robin to the XCDs.  The
     // host picks the super-tile shape: 8 x 8 on large grids, smaller on small ones so that every XCD gets work.
-    const int tiles_m = (t + PF_BM - 1) / PF_BM, tiles_n = (n + PF_BN - 1) / PF_BN;
-    const int sm_n = (tiles_m + sup_m - 1) / sup_m, sn_n = (tiles_n + sup_n - 1) / sup_n;
-    const int per = sup_m * sup_n;
-    const int j = blockIdx.x >> 3;
-    const int super = (blockIdx.x & 7) + 8 * (j / per), within = j % per;
-    if (super >= sm_n * sn_n) return;  // uniform for the whole block
-    const int tm = (super % sm_n) * sup_m + within % sup_m, tn = (super / sm_n) * sup_n + within / sup_m;
-    if (tm >= tiles_m || tn >= tiles_n) return;
-    const int m0 = tm * PF_BM, n0 = tn * PF_BN;
+    int m0, n0;
+    if (MODE == 0) {
+        const int tiles_m = (t + PF_BM - 1) / PF_BM, tiles_n = (n + PF_BN - 1) / PF_BN;
+        const int sm_n = (tiles_m + sup_m - 1) / sup_m, sn_n = (tiles_n + sup_n - 1) / sup_n;
+        const int per = sup_m * sup_n;
+        const int j = blockIdx.x >> 3;
+        const int super = (blockIdx.x & 7) + 8 * (j / per), within = j % per;
+        if (super >= sm_n * sn_n) return;  // uniform for the whole block
+        const int tm = (super % sm_n) * sup_m + within % sup_m, tn = (super / sm_n) * sup_n + within / sup_m;
+        if (tm >= tiles_m || tn >= tiles_n) return;
+        m0 = tm * PF_BM;
+        n0 = tn * PF_BN;
+    } else {
+        // grouped: blockIdx.x = column tile (fastest, so the tiles of a segment run together and share its x rows
+        // through the L2), blockIdx.y = segment.  Gate|up tiles span 128 gate and the 128 matching up columns.
+        const int seg = blockIdx.y;
+        m0 = seg * PF_BM;  // position in sorted_ids
+        if (m0 >= gp.num_post[0]) return;
+        const int e = gp.expert_ids[seg];
+        if ((unsigned)e >= (unsigned)gp.n_exp) return;
+        qt = reinterpret_cast<const u4_t*>(reinterpret_cast<const char*>(qt) + (size_t)e * gp.q_stride);
+        st = reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(st) + (size_t)e * gp.s_stride);
+        n0 = blockIdx.x * (MODE == 1 ? PF_BN / 2 : PF_BN);
+    }
 
-    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)t * (unsigned)k * 2u);
+    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)(MODE == 0 ? t : gp.x_rows) * (unsigned)k * 2u);
     const __amdgpu_buffer_rsrc_t qr = w4_make_rsrc(qt, (unsigned)row_blocks * (unsigned)kt_n * 1024u);
     const __amdgpu_buffer_rsrc_t sr = w4_make_rsrc(st, (unsigned)row_blocks * (unsigned)kg_n * 32u);
 
@@ -81,8 +117,15 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
 #pragma unroll
     for (int i = 0; i < MI; i++) {
         const int c = tid + i * PF_THREADS, row = c >> 3, kc = (c & 7) ^ (row & 7);
-        xa_off[i] = (m0 + row < t) ? ((unsigned)(m0 + row) * (unsigned)k + (unsigned)kc * 8u) * 2u : W4_OOB;
+        if (MODE == 0) {
+            xa_off[i] = (m0 + row < t) ? ((unsigned)(m0 + row) * (unsigned)k + (unsigned)kc * 8u) * 2u : W4_OOB;
+        } else {
+            const int id = gp.sorted_ids[m0 + row];  // padding rows carry the sentinel ns: zeros, never stored
+            xa_off[i] = id < gp.ns ? ((unsigned)(id / gp.x_div) * (unsigned)k + (unsigned)kc * 8u) * 2u : W4_OOB;
+        }
     }
+    int* const seg_ids = reinterpret_cast<int*>(lds_base + 2 * PF_STAGE_BYTES);
+    if (MODE != 0 && tid < PF_BM) seg_ids[tid] = gp.sorted_ids[m0 + tid];  // visible after the first barrier
     auto load_a = [&](int s, int buf) {
 #pragma unroll
         for (int i = 0; i < MI; i++)
@@ -96,7 +139,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     unsigned q_off[2][2], s_off[2];
 #pragma unroll
     for (int ni = 0; ni < 2; ni++) {
-        const int nrow = n0 + wn * 64 + ni * 32 + nl;
+        const int nrow = MODE == 1 ? ni * (n >> 1) + n0 + wn * 32 + nl : n0 + wn * 64 + ni * 32 + nl;
         const unsigned rb = (unsigned)min(nrow >> 4, row_blocks - 1);  // rows past n re-read the last block, never stored
         const unsigned r = (unsigned)(nrow & 15);
 #pragma unroll
@@ -129,7 +172,8 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     const int a_row = nl;  // + mi * 32
     // split-K over gridDim.y (narrow outputs at moderate t, where the tile grid alone cannot fill the chip): this
     // block covers k tiles [kt_lo, kt_hi) and writes an f32 partial; a second launch adds the partials in order
-    const int kt_lo = (kt_n * (int)blockIdx.y) / (int)gridDim.y, kt_hi = (kt_n * ((int)blockIdx.y + 1)) / (int)gridDim.y;
+    const int kt_lo = MODE == 0 ? (kt_n * (int)blockIdx.y) / (int)gridDim.y : 0,
+              kt_hi = MODE == 0 ? (kt_n * ((int)blockIdx.y + 1)) / (int)gridDim.y : kt_n;
     const int stages = 2 * kt_hi;
 
     load_a(2 * kt_lo, 0);
@@ -209,6 +253,45 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     }
 
     // ---- epilogue: y[m][n] = acc * unit; D register e of lane (nl, khalf) is row 8*(e/4) + 4*khalf + e%4, column nl
+    if (MODE == 1) {
+        const int n_ff = n >> 1, col = n0 + wn * 32 + nl;
+        if (col >= n_ff) return;
+#pragma unroll
+        for (int mi = 0; mi < MI; mi++) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int slot = seg_ids[mi * 32 + 8 * (e >> 2) + 4 * khalf + (e & 3)];
+                if (slot < gp.ns) {
+                    const float gt = (float)(_Float16)(acc[mi][0][e] * unit[0]), up = (float)(_Float16)(acc[mi][1][e] * unit[1]);
+                    reinterpret_cast<_Float16*>(y)[(size_t)slot * n_ff + col] = (_Float16)w4_act_mul(gt, up, gp.act_kind);
+                }
+            }
+        }
+        return;
+    }
+    if (MODE == 2) {
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++) {
+            const int col = n0 + wn * 64 + ni * 32 + nl;
+            if (col >= n) continue;
+#pragma unroll
+            for (int mi = 0; mi < MI; mi++) {
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int slot = seg_ids[mi * 32 + 8 * (e >> 2) + 4 * khalf + (e & 3)];
+                    if (slot < gp.ns) {
+                        float v = acc[mi][ni][e] * unit[ni];
+                        if (gp.topw != nullptr) v *= gp.topw[slot];
+                        if (out_f16)
+                            reinterpret_cast<_Float16*>(y)[(size_t)slot * n + col] = (_Float16)v;
+                        else
+                            reinterpret_cast<float*>(y)[(size_t)slot * n + col] = v;
+                    }
+                }
+            }
+        }
+        return;
+    }
     if (gridDim.y > 1) y = reinterpret_cast<float*>(y) + (size_t)blockIdx.y * (size_t)t * (size_t)n;  // partial (f32)
 #pragma unroll
     for (int ni = 0; ni < 2; ni++) {
@@ -238,6 +321,31 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
         prefill_body<G, SBF, MI>(qt, st, x, y, row_blocks, k, n, t, out_f16, sup_m, sup_n);                            \
     }
 
+// Grouped kernels for the expert FFN: same arguments as the streaming grouped kernels of moe.hip (blk must be 64, the
+// rows of a block tile; ws, tickets and wpb are unused).
+#define PREFILL_MOE_KERNEL(NAME, G, SBF, MODE)                                                                          \
+    extern "C" __global__ __launch_bounds__(PF_THREADS) __attribute__((amdgpu_waves_per_eu(3, 3))) void NAME(            \
+        const char* qa, const char* sa, unsigned long long q_stride, unsigned long long s_stride, const uint16_t* x,      \
+        int x_rows, int x_div, void* y, int y_f16, const float* topw, const int* sorted_ids, const int* expert_ids,      \
+        const int* num_post, int blk, int ns, int row_blocks, int k, int n, int n_exp, f4_t* ws, int* tickets, int wpb,  \
+        int act_kind) {                                                                                                  \
+        PfGroup<MODE> gp;                                                                                                \
+        gp.sorted_ids = sorted_ids;                                                                                      \
+        gp.expert_ids = expert_ids;                                                                                      \
+        gp.num_post = num_post;                                                                                          \
+        gp.topw = topw;                                                                                                  \
+        gp.q_stride = q_stride;                                                                                          \
+        gp.s_stride = s_stride;                                                                                          \
+        gp.ns = ns;                                                                                                      \
+        gp.x_rows = x_rows;                                                                                              \
+        gp.x_div = x_div;                                                                                                \
+        gp.n_exp = n_exp;                                                                                                \
+        gp.act_kind = act_kind;                                                                                          \
+        (void)blk, (void)ws, (void)tickets, (void)wpb;                                                                   \
+        prefill_body<G, SBF, 2, MODE>(reinterpret_cast<const u4_t*>(qa), reinterpret_cast<const uint16_t*>(sa), x, y,    \
+                                      row_blocks, k, n, 0, y_f16, 1, 1, gp);                                             \
+    }
+
 // y[i] = sum over the nks partials of a split-K launch, added in split order in f32; f32 or f16 out.
 extern "C" __global__ __launch_bounds__(256) void w4a16_prefill_splitk_sum(const float* __restrict__ part, void* __restrict__ y,
                                                                            int nks, size_t count, int out_f16) {
@@ -262,3 +370,11 @@ PREFILL_KERNEL(w4a16_prefill_g128_f16_m64, 128, false, 2, 3)
 PREFILL_KERNEL(w4a16_prefill_g128_bf16_m64, 128, true, 2, 3)
 PREFILL_KERNEL(w4a16_prefill_g32_f16_m64, 32, false, 2, 3)
 PREFILL_KERNEL(w4a16_prefill_g32_bf16_m64, 32, true, 2, 3)
+PREFILL_MOE_KERNEL(w4a16_moe_g128_f16_pf_glu, 128, false, 1)
+PREFILL_MOE_KERNEL(w4a16_moe_g128_f16_pf_lin, 128, false, 2)
+PREFILL_MOE_KERNEL(w4a16_moe_g128_bf16_pf_glu, 128, true, 1)
+PREFILL_MOE_KERNEL(w4a16_moe_g128_bf16_pf_lin, 128, true, 2)
+PREFILL_MOE_KERNEL(w4a16_moe_g32_f16_pf_glu, 32, false, 1)
+PREFILL_MOE_KERNEL(w4a16_moe_g32_f16_pf_lin, 32, false, 2)
+PREFILL_MOE_KERNEL(w4a16_moe_g32_bf16_pf_glu, 32, true, 1)
+PREFILL_MOE_KERNEL(w4a16_moe_g32_bf16_pf_lin, 32, true, 2)

@@ -99,6 +99,7 @@ _SIGS = {
     "w4a16_moe_scratch": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_size_t),
                                     C.POINTER(C.c_size_t)]),
     "w4a16_set_moe_shape": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
+    "w4a16_set_moe_tiled": (C.c_int, [C.c_void_p, C.c_int]),
     "w4a16_upload_lin_synth": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint64, C.c_uint64,
                                          C.c_float, C.c_float]),
     "w4a16_rms_rescale_f16": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint64]),

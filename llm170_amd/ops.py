@@ -375,6 +375,10 @@ class W4a16Dec:
     def set_moe_shape(self, block=0, waves=0):
         ffi.check(self.cc.lib.w4a16_set_moe_shape(self.cc.h, block, waves))
 
+    def set_moe_tiled(self, mode=0):
+        """MFMA-tiled grouped kernels for the expert FFN: 0 = automatic (long runs per expert), -1 = never, 1 = always."""
+        ffi.check(self.cc.lib.w4a16_set_moe_tiled(self.cc.h, mode))
+
     def bench_moe(self, names, x_dev, idx_dev, wt_dev, t, top_k, y_dev, reps, warmup=1):
         arr = (C.c_char_p * len(names))(*[n.encode() for n in names])
         ms, wall = C.c_float(), C.c_double()

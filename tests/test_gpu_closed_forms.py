@@ -119,7 +119,7 @@ def test_power_of_two_operands_group_32(dec):
 
 # ------------------------------------------------------------------ MoE expert FFN, closed form end to end
 def test_moe_ffn_exact_operands_full_shape(dec):
-    """128 experts, top-8, hidden 2048, n_ff 768, group 32, T = 512 (grouped GEMMs), 64 and 4 (direct mode), on
+    """128 experts, top-8, hidden 2048, n_ff 768, group 32, T = 512 (grouped GEMMs, streaming and MFMA-tiled), 64 and 4 (direct mode), on
     operands that make every stage exactly computable on the host:
       x[token] = c * (+1, -1, +1, ...), c = 1 or 2 by token; gate rows +7, -7, +7, ... with scale 2^-9: gate = 28 c, where silu(g) = g in
       f32 (exp(-28) < 2^-25), so act = f16(f16(gate) * f16(up)); up = power-of-two scales times integer sums (exact);
@@ -155,15 +155,20 @@ def test_moe_ffn_exact_operands_full_shape(dec):
         return stage[(e, c)]
 
     cc = dec.cc
-    for t in (512, 64, 4):
-        say("moe exact", t)
+    for t, tiled in ((512, False), (512, True), (64, False), (4, False)):  # tiled: the 32x32x16 grouped kernels
+        say("moe exact", t, "tiled" if tiled else "")
         cs = (gen.stream(77 + t, t) % np.uint64(2)).astype(np.int64) + 1
         x = (alt[None, :] * cs[:, None]).astype(np.float16).view(np.uint16)
         idx, wt = ops.moe_topk(gen.router_logits(t, E, seed=900 + t), k)
         px, pi, pw, py = cc.to_device(x), cc.to_device(idx), cc.to_device(wt), cc.alloc(t * h * 4)
-        dec.moe_ffn("p2moe", px, pi, pw, t, k, py)
+        dec.set_moe_tiled(1 if tiled else 0)
+        try:
+            dec.moe_ffn("p2moe", px, pi, pw, t, k, py)
+        finally:
+            dec.set_moe_tiled(0)
         y = cc.d2h(py, (t, h), np.float32)
         act, blk = dec.moe_scratch(3, np.uint16)
+        assert not tiled or blk == 64
         act = act.reshape(t * k, n_ff)
         c2 = None if blk == 1 else dec.moe_scratch(4, np.uint16)[0].reshape(t * k, h)
         for p_ in (px, pi, pw, py):

@@ -269,6 +269,60 @@ def test_moe_ffn_full_shape(dec, orc, full_experts, t):
     say("  blk", blk, "act identical", same, "c2", m2["rel_l2"], m2["max_ulp"], "y rel_l2", m["rel_l2"])
 
 
+# ------------------------------------------------------------------ the MFMA-tiled grouped kernels (long runs per expert)
+@pytest.mark.parametrize("group,bf", [(32, False), (32, True), (128, False), (128, True)])
+@pytest.mark.parametrize("t", [5, 40, 200, 333])
+def test_moe_ffn_tiled_small(dec, orc, small_experts, group, bf, t):
+    """The 64-slot-segment x 256-column kernels on 32x32x16 tiles, forced at sizes where most segments are ragged:
+    same stage-by-stage checks as the streaming kernels."""
+    say("moe_ffn tiled small", group, bf, t)
+    name, q13, s13, q2, s2 = small_experts[(group, bf)]
+    E, h, n_ff, k = SMALL["E"], SMALL["h"], SMALL["n_ff"], SMALL["k"]
+    x = gen.normal_f16(1500 + t, (t, h))
+    idx, wt = ops.moe_topk(gen.router_logits(t, E, seed=20 + t), k)
+    dec.set_moe_tiled(1)
+    try:
+        y, act, c2, blk = _run_ffn(dec, name, x, idx, wt, t, k, h)
+        assert blk == 64 and dec.cc.last_launch_symbol() == "w4a16_moe_topk_sum_f16"
+        _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, "tiled g%d bf%d t%d" % (group, bf, t))
+        if t == 200:
+            y, act, c2, blk = _run_ffn(dec, name, x, idx, wt, t, k, h, gelu=True)
+            _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, "tiled gelu", gelu=True)
+            # a hot expert (runs of several segments) and experts nobody chose
+            idx2 = np.empty((t, k), np.int32)
+            idx2[:, 0] = 6
+            idx2[:, 1] = np.arange(t) % 2
+            wt2 = np.full((t, k), 0.5, np.float32)
+            y, act, c2, blk = _run_ffn(dec, name, x, idx2, wt2, t, k, h)
+            _check_ffn(orc, y, act, c2, x, idx2, wt2, q13, s13, q2, s2, h, n_ff, group, bf, "tiled hot expert")
+    finally:
+        dec.set_moe_tiled(0)
+
+
+def test_moe_ffn_tiled_full_shape(dec, orc, full_experts):
+    """T = 2048 at the 35B-A3B layer shape: a mean run of 128 slots per expert, where AUTO picks the tiled kernels; and
+    never does below the threshold or with a forced segment size."""
+    name, q13, s13, q2, s2 = full_experts
+    E, h, n_ff, k, t = 128, 2048, 768, 8, 2048
+    say("moe_ffn tiled full", t)
+    x = gen.normal_f16(4242 + t, (t, h))
+    idx, wt = ops.moe_topk(gen.router_logits(t, E), k)
+    y, act, c2, blk = _run_ffn(dec, name, x, idx, wt, t, k, h)
+    assert blk == 64
+    same, m2, m = _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, 32, False, "a3b tiled t%d" % t, threads=16)
+    say("  act identical", same, "c2", m2["rel_l2"], m2["max_ulp"], "y rel_l2", m["rel_l2"])
+    dec.set_moe_tiled(-1)
+    try:
+        y2, act2, c22, blk2 = _run_ffn(dec, name, x, idx, wt, t, k, h)
+    finally:
+        dec.set_moe_tiled(0)
+    m3 = parity.compare(y, y2)
+    say("  tiled vs streaming rel_l2", m3["rel_l2"], "act identical", float(np.mean(act == act2)))
+    assert m3["rel_l2"] < 1e-4 and np.mean(act == act2) > 0.97
+    with pytest.raises(ops.W4a16Error):
+        dec.set_moe_tiled(2)
+
+
 def test_moe_errors(dec, small_experts):
     name = small_experts[(32, False)][0]
     with pytest.raises(ops.W4a16Error):
