@@ -12,6 +12,7 @@ Prints ONE JSON line.  `value` is algorithmic bytes per step / time per step (GB
 restatement of the reference's CPU contract) on the box's host cores.
 """
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -46,21 +47,41 @@ def make_copies(dec, gen, n, k, g, copies, prefix):
     return names, first
 
 
+def kernel_source_hash(kernel):
+    """sha256 (16 hex digits) over the source file a kernel is built from and the header all kernels share."""
+    csrc = os.path.join(ROOT, "llm170_amd", "csrc")
+    src = ("bench/probes.hip" if kernel in PROBE_SYMS else "kernels/decode.hip" if kernel.startswith("w4a16_decode")
+           else "kernels/prefill.hip" if kernel.startswith("w4a16_prefill") else None)
+    if src is None:
+        return None
+    h = hashlib.sha256()
+    for f in (src, "kernels/w4a16_common.hpp"):
+        with open(os.path.join(csrc, f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic(kernel):
     """HBM bytes per launch of `kernel` from the committed counter summary profiles/pmc_traffic.txt (rocprofv3 --pmc
     FETCH_SIZE / WRITE_SIZE, scaled by the plain-copy calibration): (bytes, provenance) — a recorded figure, not a
-    measurement of this run; (None, reason) when the summary has no line for the kernel this run dispatched."""
+    measurement of this run.  The summary records the hash of the kernel's source at the time of the counter runs;
+    (None, reason) when it has no line for the kernel this run dispatched or when that source has changed since."""
     path = os.path.join(ROOT, "profiles", "pmc_traffic.txt")
     if not os.path.exists(path):
         return None, "no profiles/pmc_traffic.txt"
-    recorded = ""
+    recorded, value = None, None
     for ln in open(path):
         f = ln.split()
-        if len(f) >= 3 and f[0] == "recorded_at_source_hash":
-            recorded = f[1]
+        if len(f) >= 3 and f[0] == kernel and f[1] == "kernel_source_hash":
+            recorded = f[2]
         if len(f) >= 3 and f[0] == kernel and f[1] == "traffic_bytes_per_launch":
-            return int(float(f[2])), "profiles/pmc_traffic.txt, kernel %s, recorded at source hash %s" % (kernel, recorded or "?")
-    return None, "profiles/pmc_traffic.txt has no record for %s" % kernel
+            value = int(float(f[2]))
+    if value is None:
+        return None, "profiles/pmc_traffic.txt has no record for %s" % kernel
+    now = kernel_source_hash(kernel)
+    if recorded != now:
+        return None, "profiles/pmc_traffic.txt: %s was recorded at kernel source %s, the source is now %s" % (kernel, recorded, now)
+    return value, "profiles/pmc_traffic.txt, kernel %s, recorded at kernel source %s" % (kernel, recorded)
 
 
 PROBE_SYMS = ["w4a16_copy_u4", "w4a16_read_u4", "w4a16_mfma_peak_f16"]

@@ -404,6 +404,51 @@ def test_deferred_norm_with_residual_and_norm_weight(dec, orc, t):
             cc.free(p_)
 
 
+def test_deferred_norm_residual_outlier_needs_and_gets_a_scaled_handover(dec, orc):
+    """A residual stream with elements around 1e5 (times a norm weight): norm_resid normalises in f32 first and stays
+    finite; the un-scaled f16 hand-over carries Inf, the hand-over with out_exp = 3 / in_exp = 3 gives the reference
+    sequence's result."""
+    t, hidden, n2, k1, group = 4, 640, 272, 512, 128
+    q1, s1, x = gen.make_linear(hidden, k1, group, t, seed=331)
+    q2, s2, _ = gen.make_linear(n2, hidden, group, 1, seed=332)
+    dec.upload_lin_g("no1", q1, s1, hidden, k1, group, False)
+    dec.upload_lin_g("no2", q2, s2, n2, hidden, group, False)
+    rng = np.random.default_rng(77)
+    resid0 = (rng.standard_normal((t, hidden)) * 3).astype(np.float32)
+    resid0[:, 5] = np.float32(1.0e5)
+    resid0[1, 77] = np.float32(-2.3e5)
+    nw = (1.0 + 0.3 * rng.standard_normal(hidden)).astype(np.float32)
+    nw[5] = np.float32(1.5)
+    ab = orc.gemm_lane(x, t, q1, s1, hidden, k1, group, False, 4)
+    _, _, _, ref_xn16 = orc.norm_resid(resid0, nw, ab)
+    want = orc.gemm_lane(ref_xn16, t, q2, s2, n2, hidden, group, False, 4)
+    assert np.all(np.isfinite(want))
+    cc = dec.cc
+    cap = ((hidden + 15) // 16) * 64
+    px, pw = cc.to_device(x), cc.to_device(nw)
+    pa, ps, py = cc.alloc(t * hidden * 2), cc.alloc(cap), cc.alloc(t * n2 * 4)
+    try:
+        for e, finite in ((0, False), (3, True)):
+            pr = cc.to_device(resid0)
+            cc.memset0(ps, cap)
+            n_st = dec.lin_forward_deferred_norm("no1", px, t, pa, out_f16=True, stats_out=ps, stat_rows=hidden, resid=pr,
+                                                 nw=pw, in_exp=0, out_exp=e)
+            a = _f16(cc.d2h(pa, (t, hidden), np.uint16))
+            assert bool(np.all(np.isfinite(a))) == finite
+            dec.lin_forward_deferred_norm("no2", pa, t, py, stats_in=ps, n_stats_in=n_st, in_cols=hidden, in_exp=e, out_exp=0)
+            got = cc.d2h(py, (t, n2), np.float32)
+            cc.free(pr)
+            if finite:
+                m = parity.compare(got, want)
+                say("  outlier residual, scaled hand-over: rel_l2", m["rel_l2"])
+                assert m["rel_l2"] < 1e-3
+            else:
+                assert not np.all(np.isfinite(got))
+    finally:
+        for p_ in (px, pw, pa, ps, py):
+            cc.free(p_)
+
+
 def _fused_oracle(orc, prefix, seeds, shapes, group, layers, x, threads):
     cur, sc = x, np.ones(x.shape[0], np.float32)
     for l in range(layers):
