@@ -51,8 +51,12 @@ static int pick_decode_shape(const w4a16_ctx* ctx, const W4Lin& L, size_t t, int
     // L1 — wider waves share them).  Narrow outputs: two row blocks x eight waves, so that the few blocks still bring
     // enough waves.
     const bool wide = L.row_blocks >= 1024;
-    const int rb_auto = wide ? (t <= 2 ? 1 : t <= 6 ? 2 : 4) : 2;
-    const int waves_auto = wide ? 4 : (t > 8 ? 4 : 8);
+    // a narrow output with a long k range (the 27B down projection, 320 row blocks x 136 k tiles) from seven tokens
+    // on: four row blocks per wave share the x loads, and the k slices across workgroups (decode_split) bring the
+    // workgroups back (t = 16: 21.6 -> 15.8 us, t = 12: 18.6 -> 14.9, t = 8: 14.2 -> 13.5; level at t = 6)
+    const bool long_k_narrow = !wide && L.k / 128 >= 64 && t >= 7;
+    const int rb_auto = wide ? (t <= 2 ? 1 : t <= 6 ? 2 : 4) : long_k_narrow ? 4 : 2;
+    const int waves_auto = wide ? 4 : (t > 8 || long_k_narrow ? 4 : 8);
     int rb = ctx->decode_rows_per_wave ? ctx->decode_rows_per_wave / 16 : rb_auto;
     if (rb != 1 && rb != 2 && rb != 4) return w4_fail(W4A16_ERR_ARG, "decode: rows_per_wave must be 16, 32 or 64");
     while (rb > 1 && L.row_blocks < (size_t)rb) rb >>= 1;
@@ -79,7 +83,7 @@ static int decode_split(w4a16_ctx* ctx, const W4Lin& L, size_t t, size_t blocks,
     int nks = 1;
     if (ctx->decode_ksplit > 0) {
         nks = ctx->decode_ksplit;
-    } else if (ctx->decode_ksplit == 0 && t <= 8 && blocks < (size_t)std::max(ctx->cu_count, 1) && kt_n >= 64) {
+    } else if (ctx->decode_ksplit == 0 && blocks < (size_t)std::max(ctx->cu_count, 1) && kt_n >= 64) {
         // a long k range over fewer workgroups than CUs (the 27B down projection: 160 blocks x 136 k tiles): slices
         // of about 16 k tiles, four waves each (measured 12.4 -> 11.8 us at t = 1, 13.3 -> 12.4 us at t = 4).  Shorter
         // k ranges lose more to the extra workgroups than they gain.
