@@ -247,18 +247,22 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     // so both are priced — (generations of workgroups) x (k tiles per slice) x (relative tile time) — and the cheaper
     // one runs (sweeps over the 27B shapes, t = 65..4096: within ~5 % of the better tile everywhere).
     const size_t tiles_n = (L.n + kW4PfBn - 1) / kW4PfBn, kt_n = L.k / 128, cus = (size_t)std::max(ctx->cu_count, 1);
-    auto slices_for = [&](size_t tiles, size_t slots) {
+    auto slices_for = [&](size_t tiles, size_t slots, size_t rows) {
         size_t nks = 1;
         if (ctx->prefill_ksplit > 0) {
             nks = (size_t)ctx->prefill_ksplit;
         } else if (ctx->prefill_ksplit == 0 && L.n % 4 == 0) {
             while (tiles * nks * 20 < slots * 9 && nks < 8) nks *= 2;  // until ~45 % of the slots (see below)
+            // a split launch of 64-row tiles whose slices are still long (the down projection, 136 k tiles): one more
+            // halving evens the workgroups out for less than the extra partial sums cost (t = 1024: 191 -> 181 us,
+            // t = 768: 169 -> 163 us); with 128-row tiles it does not pay (128 KiB of partial sums per workgroup)
+            if (rows == 64 && nks >= 2 && nks < 8 && kt_n / nks >= 64 && tiles * nks < 2 * slots) nks *= 2;
         }
         return std::max<size_t>(1, std::min(nks, kt_n / 4));
     };
     auto price = [&](size_t rows) {
         const size_t slots = cus * (rows == 64 ? 3 : 2), tiles = ((t + rows - 1) / rows) * tiles_n;
-        const size_t nks = slices_for(tiles, slots);
+        const size_t nks = slices_for(tiles, slots, rows);
         return (double)((tiles * nks + slots - 1) / slots) * (double)((kt_n + nks - 1) / nks) * (rows == 64 ? 0.85 : 1.0);
     };
     const size_t bm = ctx->prefill_tile_m ? (size_t)ctx->prefill_tile_m : (price(64) <= price(128) ? 64 : 128);
@@ -282,7 +286,7 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     // that cost more in partial-sum traffic than they gain; e.g. gate|up at t = 384 runs 141 us unsplit, 173 us in two
     // slices), each slice at least 4 k tiles.  Partials are f32 in a context-owned workspace, added in slice order by a
     // second launch (deterministic).
-    const size_t nks = slices_for(tiles_m * tiles_n, slots);
+    const size_t nks = slices_for(tiles_m * tiles_n, slots, bm);
     char sym[64];
     snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s%s", L.group, L.scale_bf16 ? "bf16" : "f16", bm == 64 ? "_m64" : "");
     const unsigned shmem = (unsigned)(2 * bm * kW4PfKs * 2);  // two stages of bm rows x PF_KS halves
