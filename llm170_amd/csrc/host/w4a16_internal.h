@@ -4,9 +4,11 @@
 
 #include <cstdarg>
 #include <cstdint>
+#include <array>
 #include <map>
 #include <string>
 #include <string_view>
+#include <tuple>
 #include <unordered_map>
 #include <vector>
 
@@ -79,6 +81,8 @@ struct w4a16_ctx {
     std::map<std::string, W4Experts, std::less<>> experts;
     W4MoeScratch moe;
     W4ChainScratch chain;
+    // prefill launch plans: (t, n, k, forced tile, forced slices) -> {tile rows, k slices, super-tile m, n, count}
+    std::map<std::tuple<size_t, size_t, size_t, int, int>, std::array<size_t, 5>> prefill_plans;
     int moe_block = 0, moe_waves = 0;  // 0 = automatic
     int moe_tiled = 0;                 // MFMA-tiled grouped kernel: 0 = automatic (long runs per expert), -1 = never, 1 = always
     int moe_act_kind = 0;              // activation of the expert FFN call in progress (W4A16_ACT_*)

@@ -6,6 +6,7 @@
 #include <chrono>
 #include <cmath>
 #include <cstring>
+#include <tuple>
 
 #include "w4a16_internal.h"
 
@@ -241,52 +242,101 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
         return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has a zero or non-finite scale (use the decode path)");
     if (t * L.k * 2 >= 0x80000000ull || L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
         return w4_fail(W4A16_ERR_SHAPE, "prefill: x or the tiled weights reach 2 GiB, beyond the buffer-descriptor range");
-    // Block tile 128 x 256 (two workgroups per CU) or 64 x 256 (three per CU, 64 accumulator registers).  The 64-row
-    // tile pads less, makes twice as many workgroups and loses about 15 % per row to unpacking each weight for half as
-    // many rows; which one finishes first is mostly a matter of how the workgroups divide into the slots of the chip,
-    // so both are priced — (generations of workgroups) x (k tiles per slice) x (relative tile time) — and the cheaper
-    // one runs (sweeps over the 27B shapes, t = 65..4096: within ~5 % of the better tile everywhere).
+    // Block tile 128 x 256 (two workgroups per CU) or 64 x 256 (three per CU, 64 accumulator registers), the k range
+    // whole or cut into 2, 3, 4, 6 or 8 slices (split-K: f32 partials in a context-owned workspace, added in slice
+    // order by a second launch — deterministic), and the super-tile shape: every combination is priced and the cheapest
+    // runs.  The plan depends on (t, n, k) only and is kept per shape.
     const size_t tiles_n = (L.n + kW4PfBn - 1) / kW4PfBn, kt_n = L.k / 128, cus = (size_t)std::max(ctx->cu_count, 1);
-    auto slices_for = [&](size_t tiles, size_t slots, size_t rows) {
-        size_t nks = 1;
-        if (ctx->prefill_ksplit > 0) {
-            nks = (size_t)ctx->prefill_ksplit;
-        } else if (ctx->prefill_ksplit == 0 && L.n % 4 == 0) {
-            while (tiles * nks * 20 < slots * 9 && nks < 8) nks *= 2;  // until ~45 % of the slots (see below)
-            // a split launch of 64-row tiles whose slices are still long (the down projection, 136 k tiles): one more
-            // halving evens the workgroups out for less than the extra partial sums cost (t = 1024: 191 -> 181 us,
-            // t = 768: 169 -> 163 us); with 128-row tiles it does not pay (128 KiB of partial sums per workgroup)
-            if (rows == 64 && nks >= 2 && nks < 8 && kt_n / nks >= 64 && tiles * nks < 2 * slots) nks *= 2;
+    // Super-tile shape for a grid of tiles_m x tiles_n block tiles: sup_m <= 8 along m, sup_n in {8, 4, 2, 1} along n.
+    // Super-tiles are dealt round-robin to the 8 XCDs (m fastest), so every candidate is priced by the block tiles its
+    // busiest XCD ends up with — counted exactly, partial super-tiles at the edges included — and the shape with the
+    // lightest busiest XCD wins, the larger one on ties for L2 reuse.  (A fixed 8 along m left 10 tile rows as 8 + 2:
+    // the XCDs that drew the 2-row super-tiles idled, 298 against 227 us on the down projection at t = 1280.)
+    struct Super {
+        size_t sup_m, sup_n, supers, load;
+    };
+    auto super_for = [&](size_t tiles_m) {
+        Super best{std::min<size_t>(8, tiles_m), 8, 0, ~(size_t)0};
+        for (size_t cm = std::min<size_t>(8, tiles_m); cm >= 1; cm--) {
+            for (size_t cn : {8, 4, 2, 1}) {
+                const size_t sm = (tiles_m + cm - 1) / cm, sn = (tiles_n + cn - 1) / cn, sp = sm * sn;
+                size_t per_xcd[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                for (size_t sidx = 0; sidx < sp; sidx++)
+                    per_xcd[sidx & 7] += std::min(cm, tiles_m - (sidx % sm) * cm) * std::min(cn, tiles_n - (sidx / sm) * cn);
+                const size_t load = *std::max_element(per_xcd, per_xcd + 8);
+                if (load < best.load || (load == best.load && cm * cn > best.sup_m * best.sup_n)) best = Super{cm, cn, sp, load};
+            }
         }
-        return std::max<size_t>(1, std::min(nks, kt_n / 4));
+        return best;
     };
-    auto price = [&](size_t rows) {
-        const size_t slots = cus * (rows == 64 ? 3 : 2), tiles = ((t + rows - 1) / rows) * tiles_n;
-        const size_t nks = slices_for(tiles, slots, rows);
-        return (double)((tiles * nks + slots - 1) / slots) * (double)((kt_n + nks - 1) / nks) * (rows == 64 ? 0.85 : 1.0);
+    // Price of a launch in microseconds, from measurements on MI355X (grids of exactly 256 x j workgroups of each tile,
+    // k = 17408 and 5120).  A CU holds c workgroups at once (3 of the 64-row tile, 2 of the 128-row tile); j workgroups
+    // per CU (of the busiest XCD) run as floor(j / c) full generations, `full` microseconds per k tile each, and a last
+    // partial one whose cost depends on how many workgroups share the CU — a workgroup alone runs nearly twice as fast
+    // as one of a full set (the chip is power-limited under this kernel), so the cost of a partial generation starts at
+    // more than half a full one and grows from there.  Plus a fixed cost per generation (first loads, epilogue), and for a
+    // split launch the second launch and the partial sums written and read back.  The constants started from those
+    // measurements and were then fitted to a sweep of tile x slices over 108 (n, k, t) shapes (nine linears, t = 128
+    // to 4096), minimising the time lost against the best choice of the sweep: 0.8 % lost on average, 9 % at worst,
+    // where the earlier rule (generations x slice length x a tile factor, slices by doubling) lost 3 % and 22 %; fitted
+    // on four of the linears only it lost 0.9 % / 11 % on the other five.
+    auto us_per_k_tile = [](size_t rows, double per_cu) {
+        static const double at[7] = {0.0, 0.5, 1.0, 1.5, 2.0, 2.5, 3.0};
+        static const double part64[7] = {1.0, 1.006, 1.595, 1.738, 1.95, 2.552, 2.903}, part128[5] = {1.5, 1.6, 2.416, 2.9, 3.37};
+        const double c = rows == 64 ? 3.0 : 2.0, full = rows == 64 ? 2.745 : 3.497;
+        const double* part = rows == 64 ? part64 : part128;
+        const double gens = std::floor(per_cu / c), rem = per_cu - gens * c;
+        double us = gens * full;
+        if (rem > 1e-9) {
+            const int last = rows == 64 ? 6 : 4;
+            int i = 1;
+            while (i < last && rem > at[i]) i++;
+            us += part[i - 1] + (part[i] - part[i - 1]) * (rem - at[i - 1]) / (at[i] - at[i - 1]);
+        }
+        return us;
     };
-    const size_t bm = ctx->prefill_tile_m ? (size_t)ctx->prefill_tile_m : (price(64) <= price(128) ? 64 : 128);
-    const size_t slots = cus * (bm == 64 ? 3 : 2);
-    const size_t tiles_m = (t + bm - 1) / bm;
-    // Super-tile shape: up to 8 tiles along m; along n the width in {8, 4, 2, 1} that leaves the busiest XCD with the
-    // fewest tiles (super-tiles are dealt round-robin to the 8 XCDs), the wider one on ties for L2 reuse.
-    const size_t sup_m = std::min<size_t>(8, tiles_m), sm_n = (tiles_m + sup_m - 1) / sup_m;
-    size_t sup_n = 8, supers = 0, best_load = ~(size_t)0;
-    for (size_t cand : {8, 4, 2, 1}) {
-        const size_t sp = sm_n * ((tiles_n + cand - 1) / cand), load = ((sp + 7) / 8) * sup_m * cand;
-        if (load < best_load) {
-            best_load = load;
-            sup_n = cand;
-            supers = sp;
+    struct Plan {
+        size_t bm, nks;
+        Super sup;
+    };
+    auto make_plan = [&]() {
+        Plan best{128, 1, Super{1, 1, 0, 0}};
+        double best_us = 1e30;
+        for (size_t rows : {(size_t)128, (size_t)64}) {
+            if (ctx->prefill_tile_m && (size_t)ctx->prefill_tile_m != rows) continue;
+            const size_t tiles_m = (t + rows - 1) / rows;
+            const Super sup = super_for(tiles_m);
+            const size_t forced = ctx->prefill_ksplit > 0 ? std::max<size_t>(1, std::min<size_t>((size_t)ctx->prefill_ksplit, kt_n / 4)) : 0;
+            for (size_t cand : {1, 2, 3, 4, 6, 8}) {
+                const size_t nks = forced ? forced : cand;  // a pinned slice count is the only candidate
+                if (forced && cand != 1) break;
+                if (ctx->prefill_ksplit < 0 && nks != 1) continue;
+                if (!forced && nks > 1 && (L.n % 4 != 0 || nks > kt_n / 4)) continue;
+                const double per_cu = (double)(sup.load * nks) * 8.0 / (double)cus;  // of the busiest XCD
+                const double gens = std::ceil(per_cu / (rows == 64 ? 3.0 : 2.0));
+                double us = (double)((kt_n + nks - 1) / nks) * us_per_k_tile(rows, per_cu) + 5.7 * gens;
+                if (nks > 1) us += 6.0 + (double)nks * (double)t * (double)L.n * 8.0 / 9.76e6;
+                if (us < best_us) {
+                    best_us = us;
+                    best = Plan{rows, nks, sup};
+                }
+            }
+        }
+        return best;
+    };
+    Plan plan;
+    {
+        const auto key = std::make_tuple(t, L.n, L.k, ctx->prefill_tile_m, ctx->prefill_ksplit);
+        const auto hit = ctx->prefill_plans.find(key);
+        if (hit != ctx->prefill_plans.end()) {
+            plan = Plan{hit->second[0], hit->second[1], Super{hit->second[2], hit->second[3], hit->second[4], 0}};
+        } else {
+            plan = make_plan();
+            ctx->prefill_plans[key] = {plan.bm, plan.nks, plan.sup.sup_m, plan.sup.sup_n, plan.sup.supers};
         }
     }
+    const size_t bm = plan.bm, nks = plan.nks, sup_m = plan.sup.sup_m, sup_n = plan.sup.sup_n, supers = plan.sup.supers;
     const size_t grid = ((supers + 7) / 8) * (sup_m * sup_n) * 8;
-    // Split-K when the tile grid alone leaves much of the chip idle: k slices are doubled until the launch has about
-    // 45 % as many workgroups as the chip holds at once (sweeps over the 27B shapes at t = 65..1024: more slices than
-    // that cost more in partial-sum traffic than they gain; e.g. gate|up at t = 384 runs 141 us unsplit, 173 us in two
-    // slices), each slice at least 4 k tiles.  Partials are f32 in a context-owned workspace, added in slice order by a
-    // second launch (deterministic).
-    const size_t nks = slices_for(tiles_m * tiles_n, slots, bm);
     char sym[64];
     snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s%s", L.group, L.scale_bf16 ? "bf16" : "f16", bm == 64 ? "_m64" : "");
     const unsigned shmem = (unsigned)(2 * bm * kW4PfKs * 2);  // two stages of bm rows x PF_KS halves
