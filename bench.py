@@ -259,6 +259,57 @@ def bench_chain(dec, gen, ops, args):
             "normalisation_launches_kept": kept, "normalisations_deferred": deferred, "per_gemm": per_gemm}
 
 
+PLAN_SWEEP_SHAPES = [(34816, 5120), (5120, 17408)]
+PLAN_SWEEP_T = (512, 1024, 4096)
+
+
+def plan_sweep(out_path):
+    """Times every (block tile, k slices) the prefill planner can choose at the layer shapes of the benchmark and writes
+    the table the planner test reads (profiles/prefill_plan_sweep.md): per shape every candidate's time, the fastest, and
+    what the planner picks with everything automatic."""
+    from llm170_amd import gen, ops
+    from llm170_amd import build as pkg_build
+    pkg_build.ensure_built()
+    dec = ops.W4a16Dec()
+    cc = dec.cc
+    g = 128
+    lines = ["# Prefill launch plans: every (tile, k slices) timed at the layer shapes", "",
+             "Command: `python bench.py --plan-sweep profiles/prefill_plan_sweep.md` (one MI355X; source hash %s)." % pkg_build.built_hash(),
+             "Each entry: best of 3 timed regions of 12 launches after 3 warm-up launches, HIP events on the launch stream,",
+             "f16 output, two to four weight copies rotated.  `plan` marks what `w4a16_plan_prefill` picks with every",
+             "setting automatic; `best` the fastest row of the shape.  tests/test_plan_cpu.py requires the planner's",
+             "pick to be a row within 1 % of the best.", "",
+             "| n | k | t | tile rows | k slices | us | note |", "|---|---|---|---|---|---|---|"]
+    for (n, k) in PLAN_SWEEP_SHAPES:
+        names, _ = make_copies(dec, gen, n, k, g, 2 if n > 8192 else 4, "ps%d_%d" % (n, k))
+        xd = cc.to_device(gen.normal_f16(3, (max(PLAN_SWEEP_T), k)))
+        yd = cc.alloc(max(PLAN_SWEEP_T) * n * 2)
+        time_forward(dec, names, xd, yd, max(PLAN_SWEEP_T), 30, 0, ops.PATH_PREFILL)
+        for t in PLAN_SWEEP_T:
+            rows = []
+            for tile in (64, 128):
+                for ks in (1, 2, 3, 4, 6, 8):
+                    if ks > 1 and ks > (k // 128) // 4:
+                        continue
+                    dec.set_prefill_tile(tile)
+                    dec.set_prefill_ksplit(-1 if ks == 1 else ks)
+                    us = min(time_forward(dec, names, xd, yd, t, 12, 3, ops.PATH_PREFILL, out_f16=True)[0] for _ in range(3)) * 1e3
+                    rows.append((tile, ks, us))
+            dec.set_prefill_tile(0)
+            dec.set_prefill_ksplit(0)
+            plan = ops.plan_prefill(t, n, k, cu_count=256)
+            best = min(r[2] for r in rows)
+            for tile, ks, us in rows:
+                note = " ".join(w for w, on in (("best", us == best), ("plan", (tile, ks) == (plan["tile_rows"], plan["k_slices"]))) if on)
+                lines.append("| %d | %d | %d | %d | %d | %.2f | %s |" % (n, k, t, tile, ks, us, note))
+            print("plan sweep", n, k, t, "best %.2f us" % best, "plan", plan["tile_rows"], plan["k_slices"], flush=True)
+        cc.free(xd)
+        cc.free(yd)
+    with open(out_path, "w") as fh:
+        fh.write("\n".join(lines) + "\n")
+    cc.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -268,7 +319,11 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="time the layer chain with eager launches only")
+    ap.add_argument("--plan-sweep", metavar="PATH", help="time every prefill launch plan at the layer shapes and write the table to PATH, nothing else")
     args = ap.parse_args()
+    if args.plan_sweep:
+        plan_sweep(args.plan_sweep)
+        return
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the W4A16 linear path has no collective); "
               "--gpus %d is not supported" % args.gpus, file=sys.stderr)

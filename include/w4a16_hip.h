@@ -39,7 +39,8 @@ enum {
     W4A16_ERR_UNSUPPORTED = 10003, /* group / scale dtype combination has no kernel (gptq4.rs:60-70)        */
     W4A16_ERR_NOT_FOUND = 10004,   /* linear name not registered (w4a16_dec/kernels/gemv.rs:10-13)          */
     W4A16_ERR_ARG = 10005,         /* null pointer, zero size, bad enum                                     */
-    W4A16_ERR_ASSET = 10006        /* code object file missing or unreadable (assets.rs:336-346)            */
+    W4A16_ERR_ASSET = 10006,       /* code object file missing or unreadable (assets.rs:336-346)            */
+    W4A16_ERR_STALE_GRAPH = 10007  /* a scratch buffer the graph's nodes address was replaced (buffers.rs:6-31) */
 };
 
 /* Message of the last failing call on this thread ("" if none). */
@@ -101,7 +102,13 @@ void w4a16_event_destroy(w4a16_ctx* ctx, w4a16_event* ev);
  * have to grow return W4A16_ERR_ARG (and invalidate nothing) — run the sequence once before capturing it, as the
  * reference does (warm_for_capture, w4a16_dec/graphs.rs:55).  w4a16_capture_end ends the capture, instantiates and
  * uploads the graph.  A graph replays the recorded launches with the recorded arguments: same buffers, same shapes.
- * Replays are ordered on the launch stream like any other launch.  w4a16_graph_destroy waits for the launch stream. */
+ * Replays are ordered on the launch stream like any other launch.  w4a16_graph_destroy waits for the launch stream.
+ * The recorded arguments include addresses of scratch buffers the context owns (split-K partials and tickets, the
+ * expert FFN's and the chain's intermediates).  A later eager call that needs one of them LARGER (more rows, a wider
+ * linear, more experts) frees it and allocates a new one; every graph captured before that is stale from then on and
+ * w4a16_graph_launch refuses it with W4A16_ERR_STALE_GRAPH instead of replaying onto freed memory — destroy it and
+ * capture again (the reference invalidates its graphs on every scratch reallocation, w4a16_dec/buffers.rs:6-31).
+ * Calls that fit the buffers as they are never invalidate a graph. */
 int w4a16_capture_begin(w4a16_ctx* ctx);
 int w4a16_capture_end(w4a16_ctx* ctx, w4a16_graph** out);
 int w4a16_graph_launch(w4a16_ctx* ctx, w4a16_graph* graph);
@@ -164,6 +171,22 @@ enum {
 int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16,
                       int path);
 
+/* The launch plan w4a16_lin_forward would pick on the decode path (t = 1..16) for a linear of this shape on a GPU of
+ * `cu_count` compute units with every setting automatic — rows of the output per wave (16, 32 or 64), waves per
+ * workgroup, k slices across workgroups, dynamic LDS bytes — without a context or a GPU (sk_ksp, w4a16_dec/kernels/
+ * decode.rs:3-16, is the reference's rule of the same role).  A shape whose staged scales would pass the LDS of a CU is
+ * planned with fewer rows per wave or more k slices; W4A16_ERR_SHAPE only when nothing fits.  `glu` != 0 plans the gated
+ * kernel of w4a16_lin_forward_glu.  Out pointers may be NULL. */
+int w4a16_plan_decode(size_t n, size_t k, size_t group, size_t t, int cu_count, int glu, int* rows_per_wave,
+                      int* waves_per_block, int* k_slices, size_t* lds_bytes);
+/* The launch plan of the prefill path (W4A16_PATH_PREFILL) for t rows: out = {block tile rows (64 or 128), k slices,
+ * super-tile rows, super-tile columns, super-tile count}; `tile_rows` and `k_slices` pin a choice as
+ * w4a16_set_prefill_tile / w4a16_set_prefill_ksplit do (0 = automatic); *price_us (may be NULL) receives the model's
+ * estimate for the chosen plan.  Role of the reference's per-problem choice of thread-block shape
+ * (kernels/marlin.rs:94-213).  Needs neither a context nor a GPU. */
+int w4a16_plan_prefill(size_t t, size_t n, size_t k, int cu_count, int tile_rows, int k_slices, size_t out[5],
+                       double* price_us);
+
 /* w4a16_lin_forward for callers that cannot allocate.  NO COUNTERPART IN THE REFERENCE: it exists for code under HIP graph
  * capture, tight serving loops and harnesses that forbid hipMalloc.  w4a16_lin_forward's decode launch, when it splits k
  * across workgroups (the 27B down projection does), parks partial tiles and tickets in a workspace that the context
@@ -173,9 +196,11 @@ int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t
  * with a tiled copy.  A launch whose split needs more than the array holds — workgroups x row blocks per wave x 1 KiB x
  * k slices > w4a16_noalloc_workspace_bytes(), or more than 16384 workgroups per slice — is refused with W4A16_ERR_SHAPE
  * and a message that gives both sizes.  Same results, bit for bit, as w4a16_lin_forward(..., W4A16_PATH_DECODE) under
- * the same w4a16_set_decode_* settings.  Every context on a GPU shares that GPU's array: two calls that overlap on
- * one GPU (two contexts, or one call still running when the next is issued on another stream) race; calls on one
- * launch stream are ordered and safe. */
+ * the same w4a16_set_decode_* settings.  A GPU has ONE such array.  The first context that calls this entry point on a
+ * GPU owns the array until that context is destroyed; the call from any other context on that GPU is refused with
+ * W4A16_ERR_ARG (two contexts sharing the tickets would sum each other's partial tiles).  Calls of the owning context
+ * are ordered on its launch stream and safe; the array keeps the last call's contents between calls (the tickets are
+ * left at zero by every launch). */
 int w4a16_lin_forward_noalloc(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16);
 size_t w4a16_noalloc_workspace_bytes(void);
 
@@ -227,8 +252,15 @@ int w4a16_lin_forward_glu_deferred_norm(w4a16_ctx* ctx, const char* name, uint64
 /* Both with a power-of-two factor on each hand-over, which lifts the range precondition above when the exponents come
  * from a bound on the values: x_dev holds the true activations times 2^-in_exp and y_dev receives the true output
  * times 2^-out_exp (for the gated form: the true silu(g)*u times 2^-out_exp).  The statistics, the residual stream and
- * the norm weight see true values.  Both factors are exact in f32, so wherever the un-scaled hand-over stays inside
- * the normal f16 range the results are the same numbers.  Exponents in -120..120; 0, 0 is the un-scaled call.
+ * the norm weight see true values.  Both factors are exact in f32, so an element gives the same number as in the
+ * un-scaled call exactly when BOTH its un-scaled value and its scaled value 2^-out_exp * v are normal f16 numbers
+ * (6.1e-5 <= |.| <= 65504).  A positive exponent trades range at the top for range at the bottom: an element with
+ * |v| < 2^(out_exp-14) is handed over as an f16 subnormal, with an absolute error of up to 2^(out_exp-25) instead of
+ * a relative one of 2^-11, and below 2^(out_exp-25) it becomes zero.  With exponents taken from the Cauchy-Schwarz
+ * bound below — orders of magnitude above the elements a trained layer produces — such elements are far below the
+ * row's root mean square and carry almost none of its energy (measured on the synthetic 64-layer chain: rel-L2 2e-4
+ * against the chain that normalises before rounding); parity on trained-weight activation statistics is not pinned by
+ * a test.  Exponents in -120..120; 0, 0 is the un-scaled call.
  * A bound for the output of a linear fed rows of unit root mean square: w4a16_lin_row_norm_max(W) * sqrt(k)
  * (norm_resid of the reference hands over normalised values and needs none of this, assets/norm.cu:4-48). */
 int w4a16_lin_forward_deferred_norm_scaled(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,

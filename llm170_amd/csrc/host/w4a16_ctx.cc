@@ -226,6 +226,7 @@ extern "C" void w4a16_ctx_destroy(w4a16_ctx* ctx) {
     }
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->stream2) (void)hipStreamSynchronize(ctx->stream2);
+    w4_noalloc_release(ctx);
     for (auto& a : ctx->allocs) (void)hipFree((void*)a.first);
     for (auto m : ctx->modules) (void)hipModuleUnload(m);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -379,6 +380,7 @@ extern "C" int w4a16_capture_end(w4a16_ctx* ctx, w4a16_graph** out) {
     if (!rc && g->nodes == 0) rc = w4_fail(W4A16_ERR_ARG, "capture_end: nothing was launched between begin and end");
     if (!rc) rc = w4_hip(hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0), "hipGraphInstantiate");
     if (!rc) rc = w4_hip(hipGraphUpload(g->exec, ctx->stream), "hipGraphUpload");
+    g->scratch_gen = ctx->scratch_gen;
     if (rc) {
         const std::string keep = w4_err_save();
         w4a16_graph_destroy(ctx, g);
@@ -392,6 +394,9 @@ extern "C" int w4a16_capture_end(w4a16_ctx* ctx, w4a16_graph** out) {
 extern "C" int w4a16_graph_launch(w4a16_ctx* ctx, w4a16_graph* g) {
     if (!ctx || !g || !g->exec) return w4_fail(W4A16_ERR_ARG, "graph_launch: null argument");
     if (ctx->capturing) return w4_fail(W4A16_ERR_ARG, "graph_launch while the launch stream is capturing");
+    if (g->scratch_gen != ctx->scratch_gen)
+        return w4_fail(W4A16_ERR_STALE_GRAPH, "graph_launch: a scratch buffer of the context was replaced by a larger one after this graph was captured (generation %llu, now %llu); its nodes hold the freed address: capture again",
+                       (unsigned long long)g->scratch_gen, (unsigned long long)ctx->scratch_gen);
     return w4_hip(hipGraphLaunch(g->exec, ctx->stream), "hipGraphLaunch");
 }
 

@@ -34,6 +34,7 @@ struct W4Experts {
     size_t n_exp = 0, h = 0, n_ff = 0, group = 0;
     int scale_bf16 = 0;
     size_t q13_stride = 0, s13_stride = 0, q2_stride = 0, s2_stride = 0;  // bytes per expert
+    bool scales_regular = true;  // same rule as W4Lin::scales_regular, over both arenas: the MFMA-tiled grouped kernels need it
 };
 
 // Scratch of the MoE FFN, grown on demand (reference: moe_msorted / moe_mexp / moe_mnpost / moe_mact / moe_mc2,
@@ -67,6 +68,7 @@ struct w4a16_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     size_t nodes = 0;
+    uint64_t scratch_gen = 0;  // w4a16_ctx::scratch_gen when the capture ended: the nodes hold addresses of that generation
 };
 
 struct w4a16_ctx {
@@ -100,6 +102,11 @@ struct w4a16_ctx {
     const char* last_symbol = "";  // kernel of the most recent launch (a key of `functions`: stable storage)
     uint64_t fixed_scratch = 0;  // this device's copy of the static scratch array of w4a16_noalloc.hip (device address)
     bool capturing = false;  // between w4a16_capture_begin and w4a16_capture_end: nothing may allocate, free or wait
+    // Counts the replacements of context-owned scratch buffers (w4_ensure).  A captured graph holds the addresses of
+    // the buffers of its time; once one of them has been replaced a replay would touch freed memory, so
+    // w4a16_graph_launch refuses a graph of an older generation (reference: graph_invalidate() on every scratch
+    // reallocation, w4a16_dec/buffers.rs:6-31).
+    uint64_t scratch_gen = 0;
 };
 
 // Launch constants that mirror #defines of the kernel sources (a CPU test reads both texts and compares the values):
@@ -126,12 +133,16 @@ int w4_launch(w4a16_ctx* ctx, const char* symbol, unsigned gx, unsigned gy, unsi
 
 int w4_register_lin(w4a16_ctx* ctx, const char* name, W4Lin& L);
 int w4_find_lin(w4a16_ctx* ctx, const char* name, W4Lin** out);
+// true when every scale of `count` u16 entries is finite, non-zero and (bf16) inside [2^-60, 2^60]: what a kernel that
+// carries the running unit s_prev / s_cur can take
+bool w4_scales_regular(const uint16_t* s, size_t count, int scale_bf16);
 int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes);
 int w4_dense_grouped(w4a16_ctx* ctx, const W4Lin& L, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16);
 int w4_lin_forward_fixed_ws(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16,
                             uint64_t ws, size_t ws_bytes, uint64_t tickets, size_t ticket_bytes);
 // per-device fixed scratch of the allocation-free entry point (w4a16_noalloc.hip)
 int w4_noalloc_init(w4a16_ctx* ctx);
+void w4_noalloc_release(w4a16_ctx* ctx);
 
 #define W4_TRY(expr)          \
     do {                      \

@@ -78,6 +78,10 @@ extern "C" int w4a16_upload_experts(w4a16_ctx* ctx, const char* name, size_t n_e
     E.n_ff = n_ff;
     E.group = group;
     E.scale_bf16 = scale_bf16 ? 1 : 0;
+    // the MFMA-tiled grouped kernels carry the running unit of the prefill kernel: they are taken only for arenas
+    // whose every scale that kernel can divide by (the streaming kernels only multiply by scales and take any)
+    E.scales_regular = w4_scales_regular(static_cast<const uint16_t*>(s13), s13_bytes / 2, scale_bf16) &&
+                       w4_scales_regular(static_cast<const uint16_t*>(s2), s2_bytes / 2, scale_bf16);
     int rc = tile_arena(ctx, q13, s13, n_experts, 2 * n_ff, h, group, &E.q13, &E.s13, &E.q13_stride, &E.s13_stride);
     if (!rc) rc = tile_arena(ctx, q2, s2, n_experts, h, n_ff, group, &E.q2, &E.s2, &E.q2_stride, &E.s2_stride);
     if (rc) {
@@ -190,7 +194,10 @@ int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes) {
     if (bytes <= *cap) return 0;
     if (ctx->capturing)
         return w4_fail(W4A16_ERR_ARG, "a scratch buffer would grow to %zu bytes while the launch stream is capturing: run the sequence once before the capture", bytes);
-    if (*buf) W4_TRY(w4a16_sync(ctx));  // earlier launches may still read the old buffer
+    if (*buf) {
+        W4_TRY(w4a16_sync(ctx));  // earlier launches may still read the old buffer
+        ctx->scratch_gen++;       // graphs captured so far hold its address: w4a16_graph_launch refuses them from now on
+    }
     (void)w4a16_free(ctx, *buf);
     *buf = 0;
     *cap = 0;
@@ -393,7 +400,9 @@ extern "C" int w4a16_moe_ffn_act(w4a16_ctx* ctx, const char* name, uint64_t x_de
     const size_t ns = t * top_k;
     // From a mean run of 96 slots per expert on, 64-slot segments are mostly full and the MFMA-tiled grouped kernel
     // (one segment x 256 columns per workgroup, x through LDS, 32x32x16 tiles) takes over from the streaming kernels.
-    const bool tiled = ctx->moe_tiled > 0 || (ctx->moe_tiled == 0 && ctx->moe_block == 0 && ns >= 96 * E->n_exp);
+    if (ctx->moe_tiled > 0 && !E->scales_regular)
+        return w4_fail(W4A16_ERR_UNSUPPORTED, "moe_ffn %s: the MFMA-tiled grouped kernels were requested (set_moe_tiled 1) but the experts hold a zero, non-finite or out-of-range scale; the streaming kernels serve them", name);
+    const bool tiled = ctx->moe_tiled > 0 || (ctx->moe_tiled == 0 && ctx->moe_block == 0 && E->scales_regular && ns >= 96 * E->n_exp);
     const size_t block = tiled ? 64 : pick_block(ctx, t, ns, E->n_exp, top_k);
     if (block != 1 && block != 4 && block != 16 && block != 32 && block != 48 && block != 64)
         return w4_fail(W4A16_ERR_ARG, "moe_ffn %s: segment size %zu not in {1,4,16,32,48,64}", name, block);

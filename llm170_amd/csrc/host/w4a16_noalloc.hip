@@ -8,6 +8,8 @@
 // process ends.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "w4a16_internal.h"
 
 #define W4_NOALLOC_WS_BYTES (8u << 20)       // partial tiles: workgroups x row blocks per wave x 1 KiB x k slices
@@ -19,6 +21,10 @@ static __device__ __align__(256) unsigned char scratch[W4_NOALLOC_WS_BYTES + W4_
 // Device address of each GPU's copy of the array.  In host code the array's name is only a handle for
 // hipGetSymbolAddress; every use of the memory goes through the address obtained here.
 static void* g_scratch_ptr[W4_NOALLOC_MAX_DEVICES];
+// The context that uses each GPU's array.  Partial tiles and tickets of two contexts would mix (either could draw the
+// last ticket early and sum the other's tiles), so the first caller on a GPU owns its array until it is destroyed.
+static w4a16_ctx* g_scratch_owner[W4_NOALLOC_MAX_DEVICES];
+static std::mutex g_owner_lock;
 
 extern "C" size_t w4a16_noalloc_workspace_bytes(void) { return W4_NOALLOC_WS_BYTES; }
 
@@ -42,10 +48,24 @@ int w4_noalloc_init(w4a16_ctx* ctx) {
     return 0;
 }
 
+// Called when a context is destroyed: its GPU's array is free for the next caller.
+void w4_noalloc_release(w4a16_ctx* ctx) {
+    if (ctx->device < 0 || ctx->device >= W4_NOALLOC_MAX_DEVICES) return;
+    std::lock_guard<std::mutex> hold(g_owner_lock);
+    if (g_scratch_owner[ctx->device] == ctx) g_scratch_owner[ctx->device] = nullptr;
+}
+
 extern "C" int w4a16_lin_forward_noalloc(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t,
                                          int out_f16) {
     if (!ctx || !name) return w4_fail(W4A16_ERR_ARG, "lin_forward_noalloc: null argument");
     if (!ctx->fixed_scratch) return w4_fail(W4A16_ERR_ARG, "lin_forward_noalloc: the fixed scratch was not set up");
+    {
+        std::lock_guard<std::mutex> hold(g_owner_lock);  // no allocation: a mutex and two pointer compares
+        w4a16_ctx*& owner = g_scratch_owner[ctx->device];
+        if (!owner) owner = ctx;
+        if (owner != ctx)
+            return w4_fail(W4A16_ERR_ARG, "lin_forward_noalloc: the fixed scratch of GPU %d is in use by another context (one context per GPU may use this entry point until it is destroyed)", ctx->device);
+    }
     const uint64_t ws = ctx->fixed_scratch, tickets = ctx->fixed_scratch + W4_NOALLOC_WS_BYTES;
     return w4_lin_forward_fixed_ws(ctx, name, x_dev, y_dev, t, out_f16, ws, W4_NOALLOC_WS_BYTES, tickets,
                                    W4_NOALLOC_TICKET_BYTES);

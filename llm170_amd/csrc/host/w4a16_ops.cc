@@ -41,60 +41,132 @@ static int launch_lane(w4a16_ctx* ctx, uint64_t q, uint64_t s, uint64_t x, uint6
     return w4_launch(ctx, sym, ceil_div(n, 4), ceil_div(t, kW4LaneTt), 256, 0, params);
 }
 
-// Launch shape of the row-block decode kernel.  Measured on MI355X at the 27B layer shapes (gate+up 5120x34816, down
-// 17408x5120, QKV 5120x7168, O 5120x5120): two row blocks per wave with eight waves per block (in-block split-K by 8)
-// is best or within 1 % of best for 2 <= t <= 8 on every shape and for t = 1 on the narrow outputs; a single token on
-// a wide output runs best with one row block per wave and four waves (5.5 against 5.3 TB/s on gate+up); for 9..16
-// token rows on wide outputs four row blocks per wave halve the x operand traffic.
-static int pick_decode_shape(const w4a16_ctx* ctx, const W4Lin& L, size_t t, int* rb_out, int* waves_out) {
-    // Measured on the 27B shapes.  Wide outputs (>= 1024 row blocks): four waves per block; one row block per wave for
-    // one or two tokens, two up to six, four beyond (the more tokens, the more x bytes a weight byte drags through the
-    // L1 — wider waves share them).  Narrow outputs: two row blocks x eight waves, so that the few blocks still bring
-    // enough waves.
-    const bool wide = L.row_blocks >= 1024;
-    // a narrow output with a long k range (the 27B down projection, 320 row blocks x 136 k tiles) from seven tokens
-    // on: four row blocks per wave share the x loads, and the k slices across workgroups (decode_split) bring the
-    // workgroups back (t = 16: 21.6 -> 15.8 us, t = 12: 18.6 -> 14.9, t = 8: 14.2 -> 13.5; level at t = 6)
-    const bool long_k_narrow = !wide && L.k / 128 >= 64 && t >= 7;
-    const int rb_auto = wide ? (t <= 2 ? 1 : t <= 6 ? 2 : 4) : long_k_narrow ? 4 : 2;
-    const int waves_auto = wide ? 4 : (t > 8 || long_k_narrow ? 4 : 8);
-    int rb = ctx->decode_rows_per_wave ? ctx->decode_rows_per_wave / 16 : rb_auto;
-    if (rb != 1 && rb != 2 && rb != 4) return w4_fail(W4A16_ERR_ARG, "decode: rows_per_wave must be 16, 32 or 64");
-    while (rb > 1 && L.row_blocks < (size_t)rb) rb >>= 1;
-    const int kt_n = (int)(L.k / 128);
-    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : waves_auto;
-    waves = std::max(1, std::min(std::min(waves, 8), kt_n));
-    *rb_out = rb;
-    *waves_out = waves;
+// Launch plan of the row-block decode kernel: a pure function of the linear's shape, the row count, the CU count and
+// the pinned settings, so that a CPU test can ask for it (w4a16_plan_decode).
+//
+// Shape, measured on MI355X at the 27B layer shapes (gate+up 5120x34816, down 17408x5120, QKV 5120x7168, O 5120x5120).
+// Wide outputs (>= 1024 row blocks): four waves per block; one row block per wave for one or two tokens (5.5 against
+// 5.3 TB/s on gate+up), two up to six, four beyond (the more tokens, the more x bytes a weight byte drags through the
+// L1 — wider waves share them).  Narrow outputs: two row blocks x eight waves, so that the few blocks still bring
+// enough waves; a narrow output with a long k range (the 27B down projection, 320 row blocks x 136 k tiles) from seven
+// tokens on runs four row blocks per wave, which share the x loads, with the k slices across workgroups bringing the
+// workgroups back (t = 16: 21.6 -> 15.8 us, t = 12: 18.6 -> 14.9, t = 8: 14.2 -> 13.5; level at t = 6).
+// k slices across workgroups (one launch; partial tiles and tickets in a workspace): only for a long k range over
+// fewer workgroups than CUs (the 27B down projection: 160 blocks x 136 k tiles): slices of about 16 k tiles, four waves
+// each (measured 12.4 -> 11.8 us at t = 1, 13.3 -> 12.4 us at t = 4).  Shorter k ranges lose more to the extra
+// workgroups than they gain.
+// LDS: the waves' staged scales grow with the k tiles per wave (kernels/decode.hip).  A plan that would pass the 160 KiB
+// of a CU is shrunk — automatic row blocks per wave are halved first (keeps one launch without tickets), then the k
+// range is cut into more slices — and only a shape that fits in no such plan is refused.
+struct DecodePlanIn {
+    size_t row_blocks = 0, k = 0, group = 128, t = 1;
+    int cu_count = 256;
+    int rows_per_wave = 0, waves_per_block = 0, ksplit = 0;  // pinned settings of the context, 0 = automatic
+    bool glu = false;                                        // gated kernel: two row blocks per wave by construction
+    unsigned extra_lds = 0;                                  // staging area of the input statistics
+};
+struct DecodePlan {
+    int rb = 0, waves = 0, nks = 1, kt_per_slice = 0, kt_per_wave = 0;
+    size_t blocks = 0;
+    unsigned shmem = 0;
+};
+
+// LDS bytes of one wave's staged scales (kernels/decode.hip, AUX_PW)
+static unsigned decode_scale_lds(size_t group, int rb, int kt_per_wave) {
+    return ((unsigned)(rb * kt_per_wave * (128 / (int)group) * 32) + 1023u) / 1024u * 1024u;
+}
+
+static int plan_decode(const DecodePlanIn& in, DecodePlan* out) {
+    const int kt_n = (int)(in.k / 128);
+    if (kt_n <= 0 || in.row_blocks == 0) return w4_fail(W4A16_ERR_SHAPE, "decode: empty linear");
+    const bool wide = in.row_blocks >= 1024;
+    const bool long_k_narrow = !wide && kt_n >= 64 && in.t >= 7;
+    int rb;
+    bool rb_auto = false;
+    if (in.glu) {
+        rb = 2;
+    } else if (in.rows_per_wave) {
+        rb = in.rows_per_wave / 16;
+        if (rb != 1 && rb != 2 && rb != 4) return w4_fail(W4A16_ERR_ARG, "decode: rows_per_wave must be 16, 32 or 64");
+    } else {
+        rb = wide ? (in.t <= 2 ? 1 : in.t <= 6 ? 2 : 4) : long_k_narrow ? 4 : 2;
+        rb_auto = true;
+    }
+    while (!in.glu && rb > 1 && in.row_blocks < (size_t)rb) rb >>= 1;
+    const int waves_auto = in.glu ? (in.t > 8 || wide ? 4 : 8) : wide ? 4 : (in.t > 8 || long_k_narrow ? 4 : 8);
+    const int waves_want = std::max(1, std::min(std::min(in.waves_per_block ? in.waves_per_block : waves_auto, 8), kt_n));
+    int nks_want = 1;
+    bool nks_auto = false;
+    int waves_cap = 8;
+    if (in.ksplit > 0) {
+        nks_want = in.ksplit;
+    } else if (in.ksplit == 0) {
+        nks_auto = true;
+        const size_t blocks = in.glu ? in.row_blocks / 2 : (in.row_blocks + (size_t)rb - 1) / (size_t)rb;
+        if (blocks < (size_t)std::max(in.cu_count, 1) && kt_n >= 64) {
+            nks_want = std::min(kW4DecodeMaxKsplit, kt_n / 16);
+            waves_cap = 4;
+        }
+    }
+    for (;;) {
+        DecodePlan P;
+        P.rb = rb;
+        P.blocks = in.glu ? in.row_blocks / 2 : (in.row_blocks + (size_t)rb - 1) / (size_t)rb;
+        P.nks = std::max(1, std::min(nks_want, kt_n / 2));
+        P.waves = std::min(waves_want, waves_cap);
+        if (P.nks > 1) P.waves = std::max(1, std::min(P.waves, kt_n / P.nks));
+        P.kt_per_slice = (kt_n + P.nks - 1) / P.nks;
+        P.kt_per_wave = (P.kt_per_slice + P.waves - 1) / P.waves;
+        // the split-K partial tiles [waves][rb][1 KiB]; then per wave the scales of its whole k slice (rb x tiles per
+        // wave x groups per tile x 32 bytes, in whole 1 KiB DMA instructions); then the statistics staging area
+        P.shmem = (unsigned)(P.waves * rb * 1024) + (unsigned)P.waves * decode_scale_lds(in.group, rb, P.kt_per_wave) + in.extra_lds;
+        if (P.shmem <= 160u * 1024u) {
+            *out = P;
+            return 0;
+        }
+        if (rb_auto && rb > 1) {
+            rb >>= 1;
+        } else if (nks_auto && nks_want < kW4DecodeMaxKsplit && nks_want * 2 <= kt_n / 2) {
+            nks_want = std::max(2, nks_want * 2);
+        } else {
+            return w4_fail(W4A16_ERR_SHAPE, "decode: k=%zu at group %zu needs %u bytes of LDS for the staged scales (limit 160 KiB) in every launch shape the settings allow: leave rows per wave and k slices automatic, or split k over more workgroups (w4a16_set_decode_ksplit)",
+                           in.k, in.group, P.shmem);
+        }
+    }
+}
+
+extern "C" int w4a16_plan_decode(size_t n, size_t k, size_t group, size_t t, int cu_count, int glu, int* rows_per_wave,
+                                 int* waves_per_block, int* k_slices, size_t* lds_bytes) {
+    if ((group != 128 && group != 32) || n == 0 || k == 0 || k % 128 != 0 || t == 0 || t > 16 || cu_count <= 0)
+        return w4_fail(W4A16_ERR_SHAPE, "plan_decode: n=%zu k=%zu group=%zu t=%zu cus=%d", n, k, group, t, cu_count);
+    if (glu && n % 32 != 0) return w4_fail(W4A16_ERR_SHAPE, "plan_decode: a gated linear needs n %% 32 == 0");
+    DecodePlanIn in;
+    in.row_blocks = (n + 15) / 16;
+    in.k = k;
+    in.group = group;
+    in.t = t;
+    in.cu_count = cu_count;
+    in.glu = glu != 0;
+    DecodePlan P;
+    W4_TRY(plan_decode(in, &P));
+    if (rows_per_wave) *rows_per_wave = P.rb * 16;
+    if (waves_per_block) *waves_per_block = P.waves;
+    if (k_slices) *k_slices = P.nks;
+    if (lds_bytes) *lds_bytes = P.shmem;
     return 0;
 }
 
-// k slices across workgroups for a decode launch of `blocks` workgroups, and the workspace they need: partial tiles and
-// one ticket per workgroup of a slice.  The tickets are zero when (re)allocated and every launch leaves them zero.
-// With `fixed` the workspace is the caller's (a buffer of stated size that cannot grow): a launch that needs more is
-// refused, nothing is allocated.
+// Workspace of a launch split over k across workgroups: partial tiles and one ticket per workgroup of a slice.  The
+// tickets are zero when (re)allocated and every launch leaves them zero.  With `fixed` the workspace is the caller's (a
+// buffer of stated size that cannot grow): a launch that needs more is refused, nothing is allocated.
 struct DecodeWorkspace {
     uint64_t ws = 0, tickets = 0;
     size_t ws_cap = 0, tickets_cap = 0;  // bytes
 };
 
-static int decode_split(w4a16_ctx* ctx, const W4Lin& L, size_t t, size_t blocks, int rb, int* waves, int* nks_out,
-                        DecodeWorkspace* out, const DecodeWorkspace* fixed) {
-    const int kt_n = (int)(L.k / 128);
-    int nks = 1;
-    if (ctx->decode_ksplit > 0) {
-        nks = ctx->decode_ksplit;
-    } else if (ctx->decode_ksplit == 0 && blocks < (size_t)std::max(ctx->cu_count, 1) && kt_n >= 64) {
-        // a long k range over fewer workgroups than CUs (the 27B down projection: 160 blocks x 136 k tiles): slices
-        // of about 16 k tiles, four waves each (measured 12.4 -> 11.8 us at t = 1, 13.3 -> 12.4 us at t = 4).  Shorter
-        // k ranges lose more to the extra workgroups than they gain.
-        nks = std::min(kW4DecodeMaxKsplit, kt_n / 16);
-        *waves = std::min(*waves, 4);
-    }
-    nks = std::max(1, std::min(nks, kt_n / 2));
-    if (nks > 1) {
-        *waves = std::max(1, std::min(*waves, kt_n / nks));
-        const size_t ws_need = blocks * (size_t)rb * 1024 * (size_t)nks, tk_need = blocks * 4;
+static int decode_workspace(w4a16_ctx* ctx, const DecodePlan& P, DecodeWorkspace* out, const DecodeWorkspace* fixed) {
+    if (P.nks > 1) {
+        const size_t ws_need = P.blocks * (size_t)P.rb * 1024 * (size_t)P.nks, tk_need = P.blocks * 4;
         if (fixed) {
             if (ws_need > fixed->ws_cap || tk_need > fixed->tickets_cap)
                 return w4_fail(W4A16_ERR_SHAPE, "decode: the split over k needs %zu bytes of partial tiles and %zu of tickets, the fixed workspace holds %zu and %zu",
@@ -113,7 +185,6 @@ static int decode_split(w4a16_ctx* ctx, const W4Lin& L, size_t t, size_t blocks,
         out->ws = ctx->decode_ws;
         out->tickets = ctx->decode_tickets;
     }
-    *nks_out = nks;
     return 0;
 }
 
@@ -132,11 +203,6 @@ struct DecodeNorm {
     int act = 0;             // gated projection only: W4A16_ACT_*
     int in_exp = 0, out_exp = 0;  // x holds its true value times 2^-in_exp, y receives its true value times 2^-out_exp
 };
-
-// LDS bytes of one wave's staged scales (kernels/decode.hip, AUX_PW)
-static unsigned decode_scale_lds(const W4Lin& L, int rb, int kt_per_wave) {
-    return ((unsigned)(rb * kt_per_wave * (128 / (int)L.group) * 32) + 1023u) / 1024u * 1024u;
-}
 
 static unsigned decode_stats_lds(const DecodeNorm& nm) {
     return nm.stats_in ? (unsigned)std::min<size_t>((nm.n_stats_in + 63) / 64, 8) * 1024u : 0u;
@@ -158,27 +224,35 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
                          DecodeNorm* norm = nullptr, const DecodeWorkspace* fixed_ws = nullptr) {
     if (t == 0 || t > 16) return w4_fail(W4A16_ERR_SHAPE, "decode: t=%zu outside 1..16", t);
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode: linear has no tiled copy (needs k %% 128 == 0)");
-    int rb = 0, waves = 0;
-    W4_TRY(pick_decode_shape(ctx, L, t, &rb, &waves));
     if (L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
         return w4_fail(W4A16_ERR_SHAPE, "decode: tiled weights of 2 GiB or more exceed the buffer-descriptor range");
+    DecodeNorm none;
+    DecodeNorm& nm = norm ? *norm : none;
+    W4_TRY(check_decode_norm(L, t, nm));
+    DecodePlanIn in;
+    in.row_blocks = L.row_blocks;
+    in.k = L.k;
+    in.group = L.group;
+    in.t = t;
+    in.cu_count = ctx->cu_count;
+    in.rows_per_wave = ctx->decode_rows_per_wave;
+    in.waves_per_block = ctx->decode_waves_per_block;
+    in.ksplit = ctx->decode_ksplit;
+    in.extra_lds = decode_stats_lds(nm);
+    DecodePlan P;
+    W4_TRY(plan_decode(in, &P));
+    const int rb = P.rb;
+    int waves = P.waves, nks = P.nks, kt_per_slice = P.kt_per_slice, kt_per_wave = P.kt_per_wave;
+    const size_t blocks = P.blocks;
     // x loads per k tile: one serves up to 4 token rows, two up to 8, four up to 16 (kernels/decode.hip)
     const int xl = t <= 4 ? 1 : t <= 8 ? 2 : 4;
     char sym[64];
     snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_rb%d_x%d", L.group, L.scale_bf16 ? "bf16" : "f16", rb, xl);
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
-    const size_t blocks = ceil_div(L.row_blocks, (size_t)rb);
-    int nks = 1;
     DecodeWorkspace W;
-    W4_TRY(decode_split(ctx, L, t, blocks, rb, &waves, &nks, &W, fixed_ws));
+    W4_TRY(decode_workspace(ctx, P, &W, fixed_ws));
     uint64_t ws = W.ws, tk = W.tickets;
-    // launch geometry as kernel arguments (the kernel reads nothing from the dispatch packet): k tiles per slice and
-    // per wave, both rounded up
-    int kt_per_slice = (int)ceil_div(L.k / 128, (size_t)nks), kt_per_wave = (kt_per_slice + waves - 1) / waves;
-    DecodeNorm none;
-    DecodeNorm& nm = norm ? *norm : none;
-    W4_TRY(check_decode_norm(L, t, nm));
     int ldx = (int)(nm.ldx ? nm.ldx : L.k), n_in = (int)nm.n_stats_in, stat_rows = (int)std::min<size_t>(nm.stat_rows, L.n);
     float inv_cols = nm.in_cols ? 1.0f / (float)nm.in_cols : 0.0f;
     uint64_t s_in = nm.stats_in, s_out = nm.stats_out, resid = nm.resid, nw = nm.nw;
@@ -187,13 +261,7 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     nm.n_stats_out = s_out ? std::min(blocks, (size_t)ceil_div((size_t)stat_rows, (size_t)rb * 16)) : 0;
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
                       &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind, &in_scale, &out_scale};
-    // LDS: the split-K partial tiles [waves][rb][1 KiB]; then per wave the scales of its whole k slice (rb x tiles per
-    // wave x groups per tile x 32 bytes, in whole 1 KiB DMA instructions); then the staging area of the input
-    // statistics: 1 KiB per 64 entries, at most 8
-    const unsigned shmem = (unsigned)(waves * rb * 1024) + (unsigned)waves * decode_scale_lds(L, rb, kt_per_wave) + decode_stats_lds(nm);
-    if (shmem > 160u * 1024u)
-        return w4_fail(W4A16_ERR_SHAPE, "decode: k=%zu needs %u bytes of LDS for the staged scales (limit 160 KiB): split k over more workgroups (w4a16_set_decode_ksplit) or waves", L.k, shmem);
-    return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);
+    return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), P.shmem, params);
 }
 
 // Fused gate|up projection with the SiLU*up epilogue (decode regime): y f16 [t][n/2].
@@ -203,23 +271,31 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
     if (L.n % 32 != 0) return w4_fail(W4A16_ERR_SHAPE, "decode glu: n=%zu must be a multiple of 32 (gate and up halves of whole row blocks)", L.n);
     if (L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
         return w4_fail(W4A16_ERR_SHAPE, "decode: tiled weights of 2 GiB or more exceed the buffer-descriptor range");
-    const int kt_n = (int)(L.k / 128);
-    int waves = ctx->decode_waves_per_block ? ctx->decode_waves_per_block : (t > 8 || L.row_blocks >= 1024 ? 4 : 8);
-    waves = std::max(1, std::min(std::min(waves, 8), kt_n));
+    DecodeNorm none;
+    DecodeNorm& nm = norm ? *norm : none;
+    W4_TRY(check_decode_norm(L, t, nm));
+    DecodePlanIn in;
+    in.row_blocks = L.row_blocks;
+    in.k = L.k;
+    in.group = L.group;
+    in.t = t;
+    in.cu_count = ctx->cu_count;
+    in.waves_per_block = ctx->decode_waves_per_block;
+    in.ksplit = ctx->decode_ksplit;
+    in.glu = true;
+    in.extra_lds = decode_stats_lds(nm);
+    DecodePlan P;
+    W4_TRY(plan_decode(in, &P));
+    int waves = P.waves, nks = P.nks, kt_per_slice = P.kt_per_slice, kt_per_wave = P.kt_per_wave;
+    const size_t blocks = P.blocks;
     const int xl = t <= 4 ? 1 : t <= 8 ? 2 : 4;
     char sym[64];
     snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_glu_x%d", L.group, L.scale_bf16 ? "bf16" : "f16", xl);
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = 1;
-    const size_t blocks = L.row_blocks / 2;
-    int nks = 1;
     DecodeWorkspace W;
-    W4_TRY(decode_split(ctx, L, t, blocks, 2, &waves, &nks, &W, nullptr));
+    W4_TRY(decode_workspace(ctx, P, &W, nullptr));
     uint64_t ws = W.ws, tk = W.tickets;
-    int kt_per_slice = (kt_n + nks - 1) / nks, kt_per_wave = (kt_per_slice + waves - 1) / waves;
-    DecodeNorm none;
-    DecodeNorm& nm = norm ? *norm : none;
-    W4_TRY(check_decode_norm(L, t, nm));
     if (nm.stats_out || nm.resid || nm.nw)
         return w4_fail(W4A16_ERR_UNSUPPORTED, "decode glu: the gated output takes no statistics, residual or norm weight");
     int ldx = (int)(nm.ldx ? nm.ldx : L.k), n_in = (int)nm.n_stats_in, stat_rows = 0;
@@ -231,32 +307,32 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
     float in_scale = std::ldexp(1.0f, nm.in_exp), out_scale = std::ldexp(1.0f, -nm.out_exp);
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
                       &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind, &in_scale, &out_scale};
-    const unsigned shmem = (unsigned)(waves * 2 * 1024) + (unsigned)waves * decode_scale_lds(L, 2, kt_per_wave) + decode_stats_lds(nm);
-    return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), shmem, params);
+    return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), P.shmem, params);
 }
 
-// Prefill GEMM (kernels/prefill.hip).
-static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16) {
-    if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has no tiled copy (needs k %% 128 == 0)");
-    if (!L.scales_regular)
-        return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has a zero or non-finite scale (use the decode path)");
-    if (t * L.k * 2 >= 0x80000000ull || L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
-        return w4_fail(W4A16_ERR_SHAPE, "prefill: x or the tiled weights reach 2 GiB, beyond the buffer-descriptor range");
-    // Block tile 128 x 256 (two workgroups per CU) or 64 x 256 (three per CU, 64 accumulator registers), the k range
-    // whole or cut into 2, 3, 4, 6 or 8 slices (split-K: f32 partials in a context-owned workspace, added in slice
-    // order by a second launch — deterministic), and the super-tile shape: every combination is priced and the cheapest
-    // runs.  The plan depends on (t, n, k) only and is kept per shape.
-    const size_t tiles_n = (L.n + kW4PfBn - 1) / kW4PfBn, kt_n = L.k / 128, cus = (size_t)std::max(ctx->cu_count, 1);
+// Launch plan of the prefill GEMM (kernels/prefill.hip): a pure function of (t, n, k), the CU count and the pinned
+// settings, so that a CPU test can pin what it chooses at the layer shapes (w4a16_plan_prefill).
+// Block tile 128 x 256 (two workgroups per CU) or 64 x 256 (three per CU, 64 accumulator registers), the k range whole
+// or cut into 2, 3, 4, 6 or 8 slices (split-K: f32 partials in a context-owned workspace, added in slice order by a
+// second launch — deterministic), and the super-tile shape: every combination is priced and the cheapest runs.
+struct PrefillSuper {
+    size_t sup_m, sup_n, supers, load;
+};
+struct PrefillPlan {
+    size_t bm, nks;
+    PrefillSuper sup;
+    double us;  // the price it won with
+};
+
+static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t cus, int tile_m_forced, int ksplit_forced) {
+    const size_t tiles_n = (n + kW4PfBn - 1) / kW4PfBn, kt_n = k / 128;
     // Super-tile shape for a grid of tiles_m x tiles_n block tiles: sup_m <= 8 along m, sup_n in {8, 4, 2, 1} along n.
     // Super-tiles are dealt round-robin to the 8 XCDs (m fastest), so every candidate is priced by the block tiles its
     // busiest XCD ends up with — counted exactly, partial super-tiles at the edges included — and the shape with the
     // lightest busiest XCD wins, the larger one on ties for L2 reuse.  (A fixed 8 along m left 10 tile rows as 8 + 2:
     // the XCDs that drew the 2-row super-tiles idled, 298 against 227 us on the down projection at t = 1280.)
-    struct Super {
-        size_t sup_m, sup_n, supers, load;
-    };
     auto super_for = [&](size_t tiles_m) {
-        Super best{std::min<size_t>(8, tiles_m), 8, 0, ~(size_t)0};
+        PrefillSuper best{std::min<size_t>(8, tiles_m), 8, 0, ~(size_t)0};
         for (size_t cm = std::min<size_t>(8, tiles_m); cm >= 1; cm--) {
             for (size_t cn : {8, 4, 2, 1}) {
                 const size_t sm = (tiles_m + cm - 1) / cm, sn = (tiles_n + cn - 1) / cn, sp = sm * sn;
@@ -264,7 +340,7 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
                 for (size_t sidx = 0; sidx < sp; sidx++)
                     per_xcd[sidx & 7] += std::min(cm, tiles_m - (sidx % sm) * cm) * std::min(cn, tiles_n - (sidx / sm) * cn);
                 const size_t load = *std::max_element(per_xcd, per_xcd + 8);
-                if (load < best.load || (load == best.load && cm * cn > best.sup_m * best.sup_n)) best = Super{cm, cn, sp, load};
+                if (load < best.load || (load == best.load && cm * cn > best.sup_m * best.sup_n)) best = PrefillSuper{cm, cn, sp, load};
             }
         }
         return best;
@@ -295,43 +371,58 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
         }
         return us;
     };
-    struct Plan {
-        size_t bm, nks;
-        Super sup;
-    };
-    auto make_plan = [&]() {
-        Plan best{128, 1, Super{1, 1, 0, 0}};
-        double best_us = 1e30;
-        for (size_t rows : {(size_t)128, (size_t)64}) {
-            if (ctx->prefill_tile_m && (size_t)ctx->prefill_tile_m != rows) continue;
-            const size_t tiles_m = (t + rows - 1) / rows;
-            const Super sup = super_for(tiles_m);
-            const size_t forced = ctx->prefill_ksplit > 0 ? std::max<size_t>(1, std::min<size_t>((size_t)ctx->prefill_ksplit, kt_n / 4)) : 0;
-            for (size_t cand : {1, 2, 3, 4, 6, 8}) {
-                const size_t nks = forced ? forced : cand;  // a pinned slice count is the only candidate
-                if (forced && cand != 1) break;
-                if (ctx->prefill_ksplit < 0 && nks != 1) continue;
-                if (!forced && nks > 1 && (L.n % 4 != 0 || nks > kt_n / 4)) continue;
-                const double per_cu = (double)(sup.load * nks) * 8.0 / (double)cus;  // of the busiest XCD
-                const double gens = std::ceil(per_cu / (rows == 64 ? 3.0 : 2.0));
-                double us = (double)((kt_n + nks - 1) / nks) * us_per_k_tile(rows, per_cu) + 5.7 * gens;
-                if (nks > 1) us += 6.0 + (double)nks * (double)t * (double)L.n * 8.0 / 9.76e6;
-                if (us < best_us) {
-                    best_us = us;
-                    best = Plan{rows, nks, sup};
-                }
-            }
+    PrefillPlan best{128, 1, PrefillSuper{1, 1, 0, 0}, 1e30};
+    for (size_t rows : {(size_t)128, (size_t)64}) {
+        if (tile_m_forced && (size_t)tile_m_forced != rows) continue;
+        const size_t tiles_m = (t + rows - 1) / rows;
+        const PrefillSuper sup = super_for(tiles_m);
+        const size_t forced = ksplit_forced > 0 ? std::max<size_t>(1, std::min<size_t>((size_t)ksplit_forced, kt_n / 4)) : 0;
+        for (size_t cand : {1, 2, 3, 4, 6, 8}) {
+            const size_t nks = forced ? forced : cand;  // a pinned slice count is the only candidate
+            if (forced && cand != 1) break;
+            if (ksplit_forced < 0 && nks != 1) continue;
+            if (!forced && nks > 1 && (n % 4 != 0 || nks > kt_n / 4)) continue;
+            const double per_cu = (double)(sup.load * nks) * 8.0 / (double)cus;  // of the busiest XCD
+            const double gens = std::ceil(per_cu / (rows == 64 ? 3.0 : 2.0));
+            double us = (double)((kt_n + nks - 1) / nks) * us_per_k_tile(rows, per_cu) + 5.7 * gens;
+            if (nks > 1) us += 6.0 + (double)nks * (double)t * (double)n * 8.0 / 9.76e6;
+            if (us < best.us) best = PrefillPlan{rows, nks, sup, us};
         }
-        return best;
-    };
-    Plan plan;
+    }
+    return best;
+}
+
+extern "C" int w4a16_plan_prefill(size_t t, size_t n, size_t k, int cu_count, int tile_rows, int k_slices, size_t out[5],
+                                  double* price_us) {
+    if (t == 0 || n == 0 || k == 0 || k % 128 != 0 || cu_count <= 0 || !out ||
+        (tile_rows != 0 && tile_rows != 64 && tile_rows != 128) || k_slices < -1 || k_slices > 16)
+        return w4_fail(W4A16_ERR_ARG, "plan_prefill: t=%zu n=%zu k=%zu cus=%d tile=%d slices=%d", t, n, k, cu_count, tile_rows, k_slices);
+    const PrefillPlan P = plan_prefill(t, n, k, (size_t)cu_count, tile_rows, k_slices);
+    out[0] = P.bm;
+    out[1] = P.nks;
+    out[2] = P.sup.sup_m;
+    out[3] = P.sup.sup_n;
+    out[4] = P.sup.supers;
+    if (price_us) *price_us = P.us;
+    return 0;
+}
+
+// Prefill GEMM (kernels/prefill.hip).
+static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16) {
+    if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has no tiled copy (needs k %% 128 == 0)");
+    if (!L.scales_regular)
+        return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has a zero or non-finite scale (use the decode path)");
+    if (t * L.k * 2 >= 0x80000000ull || L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
+        return w4_fail(W4A16_ERR_SHAPE, "prefill: x or the tiled weights reach 2 GiB, beyond the buffer-descriptor range");
+    // the plan depends on (t, n, k) and the pinned settings only and is kept per shape
+    PrefillPlan plan;
     {
         const auto key = std::make_tuple(t, L.n, L.k, ctx->prefill_tile_m, ctx->prefill_ksplit);
         const auto hit = ctx->prefill_plans.find(key);
         if (hit != ctx->prefill_plans.end()) {
-            plan = Plan{hit->second[0], hit->second[1], Super{hit->second[2], hit->second[3], hit->second[4], 0}};
+            plan = PrefillPlan{hit->second[0], hit->second[1], PrefillSuper{hit->second[2], hit->second[3], hit->second[4], 0}, 0.0};
         } else {
-            plan = make_plan();
+            plan = plan_prefill(t, L.n, L.k, (size_t)std::max(ctx->cu_count, 1), ctx->prefill_tile_m, ctx->prefill_ksplit);
             ctx->prefill_plans[key] = {plan.bm, plan.nks, plan.sup.sup_m, plan.sup.sup_n, plan.sup.supers};
         }
     }
@@ -389,6 +480,23 @@ extern "C" int w4a16_gemm_host(w4a16_ctx* ctx, const uint16_t* x_f16, size_t t, 
 }
 
 // ------------------------------------------------------------------------------------------------ registration
+// The MFMA prefill kernels multiply their accumulators by s_prev / s_cur at every group boundary and hold sum / s_cur:
+// every scale must be finite and non-zero, and a bf16 scale inside [2^-60, 2^60], so that neither a quotient of two
+// scales nor an accumulator expressed in the smallest one leaves the f32 range (f16 scales span 2^-24 .. 2^16 and
+// always qualify; a bf16 subnormal or 1e-38 does not).
+bool w4_scales_regular(const uint16_t* sp, size_t count, int scale_bf16) {
+    const unsigned expmask = scale_bf16 ? 0x7F80u : 0x7C00u;
+    for (size_t i = 0; i < count; i++) {
+        const unsigned b = sp[i];
+        if ((b & 0x7FFFu) == 0 || (b & expmask) == expmask) return false;
+        if (scale_bf16) {
+            const unsigned e = (b >> 7) & 0xFFu;  // biased exponent, 127 = 2^0
+            if (e < 127u - 60u || e > 127u + 60u) return false;
+        }
+    }
+    return true;
+}
+
 static void free_lin(w4a16_ctx* ctx, W4Lin& L) {
     (void)w4a16_free(ctx, L.q_raw);
     (void)w4a16_free(ctx, L.s_raw);
@@ -412,28 +520,9 @@ extern "C" int w4a16_upload_lin(w4a16_ctx* ctx, const char* name, const void* q,
     L.k = k;
     L.group = group;
     L.scale_bf16 = scale_bf16 ? 1 : 0;
-    {
-        const uint16_t* sp = static_cast<const uint16_t*>(s);
-        const size_t ns = slen_bytes / 2;
-        // "regular": what the MFMA prefill kernel can carry as a running unit (it multiplies its accumulators by
-        // s_prev / s_cur at every group boundary and holds sum / s_cur) — finite, non-zero, and for bf16 scales inside
-        // [2^-60, 2^60], so that neither a quotient of two scales nor an accumulator expressed in the smallest one
-        // leaves the f32 range (f16 scales span 2^-24 .. 2^16 and always qualify; a bf16 subnormal or 1e-38 does not).
-        // Other linears are served by the streaming kernels, which only ever multiply by a scale.
-        const unsigned expmask = scale_bf16 ? 0x7F80u : 0x7C00u;
-        for (size_t i = 0; i < ns; i++) {
-            const unsigned b = sp[i];
-            bool bad = (b & 0x7FFFu) == 0 || (b & expmask) == expmask;
-            if (!bad && scale_bf16) {
-                const unsigned e = (b >> 7) & 0xFFu;  // biased exponent, 127 = 2^0
-                bad = e < 127u - 60u || e > 127u + 60u;
-            }
-            if (bad) {
-                L.scales_regular = false;
-                break;
-            }
-        }
-    }
+    // "regular": what the MFMA prefill kernel can carry as a running unit (w4_scales_regular).  Other linears are served
+    // by the streaming kernels, which only ever multiply by a scale.
+    L.scales_regular = w4_scales_regular(static_cast<const uint16_t*>(s), slen_bytes / 2, scale_bf16);
     int rc = w4a16_alloc(ctx, qlen_bytes, &L.q_raw);
     if (!rc) rc = w4a16_alloc(ctx, slen_bytes, &L.s_raw);
     if (!rc) rc = w4a16_h2d(ctx, L.q_raw, q, qlen_bytes);

@@ -6,7 +6,8 @@ import os
 PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG, "libw4a16hip.so")
 
-ERR_SHAPE, ERR_SYMBOL, ERR_UNSUPPORTED, ERR_NOT_FOUND, ERR_ARG, ERR_ASSET = 10001, 10002, 10003, 10004, 10005, 10006
+ERR_SHAPE, ERR_SYMBOL, ERR_UNSUPPORTED, ERR_NOT_FOUND, ERR_ARG, ERR_ASSET, ERR_STALE_GRAPH = (
+    10001, 10002, 10003, 10004, 10005, 10006, 10007)
 PATH_AUTO, PATH_LANE, PATH_DECODE, PATH_PREFILL, PATH_STREAM = 0, 1, 2, 3, 4
 ACT_SILU, ACT_GELU_TANH = 0, 1
 
@@ -56,6 +57,10 @@ _SIGS = {
     "w4a16_lin_forward": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_size_t, C.c_int, C.c_int]),
     "w4a16_lin_forward_noalloc": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_size_t, C.c_int]),
     "w4a16_noalloc_workspace_bytes": (C.c_size_t, []),
+    "w4a16_plan_decode": (C.c_int, [C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.POINTER(C.c_int),
+                                    C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_size_t)]),
+    "w4a16_plan_prefill": (C.c_int, [C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_int,
+                                     C.POINTER(C.c_size_t), C.POINTER(C.c_double)]),
     "w4a16_lin_forward_glu": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_size_t]),
     "w4a16_lin_forward_glu_act": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_size_t, C.c_int]),
     "w4a16_lin_forward_deferred_norm": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64,

@@ -18,6 +18,25 @@ from . import ffi
 from .ffi import ACT_GELU_TANH, ACT_SILU, PATH_AUTO, PATH_DECODE, PATH_LANE, PATH_PREFILL, PATH_STREAM, W4a16Error  # noqa: F401
 
 
+def plan_decode(n, k, group, t, cu_count=256, glu=False):
+    """Launch plan of the decode path for a linear of this shape (no context, no GPU): dict of rows_per_wave,
+    waves_per_block, k_slices, lds_bytes."""
+    rows, waves, nks, lds = C.c_int(), C.c_int(), C.c_int(), C.c_size_t()
+    ffi.check(ffi.load().w4a16_plan_decode(n, k, group, t, cu_count, int(bool(glu)), C.byref(rows), C.byref(waves),
+                                           C.byref(nks), C.byref(lds)))
+    return {"rows_per_wave": rows.value, "waves_per_block": waves.value, "k_slices": nks.value, "lds_bytes": lds.value}
+
+
+def plan_prefill(t, n, k, cu_count=256, tile_rows=0, k_slices=0):
+    """Launch plan of the prefill path (no context, no GPU): dict of tile_rows, k_slices, super_m, super_n, supers,
+    price_us."""
+    out = (C.c_size_t * 5)()
+    us = C.c_double()
+    ffi.check(ffi.load().w4a16_plan_prefill(t, n, k, cu_count, tile_rows, k_slices, out, C.byref(us)))
+    return {"tile_rows": out[0], "k_slices": out[1], "super_m": out[2], "super_n": out[3], "supers": out[4],
+            "price_us": us.value}
+
+
 def check_shapes(t, qlen, slen, xlen, n, k, group):
     """gptq4.rs:31-58.  Raises W4a16Error(ERR_SHAPE) on violation."""
     ffi.check(ffi.load().w4a16_check_shapes(t, qlen, slen, xlen, n, k, group))

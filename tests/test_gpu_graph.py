@@ -150,3 +150,44 @@ def test_chain_graph_64_layers_at_27b_shapes(dec):
         graph.destroy()
     cc.free(px)
     cc.free(py)
+
+
+def test_graph_is_refused_after_its_scratch_buffer_was_replaced(dec):
+    """A graph holds the addresses of the context's scratch buffers of its time (here the partial tiles of a decode
+    launch split over k).  An eager call that needs the buffer larger replaces it; a replay would then write freed
+    memory, so graph_launch refuses the stale graph (reference: graph_invalidate on every scratch reallocation,
+    w4a16_dec/buffers.rs:6-31).  Calls that fit the buffers leave the graph valid."""
+    d = ops.W4a16Dec()  # a context of its own: the workspace must start small
+    cc = d.cc
+    try:
+        g, t = 128, 4
+        q1, s1, x = gen.make_linear(256, 1024, g, t, seed=11)
+        q2, s2, _ = gen.make_linear(4096, 1024, g, 1, seed=12)
+        d.upload_lin_g("small", q1, s1, 256, 1024, g, False)
+        d.upload_lin_g("large", q2, s2, 4096, 1024, g, False)
+        px, py = cc.to_device(x), cc.alloc(t * 4096 * 4)
+        d.set_decode_ksplit(4)
+        d.lin_forward("small", px, py, t, path=ops.PATH_DECODE)  # sizes the workspace for the small linear
+        eager = cc.d2h(py, (t, 256), np.uint32)
+        cc.capture_begin()
+        d.lin_forward("small", px, py, t, path=ops.PATH_DECODE)
+        graph = cc.capture_end()
+        graph.launch()
+        assert np.array_equal(cc.d2h(py, (t, 256), np.uint32), eager)
+        d.lin_forward("small", px, py, t, path=ops.PATH_DECODE)  # fits: nothing is replaced
+        graph.launch()
+        assert np.array_equal(cc.d2h(py, (t, 256), np.uint32), eager)
+        d.lin_forward("large", px, py, t, path=ops.PATH_DECODE)  # 16 times the partial tiles: the workspace is replaced
+        cc.sync()
+        with pytest.raises(ops.W4a16Error) as e:
+            graph.launch()
+        assert e.value.code == ffi.ERR_STALE_GRAPH and "capture again" in str(e.value)
+        graph.destroy()
+        cc.capture_begin()  # a new capture works and replays
+        d.lin_forward("small", px, py, t, path=ops.PATH_DECODE)
+        graph = cc.capture_end()
+        graph.launch()
+        assert np.array_equal(cc.d2h(py, (t, 256), np.uint32), eager)
+        graph.destroy()
+    finally:
+        cc.close()

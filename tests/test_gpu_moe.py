@@ -323,6 +323,46 @@ def test_moe_ffn_tiled_full_shape(dec, orc, full_experts):
         dec.set_moe_tiled(2)
 
 
+@pytest.mark.parametrize("group,bf", [(32, True), (128, False)])
+def test_moe_irregular_scales_stay_off_the_tiled_kernels(dec, orc, group, bf):
+    """Experts with a zero scale (and, for bf16, a scale of about 1e-38) at a size where AUTO would pick the MFMA-tiled
+    grouped kernels: those carry sum / s_cur as a running unit and would produce NaN; the upload marks the arenas
+    irregular, AUTO stays on the streaming kernels (same results as with the tiled kernels switched off, checked
+    against the oracle) and a forced tiled launch is refused."""
+    E, h, n_ff, k, t = 4, 256, 128, 2, 256  # mean run per expert 128 >= 96: AUTO would go tiled
+    q13, s13, q2, s2 = gen.make_experts(E, h, n_ff, group, seed=gen.GATE_SEED + 7 * group)
+    if bf:
+        s13, s2 = _bf16_scales(s13), _bf16_scales(s2)
+    x = gen.normal_f16(77, (t, h))
+    idx, wt = ops.moe_topk(gen.router_logits(t, E, seed=5), k)
+    dec.upload_experts("regular", q13, s13, q2, s2, E, h, n_ff, group, bf)
+    y0, _, _, blk0 = _run_ffn(dec, "regular", x, idx, wt, t, k, h)
+    assert blk0 == 64, "the regular arenas take the tiled kernels at this size"
+    s13 = s13.copy()
+    s2 = s2.copy()
+    s13[1, 5, 0] = 0            # a zero scale in expert 1, gate row 5, first group
+    s2[2, 9, 1 if n_ff // group > 1 else 0] = 0x0001 if bf else 0  # bf16: 9e-41, far below 2^-60; f16: another zero
+    if bf:
+        s13[3, 40, 1] = 0x0080  # bf16 1.18e-38 (the smallest normal)
+    dec.upload_experts("irregular", q13, s13, q2, s2, E, h, n_ff, group, bf)
+    y, act, c2, blk = _run_ffn(dec, "irregular", x, idx, wt, t, k, h)
+    assert np.all(np.isfinite(y)), "NaN or Inf from an irregular scale"
+    dec.set_moe_tiled(-1)
+    try:
+        y_stream, act_s, c2_s, blk_s = _run_ffn(dec, "irregular", x, idx, wt, t, k, h)
+    finally:
+        dec.set_moe_tiled(0)
+    assert blk == blk_s and np.array_equal(y.view(np.uint32), y_stream.view(np.uint32)), "AUTO = streaming kernels"
+    _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, "irregular scales g%d bf%d" % (group, bf))
+    dec.set_moe_tiled(1)
+    try:
+        with pytest.raises(ops.W4a16Error) as e:
+            _run_ffn(dec, "irregular", x, idx, wt, t, k, h)
+        assert "scale" in str(e.value)
+    finally:
+        dec.set_moe_tiled(0)
+
+
 def test_moe_errors(dec, small_experts):
     name = small_experts[(32, False)][0]
     with pytest.raises(ops.W4a16Error):

@@ -90,3 +90,32 @@ def test_noalloc_entry_point_equals_lin_forward_two_calls_second_smaller():
         cc.free(yd)
     finally:
         dec.cc.close()
+
+
+def test_noalloc_scratch_has_one_owner_per_gpu():
+    """The fixed scratch of a GPU serves one context at a time: two contexts sharing its tickets could sum each other's
+    partial tiles.  The second context is refused until the first is destroyed."""
+    a, b = ops.W4a16Dec(), ops.W4a16Dec()
+    try:
+        q, s, x = gen.make_linear(208, 2560, 128, 2, seed=43)
+        outs = []
+        for d in (a, b):
+            d.upload_lin_g("lin", q, s, 208, 2560, 128, False)
+            d.set_decode_ksplit(4)
+        xa, ya = a.cc.to_device(x), a.cc.alloc(2 * 208 * 4)
+        xb, yb = b.cc.to_device(x), b.cc.alloc(2 * 208 * 4)
+        a.lin_forward_noalloc("lin", xa, ya, 2)
+        want = a.cc.d2h(ya, (2, 208), np.uint32)
+        with pytest.raises(ops.W4a16Error) as e:
+            b.lin_forward_noalloc("lin", xb, yb, 2)
+        assert e.value.code == ffi.ERR_ARG and "another context" in str(e.value)
+        b.lin_forward("lin", xb, yb, 2, path=ops.PATH_DECODE)  # the allocating entry point is per context and works
+        assert np.array_equal(b.cc.d2h(yb, (2, 208), np.uint32), want)
+        a.cc.close()
+        a = None
+        b.lin_forward_noalloc("lin", xb, yb, 2)  # the owner is gone: the array is free again
+        assert np.array_equal(b.cc.d2h(yb, (2, 208), np.uint32), want)
+    finally:
+        if a is not None:
+            a.cc.close()
+        b.cc.close()
