@@ -422,10 +422,68 @@ def main():
     ref_s = oracle.gemm_lane_sample(xp, q0, s0, k, g, rows, toks)
     par_pf = parity.assert_close(gen.f16_bits_to_f32(yp[toks, rows]), gen.f16_bits_to_f32(gen.f32_to_f16_bits(ref_s)),
                                  "prefill f16 out, sample")
-    cc.free(xpd)
-    cc.free(ypd)
     extra["parity_prefill_f16_sample2048"] = {a: par_pf[a] for a in keys}
     extra["prefill_ms_spread"] = spread(pf_samples, 1.0, 4)
+    if not args.no_extra:
+        # every one of the 4096 x 34816 outputs of the launch just timed against the bit-exact device twin of the lane
+        # order (itself pinned to the CPU oracle on the sample above): the full-shape strict-failure count
+        ytw = cc.alloc(mp * n * 4)
+        dec.upload_lin_g("gate_up.twin", q0, s0, n, k, g, False)  # the timed copies dropped their as-given operands
+        dec.lin_forward("gate_up.twin", xpd, ytw, mp, out_f16=False, path=ops.PATH_LANE)
+        twin = cc.d2h(ytw, (mp, n), np.float32)
+        cc.free(ytw)
+        if not np.array_equal(twin[toks, rows].view(np.uint32), ref_s.view(np.uint32)):
+            raise RuntimeError("prefill: the device twin of the lane order differs from the CPU oracle on the sample")
+        par_full = parity.assert_close(gen.f16_bits_to_f32(yp), gen.f16_bits_to_f32(gen.f32_to_f16_bits(twin)),
+                                       "prefill f16 out, all outputs against the device twin")
+        extra["parity_prefill_f16_full_vs_device_twin"] = dict({a: par_full[a] for a in keys}, outputs=int(mp) * int(n))
+        del twin
+        # the same GEMM with the SiLU*up epilogue (f16 [M][N/2] out): what the prefill chain runs for gate|up
+        yg = cc.alloc(mp * (n // 2) * 2)
+        e0, e1 = cc.event(), cc.event()
+        glu_samples = []
+        for r in range(ROUNDS):
+            for i in range(5):
+                dec.lin_forward_glu(names[i % len(names)], xpd, yg, mp)
+            e0.record()
+            for i in range(psteps):
+                dec.lin_forward_glu(names[(5 + i) % len(names)], xpd, yg, mp)
+            e1.record()
+            cc.sync()
+            glu_samples.append(e0.elapsed_ms(e1) / psteps)
+        glu_kernel = cc.last_launch_symbol()
+        glu_ms = sorted(glu_samples)[ROUNDS // 2]
+        # same bits as the plain launch followed by the element-wise kernel (checked on the first copy)
+        y32 = cc.alloc(mp * n * 4)
+        ya = cc.alloc(mp * (n // 2) * 2)
+        dec.lin_forward(names[0], xpd, y32, mp, out_f16=False, path=ops.PATH_PREFILL)
+        dec.silu_mul_f16(y32, n // 2, mp, ya)
+        dec.lin_forward_glu(names[0], xpd, yg, mp)
+        glu_same = bool(np.array_equal(cc.d2h(ya, (mp, n // 2), np.uint16), cc.d2h(yg, (mp, n // 2), np.uint16)))
+        if not glu_same:
+            raise RuntimeError("prefill: the gated launch differs from linear + silu_mul")
+        # what the fusion replaces: the element-wise launch over the f32 [M][N] intermediate
+        ew_samples = []
+        for r in range(ROUNDS):
+            e0.record()
+            for i in range(psteps):
+                dec.silu_mul_f16(y32, n // 2, mp, ya)
+            e1.record()
+            cc.sync()
+            ew_samples.append(e0.elapsed_ms(e1) / psteps)
+        ew_ms = sorted(ew_samples)[ROUNDS // 2]
+        for p_ in (y32, ya, yg):
+            cc.free(p_)
+        glu_tf = pf_flops / (glu_ms * 1e-3) / 1e12
+        extra["prefill_gate_up_silu_fused"] = {
+            "workload": "prefill GEMM M=4096 K=5120 N=34816 g128 with SiLU*up in the epilogue, f16 [M][N/2] out",
+            "ms": round(glu_ms, 4), "ms_spread": spread(glu_samples, 1.0, 4), "TFLOPs": round(glu_tf, 1),
+            "mfma_frac": round(glu_tf / MFMA_F16_PEAK_TFLOPS, 4), "kernel": glu_kernel,
+            "equals_linear_then_silu_mul_bits": glu_same,
+            "plain_launch_ms": round(pf_ms, 4), "separate_silu_mul_launch_ms": round(ew_ms, 4),
+            "two_launch_sequence_ms": round(pf_ms + ew_ms, 4)}
+    cc.free(xpd)
+    cc.free(ypd)
 
     if not args.no_extra:
         table = []
@@ -462,6 +520,7 @@ def main():
                                "TFLOPs": round(tf, 1), "mfma_frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
                                "kernel": cc.last_launch_symbol()})
         extra["prefill_table"] = ptable
+        down4096 = [r for r in ptable if r["shape"].startswith("down") and r["M"] == 4096][0]
         for p_ in (xp2, yp2, xp1, x2d):
             cc.free(p_)
         extra["moe_table"] = bench_moe(dec, gen, ops, args)
@@ -496,6 +555,13 @@ def main():
         "cpu_baseline": cpu,
         "extra": extra,
     }
+    if not args.no_extra:
+        pf2_traffic, pf2_src = measured_traffic(down4096["kernel"])
+        line["roofline_prefill_down"] = {
+            "bound": "mfma", "achieved": down4096["TFLOPs"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": down4096["mfma_frac"], "traffic": pf2_traffic, "traffic_source": pf2_src, "kernel": down4096["kernel"],
+            "workload": "prefill GEMM M=4096 K=17408 N=5120 g128", "ms_per_launch": down4096["ms"],
+            "algorithmic_flops_per_launch": 2.0 * 4096 * 5120 * 17408}
     print(json.dumps(line))
 
 

@@ -207,8 +207,12 @@ size_t w4a16_noalloc_workspace_bytes(void);
 /* The gate|up projection of a dense FFN with the elementwise kernel that follows it folded in
  * (gemv_multi_dev of the gate/up group + ew_dev_fused, w4a16_dec/chains.rs:271-287, assets/ew.cu:9-32):
  * y[r][c] = f16(silu(g) * u), g = (W x)[r][c], u = (W x)[r][n/2 + c], f32 arithmetic, for a linear whose rows 0..n/2 are
- * the gate and n/2..n the up projection (n % 32 == 0).  t <= 16 (decode regime); y_f16_dev: f16 [t][n/2].  Same values
- * as w4a16_lin_forward (decode path, same launch shape) followed by w4a16_silu_mul_f16. */
+ * the gate and n/2..n the up projection (n % 32 == 0).  y_f16_dev: f16 [t][n/2].  Any t: up to 16 rows the decode
+ * kernel, up to 64 (and for a linear with a zero or non-finite scale) the weight-streaming kernel, beyond that the
+ * MFMA-tiled prefill kernel, each with the activation in its epilogue — the pair lin_forward + ew of the reference's
+ * prefill chain (w4a16_dec/prefill.rs:148-207) in one launch.  Same values, bit for bit, as w4a16_lin_forward on the
+ * same path and launch shape followed by w4a16_silu_mul_f16 (the gated streaming kernel never splits over k; compare
+ * with w4a16_set_decode_ksplit(-1)), without the [t][n] f32 round trip. */
 int w4a16_lin_forward_glu(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_f16_dev, size_t t);
 /* The same with the activation named: act = W4A16_ACT_SILU (above) or W4A16_ACT_GELU_TANH, the elementwise kernel the
  * reference launches for gelu-gated models (ew_gelu, assets/ew.cu:34-57):

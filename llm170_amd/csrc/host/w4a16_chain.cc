@@ -120,8 +120,9 @@ extern "C" int w4a16_chain_forward(w4a16_ctx* ctx, const char* prefix, size_t la
         W4_TRY(w4a16_rms_rescale_f16(ctx, S.y32, L[0]->n, hidden, t, S.h16a));
         W4_TRY(w4a16_lin_forward(ctx, nm[1], S.h16a, S.y32, t, 0, W4A16_PATH_AUTO));
         W4_TRY(w4a16_rms_rescale_f16(ctx, S.y32, hidden, hidden, t, S.h16a));
-        if (t <= 16 && L[2]->q_tiled && L[2]->n % 32 == 0) {
-            // decode regime: SiLU*up is the epilogue of the gate|up kernel
+        if (L[2]->q_tiled && L[2]->n % 32 == 0) {
+            // SiLU*up is the epilogue of the gate|up kernel in every regime (decode, streaming, MFMA tiles): same bits
+            // as the linear followed by the element-wise launch, without the [t][2 n_ff] f32 round trip
             W4_TRY(w4a16_lin_forward_glu(ctx, nm[2], S.h16a, S.h16b, t));
         } else {
             W4_TRY(w4a16_lin_forward(ctx, nm[2], S.h16a, S.y32, t, 0, W4A16_PATH_AUTO));

@@ -137,7 +137,8 @@ int w4_find_lin(w4a16_ctx* ctx, const char* name, W4Lin** out);
 // carries the running unit s_prev / s_cur can take
 bool w4_scales_regular(const uint16_t* s, size_t count, int scale_bf16);
 int w4_ensure(w4a16_ctx* ctx, uint64_t* buf, size_t* cap, size_t bytes);
-int w4_dense_grouped(w4a16_ctx* ctx, const W4Lin& L, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16);
+// glu_act >= 0: L is a fused gate|up linear and y_dev receives f16 [t][n/2] = act(gate) * up on the f32 sums
+int w4_dense_grouped(w4a16_ctx* ctx, const W4Lin& L, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16, int glu_act = -1);
 int w4_lin_forward_fixed_ws(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16,
                             uint64_t ws, size_t ws_bytes, uint64_t tickets, size_t ticket_bytes);
 // per-device fixed scratch of the allocation-free entry point (w4a16_noalloc.hip)

@@ -286,7 +286,7 @@ static int launch_moe_gemm(w4a16_ctx* ctx, const W4Experts& E, bool glu, uint64_
 // token, segments of up to 64 tokens.  Between the streaming decode kernel (t <= 16: x operands straight from global
 // memory) and the 128-row MFMA tiles of the prefill kernel, this regime is still bound by the weight stream, and the
 // grouped kernel shares each x tile among all waves of a workgroup through LDS.
-int w4_dense_grouped(w4a16_ctx* ctx, const W4Lin& L, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16) {
+int w4_dense_grouped(w4a16_ctx* ctx, const W4Lin& L, uint64_t x_dev, uint64_t y_dev, size_t t, int out_f16, int glu_act) {
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "stream: linear has no tiled copy (needs k %% 128 == 0)");
     if (t > 0x7fffffffu / 2) return w4_fail(W4A16_ERR_SHAPE, "stream: t=%zu too large", t);
     W4MoeScratch& S = ctx->moe;
@@ -314,19 +314,30 @@ int w4_dense_grouped(w4a16_ctx* ctx, const W4Lin& L, uint64_t x_dev, uint64_t y_
         W4_TRY(w4a16_alloc(ctx, 8, &S.always));
         W4_TRY(w4a16_h2d(ctx, S.always, big, 8));
     }
+    const bool glu = glu_act >= 0;
     W4Experts E;
-    E.q2 = L.q_tiled;
-    E.s2 = L.s_tiled;
     E.n_exp = 1;
-    E.h = L.n;
-    E.n_ff = L.k;
     E.group = L.group;
     E.scale_bf16 = L.scale_bf16;
+    if (glu) {  // the linear is the "gate|up arena" of its one expert: n = 2 n_ff rows over k = h
+        if (L.n % 32 != 0) return w4_fail(W4A16_ERR_SHAPE, "stream glu: n=%zu must be a multiple of 32", L.n);
+        E.q13 = L.q_tiled;
+        E.s13 = L.s_tiled;
+        E.h = L.k;
+        E.n_ff = L.n / 2;
+    } else {
+        E.q2 = L.q_tiled;
+        E.s2 = L.s_tiled;
+        E.h = L.n;
+        E.n_ff = L.k;
+    }
     // k slices until the launch has a few workgroups per CU
-    const size_t waves = ctx->moe_waves >= 8 ? 8 : 4, units = (L.row_blocks + 1) / 2;
+    const size_t waves = ctx->moe_waves >= 8 ? 8 : 4, units = glu ? L.row_blocks / 2 : (L.row_blocks + 1) / 2;
     const size_t groups = (units + waves - 1) / waves;
     size_t nks = 1;
-    if (ctx->decode_ksplit > 0) {
+    if (glu) {
+        nks = 1;  // the gated kernel does not split over k
+    } else if (ctx->decode_ksplit > 0) {
         nks = (size_t)ctx->decode_ksplit;
     } else if (ctx->decode_ksplit == 0) {
         // only while the launch has fewer workgroups than CUs: the 27B down projection (40 unit groups) runs 8 slices
@@ -334,6 +345,14 @@ int w4_dense_grouped(w4a16_ctx* ctx, const W4Lin& L, uint64_t x_dev, uint64_t y_
         while (groups * segs * nks < (size_t)std::max(ctx->cu_count, 1) && nks < 8) nks *= 2;
     }
     // the grid covers exactly `segs` segments, so the "padded total" may be the constant no segment start reaches
+    if (glu) {
+        // bit 1: the activation takes the f32 sums (the expert FFN rounds gate and up to f16 first)
+        const int keep = ctx->moe_act_kind;
+        ctx->moe_act_kind = glu_act | 2;
+        const int rc = launch_moe_gemm(ctx, E, true, x_dev, t, 1, y_dev, 1, 0, t, block, segs, S.iota, S.zeros, S.always, 1);
+        ctx->moe_act_kind = keep;
+        return rc;
+    }
     return launch_moe_gemm(ctx, E, false, x_dev, t, 1, y_dev, out_f16, 0, t, block, segs, S.iota, S.zeros, S.always, nks);
 }
 

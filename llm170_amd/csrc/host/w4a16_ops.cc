@@ -324,8 +324,9 @@ struct PrefillPlan {
     double us;  // the price it won with
 };
 
-static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t cus, int tile_m_forced, int ksplit_forced) {
-    const size_t tiles_n = (n + kW4PfBn - 1) / kW4PfBn, kt_n = k / 128;
+static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t cus, int tile_m_forced, int ksplit_forced, bool glu = false) {
+    // a gated launch tiles the n/2 output columns by 128 (each block tile holds the matching 128 up columns as well)
+    const size_t tiles_n = glu ? (n / 2 + kW4PfBn / 2 - 1) / (kW4PfBn / 2) : (n + kW4PfBn - 1) / kW4PfBn, kt_n = k / 128;
     // Super-tile shape for a grid of tiles_m x tiles_n block tiles: sup_m <= 8 along m, sup_n in {8, 4, 2, 1} along n.
     // Super-tiles are dealt round-robin to the 8 XCDs (m fastest), so every candidate is priced by the block tiles its
     // busiest XCD ends up with — counted exactly, partial super-tiles at the edges included — and the shape with the
@@ -381,7 +382,7 @@ static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t cus, int ti
             const size_t nks = forced ? forced : cand;  // a pinned slice count is the only candidate
             if (forced && cand != 1) break;
             if (ksplit_forced < 0 && nks != 1) continue;
-            if (!forced && nks > 1 && (n % 4 != 0 || nks > kt_n / 4)) continue;
+            if (!forced && nks > 1 && (n % (glu ? 8 : 4) != 0 || nks > kt_n / 4)) continue;
             const double per_cu = (double)(sup.load * nks) * 8.0 / (double)cus;  // of the busiest XCD
             const double gens = std::ceil(per_cu / (rows == 64 ? 3.0 : 2.0));
             double us = (double)((kt_n + nks - 1) / nks) * us_per_k_tile(rows, per_cu) + 5.7 * gens;
@@ -407,8 +408,11 @@ extern "C" int w4a16_plan_prefill(size_t t, size_t n, size_t k, int cu_count, in
     return 0;
 }
 
-// Prefill GEMM (kernels/prefill.hip).
-static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16) {
+// Prefill GEMM (kernels/prefill.hip).  glu_act >= 0: the linear is a fused gate|up projection and y receives
+// f16 [t][n/2] = act(gate) * up (W4A16_ACT_*), the element-wise kernel folded into the epilogue.
+static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16, int glu_act = -1) {
+    const bool glu = glu_act >= 0;
+    if (glu && L.n % 32 != 0) return w4_fail(W4A16_ERR_SHAPE, "prefill glu: n=%zu must be a multiple of 32 (gate and up halves of whole row blocks)", L.n);
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has no tiled copy (needs k %% 128 == 0)");
     if (!L.scales_regular)
         return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has a zero or non-finite scale (use the decode path)");
@@ -417,38 +421,38 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     // the plan depends on (t, n, k) and the pinned settings only and is kept per shape
     PrefillPlan plan;
     {
-        const auto key = std::make_tuple(t, L.n, L.k, ctx->prefill_tile_m, ctx->prefill_ksplit);
+        const auto key = std::make_tuple(t, L.n, L.k, ctx->prefill_tile_m + (glu ? 1000 : 0), ctx->prefill_ksplit);
         const auto hit = ctx->prefill_plans.find(key);
         if (hit != ctx->prefill_plans.end()) {
             plan = PrefillPlan{hit->second[0], hit->second[1], PrefillSuper{hit->second[2], hit->second[3], hit->second[4], 0}, 0.0};
         } else {
-            plan = plan_prefill(t, L.n, L.k, (size_t)std::max(ctx->cu_count, 1), ctx->prefill_tile_m, ctx->prefill_ksplit);
+            plan = plan_prefill(t, L.n, L.k, (size_t)std::max(ctx->cu_count, 1), ctx->prefill_tile_m, ctx->prefill_ksplit, glu);
             ctx->prefill_plans[key] = {plan.bm, plan.nks, plan.sup.sup_m, plan.sup.sup_n, plan.sup.supers};
         }
     }
     const size_t bm = plan.bm, nks = plan.nks, sup_m = plan.sup.sup_m, sup_n = plan.sup.sup_n, supers = plan.sup.supers;
     const size_t grid = ((supers + 7) / 8) * (sup_m * sup_n) * 8;
     char sym[64];
-    snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s%s", L.group, L.scale_bf16 ? "bf16" : "f16", bm == 64 ? "_m64" : "");
+    snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s%s%s", L.group, L.scale_bf16 ? "bf16" : "f16", bm == 64 ? "_m64" : "", glu ? "_glu" : "");
     const unsigned shmem = (unsigned)(2 * bm * kW4PfKs * 2);  // two stages of bm rows x PF_KS halves
     uint64_t qt = L.q_tiled, st = L.s_tiled;
-    int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
-    int spm = (int)sup_m, spn = (int)sup_n;
+    int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = (out_f16 || glu) ? 1 : 0;
+    int spm = (int)sup_m, spn = (int)sup_n, act = glu ? glu_act : 0, glu_i = glu ? 1 : 0;
     if (nks == 1) {
-        void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &spm, &spn};
+        void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &spm, &spn, &act};  // act: gated kernels only
         return w4_launch(ctx, sym, (unsigned)grid, 1, kW4PfThreads, shmem, params);
     }
-    if (L.n % 4 != 0) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: split-K needs n %% 4 == 0");
+    if (L.n % (glu ? 8 : 4) != 0) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: split-K needs n %% %d == 0", glu ? 8 : 4);
     const size_t count = t * L.n;
     W4_TRY(w4_ensure(ctx, &ctx->prefill_ws, &ctx->prefill_ws_cap, count * 4 * nks));
     uint64_t ws = ctx->prefill_ws;
     int zero = 0;
-    void* params[] = {&qt, &st, &x, &ws, &row_blocks, &ki, &ni, &ti, &zero, &spm, &spn};
+    void* params[] = {&qt, &st, &x, &ws, &row_blocks, &ki, &ni, &ti, &zero, &spm, &spn, &act};
     W4_TRY(w4_launch(ctx, sym, (unsigned)grid, (unsigned)nks, kW4PfThreads, shmem, params));
     int nksi = (int)nks;
     size_t cnt = count;
-    void* rp[] = {&ws, &y, &nksi, &cnt, &of};
-    return w4_launch(ctx, "w4a16_prefill_splitk_sum", std::min<unsigned>(ceil_div(count / 4, 256), 4096), 1, 256, 0, rp);
+    void* rp[] = {&ws, &y, &nksi, &cnt, &of, &glu_i, &ni, &act};
+    return w4_launch(ctx, "w4a16_prefill_splitk_sum", std::min<unsigned>(ceil_div(count / (glu ? 8 : 4), 256), 4096), 1, 256, 0, rp);
 }
 
 // ------------------------------------------------------------------------------------------------ Gptq4::gemm
@@ -717,9 +721,19 @@ extern "C" int w4a16_lin_forward_glu_act(w4a16_ctx* ctx, const char* name, uint6
     W4_TRY(w4_find_lin(ctx, name, &L));
     if (!x_dev || !y_f16_dev || t == 0) return w4_fail(W4A16_ERR_ARG, "lin_forward_glu %s: null operand or t=0", name);
     W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
-    DecodeNorm nm;
-    nm.act = act;
-    return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t, &nm);
+    if (act != W4A16_ACT_SILU && act != W4A16_ACT_GELU_TANH)
+        return w4_fail(W4A16_ERR_ARG, "lin_forward_glu %s: activation %d (0 = silu, 1 = gelu, tanh form)", name, act);
+    if (t <= 16) {
+        DecodeNorm nm;
+        nm.act = act;
+        return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t, &nm);
+    }
+    // beyond the decode regime the same split as w4a16_lin_forward's AUTO: the weight-streaming kernel up to 64 rows
+    // (and for scales the MFMA kernel cannot divide by), the tiled MFMA GEMM above — each with the gated epilogue
+    if (L->n % 32 != 0) return w4_fail(W4A16_ERR_SHAPE, "lin_forward_glu %s: n=%zu must be a multiple of 32", name, L->n);
+    if (!L->q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "lin_forward_glu %s: linear has no tiled copy (needs k %% 128 == 0)", name);
+    if (t <= 64 || !L->scales_regular) return w4_dense_grouped(ctx, *L, x_dev, y_f16_dev, t, 1, act);
+    return launch_prefill(ctx, *L, x_dev, y_f16_dev, t, 1, act);
 }
 
 // Largest row norm of the dequantised weights (kernels/layout.hip, w4a16_row_norm_max_*), computed on the first request

@@ -71,8 +71,12 @@ __device__ __forceinline__ void moe_store(f4_t a0, f4_t a1, int slot, int q, int
         h4_t o;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float g = moe_round_f16(a0[i]), up = moe_round_f16(a1[i]);
-            o[i] = (_Float16)w4_act_mul(g, up, act_kind);
+            // expert FFN: gate and up are f16 tensors in the reference and are rounded first; a dense gated linear
+            // (bit 1 of act_kind) applies the activation to the f32 sums, like the separate element-wise kernel
+            float g = (act_kind & 2) ? a0[i] : moe_round_f16(a0[i]), up = (act_kind & 2) ? a1[i] : moe_round_f16(a1[i]);
+            float v = w4_act_mul(g, up, act_kind & 1);
+            asm volatile("" : "+v"(v));  // the product is rounded to f32 before the f16 conversion
+            o[i] = (_Float16)v;
         }
         *reinterpret_cast<h4_t*>(reinterpret_cast<_Float16*>(y) + (size_t)slot * n_ff + u * 16 + 4 * q) = o;
     } else {
@@ -113,8 +117,9 @@ __device__ __forceinline__ void moe_store(f4_t a0, f4_t a1, int slot, int q, int
 //   A segment whose expert id is outside 0..n_exp-1 is skipped (its slots stay unwritten).
 //   ws / tickets: workspace and zeroed counters of a launch split over k across workgroups (gridDim.y slices; the
 //   LDS-staged kernel only): [slice][block][wave][2*TT] partial tiles, one counter per (block, wave).
-//   act_kind (GLU only): 0 = silu(gate) * up (w4a16_moe_act_silu_f16), 1 = the tanh form of gelu on the gate
-//   (w4a16_moe_act_gelu_f16, assets/moe.cu:1635-1647).
+//   act_kind (GLU only): bit 0: 0 = silu(gate) * up (w4a16_moe_act_silu_f16), 1 = the tanh form of gelu on the gate
+//   (w4a16_moe_act_gelu_f16, assets/moe.cu:1635-1647); bit 1: gate and up enter the activation as f32 sums (a dense
+//   gated linear) instead of being rounded to f16 first (the expert FFN).
 //   wpb: waves per block (the block size, as an argument: read from the dispatch packet it costs one more dependent
 //   scalar-cache miss before the first weight load).
 #define MOE_PARAMS                                                                                                  \

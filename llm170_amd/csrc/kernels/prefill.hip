@@ -50,6 +50,14 @@ __device__ __forceinline__ float pf_ratio(float s_prev, float s_cur) {
 //     the lane that holds a gate sum holds the matching up sum; both are rounded to f16 (the reference materialises
 //     them as f16) and act[slot][c] = f16(act(gate) * up) is written, f16 [ns][n_ff];
 //   MODE 2 (down, n = hidden): y[slot][c] = sum * topw[slot] as f16 or f32 [ns][n].
+//
+// Dense gated form (MODE 3): a fused gate|up linear (rows 0..n/2 gate, n/2..n up) with the element-wise kernel that
+// follows it in the reference's prefill chain (lin_forward + ew, w4a16_dec/prefill.rs:148-207, assets/ew.cu:9-57)
+// folded into the epilogue: column pairing as in MODE 1, tile numbering and split-K as in MODE 0, and
+// y[m][c] = f16(act(g) * u) on the f32 sums g, u (f16 [t][n/2]) — the bits of the MODE 0 launch with f32 output
+// followed by w4a16_act_mul_f16, without the [t][n] f32 round trip (285 of the 419 MB a 4096-row launch moves on the
+// 27B gate|up shape).  A split launch writes f32 partials of all n columns and w4a16_prefill_splitk_sum applies the
+// activation after adding them.
 template <int MODE>
 struct PfGroup {
     const int* sorted_ids;
@@ -78,8 +86,10 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     // at a time share x slabs and weight panels through its L2.  Super-tiles are dealt round-robin to the XCDs.  The
     // host picks the super-tile shape: 8 x 8 on large grids, smaller on small ones so that every XCD gets work.
     int m0, n0;
-    if (MODE == 0) {
-        const int tiles_m = (t + PF_BM - 1) / PF_BM, tiles_n = (n + PF_BN - 1) / PF_BN;
+    constexpr bool DENSE = MODE == 0 || MODE == 3, PAIRED = MODE == 1 || MODE == 3;  // PAIRED: gate and up columns per wave
+    if (DENSE) {
+        const int tiles_m = (t + PF_BM - 1) / PF_BM,
+                  tiles_n = MODE == 3 ? ((n >> 1) + PF_BN / 2 - 1) / (PF_BN / 2) : (n + PF_BN - 1) / PF_BN;
         const int sm_n = (tiles_m + sup_m - 1) / sup_m, sn_n = (tiles_n + sup_n - 1) / sup_n;
         const int per = sup_m * sup_n;
         const int j = blockIdx.x >> 3;
@@ -88,7 +98,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
         const int tm = (super % sm_n) * sup_m + within % sup_m, tn = (super / sm_n) * sup_n + within / sup_m;
         if (tm >= tiles_m || tn >= tiles_n) return;
         m0 = tm * PF_BM;
-        n0 = tn * PF_BN;
+        n0 = tn * (MODE == 3 ? PF_BN / 2 : PF_BN);
     } else {
         // grouped: blockIdx.x = column tile (fastest, so the tiles of a segment run together and share its x rows
         // through the L2), blockIdx.y = segment.  Gate|up tiles span 128 gate and the 128 matching up columns.
@@ -102,7 +112,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
         n0 = blockIdx.x * (MODE == 1 ? PF_BN / 2 : PF_BN);
     }
 
-    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)(MODE == 0 ? t : gp.x_rows) * (unsigned)k * 2u);
+    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)(DENSE ? t : gp.x_rows) * (unsigned)k * 2u);
     const __amdgpu_buffer_rsrc_t qr = w4_make_rsrc(qt, (unsigned)row_blocks * (unsigned)kt_n * 1024u);
     const __amdgpu_buffer_rsrc_t sr = w4_make_rsrc(st, (unsigned)row_blocks * (unsigned)kg_n * 32u);
 
@@ -117,7 +127,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
 #pragma unroll
     for (int i = 0; i < MI; i++) {
         const int c = tid + i * PF_THREADS, row = c >> 3, kc = (c & 7) ^ (row & 7);
-        if (MODE == 0) {
+        if (DENSE) {
             xa_off[i] = (m0 + row < t) ? ((unsigned)(m0 + row) * (unsigned)k + (unsigned)kc * 8u) * 2u : W4_OOB;
         } else {
             const int id = gp.sorted_ids[m0 + row];  // padding rows carry the sentinel ns: zeros, never stored
@@ -125,7 +135,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
         }
     }
     int* const seg_ids = reinterpret_cast<int*>(lds_base + 2 * PF_STAGE_BYTES);
-    if (MODE != 0 && tid < PF_BM) seg_ids[tid] = gp.sorted_ids[m0 + tid];  // visible after the first barrier
+    if (!DENSE && tid < PF_BM) seg_ids[tid] = gp.sorted_ids[m0 + tid];  // visible after the first barrier
     auto load_a = [&](int s, int buf) {
 #pragma unroll
         for (int i = 0; i < MI; i++)
@@ -139,7 +149,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     unsigned q_off[2][2], s_off[2];
 #pragma unroll
     for (int ni = 0; ni < 2; ni++) {
-        const int nrow = MODE == 1 ? ni * (n >> 1) + n0 + wn * 32 + nl : n0 + wn * 64 + ni * 32 + nl;
+        const int nrow = PAIRED ? ni * (n >> 1) + n0 + wn * 32 + nl : n0 + wn * 64 + ni * 32 + nl;
         const unsigned rb = (unsigned)min(nrow >> 4, row_blocks - 1);  // rows past n re-read the last block, never stored
         const unsigned r = (unsigned)(nrow & 15);
 #pragma unroll
@@ -172,8 +182,8 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     const int a_row = nl;  // + mi * 32
     // split-K over gridDim.y (narrow outputs at moderate t, where the tile grid alone cannot fill the chip): this
     // block covers k tiles [kt_lo, kt_hi) and writes an f32 partial; a second launch adds the partials in order
-    const int kt_lo = MODE == 0 ? (kt_n * (int)blockIdx.y) / (int)gridDim.y : 0,
-              kt_hi = MODE == 0 ? (kt_n * ((int)blockIdx.y + 1)) / (int)gridDim.y : kt_n;
+    const int kt_lo = DENSE ? (kt_n * (int)blockIdx.y) / (int)gridDim.y : 0,
+              kt_hi = DENSE ? (kt_n * ((int)blockIdx.y + 1)) / (int)gridDim.y : kt_n;
     const int stages = 2 * kt_hi;
 
     load_a(2 * kt_lo, 0);
@@ -292,11 +302,30 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
         }
         return;
     }
+    if (MODE == 3 && gridDim.y == 1) {
+        const int n_ff = n >> 1, col = n0 + wn * 32 + nl;
+        if (col >= n_ff) return;
+#pragma unroll
+        for (int mi = 0; mi < MI; mi++) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int row = m0 + mi * 32 + 8 * (e >> 2) + 4 * khalf + (e & 3);
+                if (row < t) {
+                    float gt = acc[mi][0][e] * unit[0], up = acc[mi][1][e] * unit[1];
+                    asm volatile("" : "+v"(gt), "+v"(up));  // the sums are rounded to f32 as the separate launch stores them
+                    float v = w4_act_mul(gt, up, gp.act_kind);
+                    asm volatile("" : "+v"(v));  // and the product before the f16 conversion, as in the separate kernel
+                    reinterpret_cast<_Float16*>(y)[(size_t)row * n_ff + col] = (_Float16)v;
+                }
+            }
+        }
+        return;
+    }
     if (gridDim.y > 1) y = reinterpret_cast<float*>(y) + (size_t)blockIdx.y * (size_t)t * (size_t)n;  // partial (f32)
 #pragma unroll
     for (int ni = 0; ni < 2; ni++) {
-        const int col = n0 + wn * 64 + ni * 32 + nl;
-        if (col >= n) continue;
+        const int col = MODE == 3 ? ni * (n >> 1) + n0 + wn * 32 + nl : n0 + wn * 64 + ni * 32 + nl;
+        if (MODE == 3 ? n0 + wn * 32 + nl >= (n >> 1) : col >= n) continue;
 #pragma unroll
         for (int mi = 0; mi < MI; mi++) {
 #pragma unroll
@@ -319,6 +348,17 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
         const u4_t* qt, const uint16_t* st, const uint16_t* x, void* y, int row_blocks, int k, int n, int t,          \
         int out_f16, int sup_m, int sup_n) {                                                                           \
         prefill_body<G, SBF, MI>(qt, st, x, y, row_blocks, k, n, t, out_f16, sup_m, sup_n);                            \
+    }
+
+// Dense gated kernels: the arguments of PREFILL_KERNEL plus the activation (W4A16_ACT_*); y is f16 [t][n/2], or the f32
+// partials [slices][t][n] of a split launch.
+#define PREFILL_GLU_KERNEL(NAME, G, SBF, MI, WPE)                                                                  \
+    extern "C" __global__ __launch_bounds__(PF_THREADS) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(      \
+        const u4_t* qt, const uint16_t* st, const uint16_t* x, void* y, int row_blocks, int k, int n, int t,          \
+        int out_f16, int sup_m, int sup_n, int act_kind) {                                                             \
+        PfGroup<3> gp;                                                                                                 \
+        gp.act_kind = act_kind;                                                                                        \
+        prefill_body<G, SBF, MI, 3>(qt, st, x, y, row_blocks, k, n, t, out_f16, sup_m, sup_n, gp);                     \
     }
 
 // Grouped kernels for the expert FFN: same arguments as the streaming grouped kernels of moe.hip (blk must be 64, the
@@ -347,8 +387,32 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     }
 
 // y[i] = sum over the nks partials of a split-K launch, added in split order in f32; f32 or f16 out.
+// glu != 0: the partials are those of a fused gate|up linear, [slices][t][n]; y is f16 [t][n/2] = act(g) * u on the
+// summed gate and up columns (act_kind as in w4_act_mul), the same arithmetic as the unsplit gated epilogue.
 extern "C" __global__ __launch_bounds__(256) void w4a16_prefill_splitk_sum(const float* __restrict__ part, void* __restrict__ y,
-                                                                           int nks, size_t count, int out_f16) {
+                                                                           int nks, size_t count, int out_f16, int glu,
+                                                                           int n, int act_kind) {
+    if (glu) {
+        const size_t n_ff = (size_t)(n >> 1), q_ff = n_ff / 4, total = (count / (size_t)n) * q_ff;  // n_ff % 4 == 0 (host)
+        for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+            const size_t row = i / q_ff, c4 = i - row * q_ff;
+            const float* pg = part + row * (size_t)n + c4 * 4;
+            f4_t g = *reinterpret_cast<const f4_t*>(pg), u = *reinterpret_cast<const f4_t*>(pg + n_ff);
+            for (int ks = 1; ks < nks; ks++) {
+                g += *reinterpret_cast<const f4_t*>(pg + (size_t)ks * count);
+                u += *reinterpret_cast<const f4_t*>(pg + (size_t)ks * count + n_ff);
+            }
+            h4_t o;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float v = w4_act_mul(g[j], u[j], act_kind);
+                asm volatile("" : "+v"(v));
+                o[j] = (_Float16)v;
+            }
+            reinterpret_cast<h4_t*>(y)[row * q_ff + c4] = o;
+        }
+        return;
+    }
     const size_t n4 = count / 4;  // count = t*n with n % 4 == 0 is guaranteed by the host
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) {
         f4_t a = reinterpret_cast<const f4_t*>(part)[i];
@@ -370,6 +434,14 @@ PREFILL_KERNEL(w4a16_prefill_g128_f16_m64, 128, false, 2, 3)
 PREFILL_KERNEL(w4a16_prefill_g128_bf16_m64, 128, true, 2, 3)
 PREFILL_KERNEL(w4a16_prefill_g32_f16_m64, 32, false, 2, 3)
 PREFILL_KERNEL(w4a16_prefill_g32_bf16_m64, 32, true, 2, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_f16_glu, 128, false, 4, 2)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_bf16_glu, 128, true, 4, 2)
+PREFILL_GLU_KERNEL(w4a16_prefill_g32_f16_glu, 32, false, 4, 2)
+PREFILL_GLU_KERNEL(w4a16_prefill_g32_bf16_glu, 32, true, 4, 2)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_f16_m64_glu, 128, false, 2, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_bf16_m64_glu, 128, true, 2, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g32_f16_m64_glu, 32, false, 2, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g32_bf16_m64_glu, 32, true, 2, 3)
 PREFILL_MOE_KERNEL(w4a16_moe_g128_f16_pf_glu, 128, false, 1)
 PREFILL_MOE_KERNEL(w4a16_moe_g128_f16_pf_lin, 128, false, 2)
 PREFILL_MOE_KERNEL(w4a16_moe_g128_bf16_pf_glu, 128, true, 1)

@@ -113,6 +113,56 @@ def test_fused_glu_equals_linear_then_silu_mul(dec, orc, n, k, group, bf16, t):
     assert np.mean(got == want) > 0.97
 
 
+@pytest.mark.parametrize("n,k,group,bf16,t", [
+    (34816, 5120, 128, False, 64), (34816, 5120, 128, False, 512), (34816, 5120, 128, False, 4096),
+    (34816, 5120, 128, False, 17), (34816, 5120, 128, False, 1000),
+    (1024, 2048, 32, True, 40), (1024, 2048, 32, True, 300), (5120, 17408, 128, False, 512), (2080, 512, 128, False, 130)])
+def test_fused_glu_beyond_the_decode_regime(dec, orc, n, k, group, bf16, t):
+    """w4a16_lin_forward_glu at 17..64 rows (weight-streaming kernel) and above (MFMA tiles, both block tiles, split-K
+    on the narrow shape, ragged last tiles): the bits of the plain launch on the same path followed by the
+    element-wise kernel (the reference's prefill chain runs exactly that pair, w4a16_dec/prefill.rs:148-207 +
+    assets/ew.cu:9-32), and a seeded sample against the oracle's silu_mul of the lane GEMM."""
+    say("glu beyond decode", n, k, group, bf16, t)
+    q, s, x = gen.make_linear(n, k, group, t, seed=73)
+    if bf16:
+        s = (gen.f16_bits_to_f32(s).view(np.uint32) >> 16).astype(np.uint16)
+    dec.upload_lin_g("glu", q, s, n, k, group, bf16)
+    cc = dec.cc
+    px, pg, pa, pb = cc.to_device(x), cc.alloc(t * n * 4), cc.alloc(t * (n // 2) * 2), cc.alloc(t * (n // 2) * 2)
+    path = ops.PATH_STREAM if t <= 64 else ops.PATH_PREFILL
+    if t <= 64:
+        dec.set_decode_ksplit(-1)  # the gated streaming kernel never splits over k: same summation order for the pair
+    try:
+        dec.lin_forward("glu", px, pg, t, path=path)
+    finally:
+        dec.set_decode_ksplit(0)
+    want_sym = cc.last_launch_symbol()
+    dec.silu_mul_f16(pg, n // 2, t, pa)
+    dec.lin_forward_glu("glu", px, pb, t)
+    got_sym = cc.last_launch_symbol()
+    say("   plain:", want_sym, "gated:", got_sym)
+    two, one = cc.d2h(pa, (t, n // 2), np.uint16), cc.d2h(pb, (t, n // 2), np.uint16)
+    if t > 64 and "splitk" not in want_sym:
+        assert got_sym.endswith("_glu") and got_sym[:-4] == want_sym
+    assert np.array_equal(one, two)
+    # gelu on the same launch shape
+    dec.act_mul_f16(pg, n // 2, t, pa, gelu=True)
+    dec.lin_forward_glu("glu", px, pb, t, gelu=True)
+    assert np.array_equal(cc.d2h(pb, (t, n // 2), np.uint16), cc.d2h(pa, (t, n // 2), np.uint16))
+    for p in (px, pg, pa, pb):
+        cc.free(p)
+    cols = (gen.stream(93, 3000) % np.uint64(n // 2)).astype(np.uint32)
+    toks = (gen.stream(94, 3000) % np.uint64(t)).astype(np.uint32)
+    gate = orc.gemm_lane_sample(x, q, s, k, group, cols, toks, bf16)
+    up = orc.gemm_lane_sample(x, q, s, k, group, cols + np.uint32(n // 2), toks, bf16)
+    want = orc.silu_mul_f16_rows(np.stack([gate, up], axis=1).reshape(-1, 2))[:, 0]
+    got = one[toks, cols]
+    a, b = _f16(got).astype(np.float64), _f16(want).astype(np.float64)
+    rms = float(np.sqrt(np.mean(b * b)))
+    assert np.all(np.abs(a - b) <= 2 * parity.f16_ulp(np.maximum(np.abs(b), rms / parity.CLAMP_DIV)))
+    assert np.mean(got == want) > 0.97
+
+
 @pytest.mark.parametrize("n,k,group,t", [(1024, 256, 128, 1), (2048, 512, 32, 5), (1024, 256, 128, 16),
                                          (34816, 5120, 128, 4)])
 def test_fused_glu_gelu(dec, orc, n, k, group, t):
@@ -151,9 +201,13 @@ def test_fused_glu_errors(dec):
     dec.upload_lin_synth("glu_odd", 48, 256, 128, 1, 2)  # n = 48: halves are not whole row blocks
     with pytest.raises(ops.W4a16Error):
         dec.lin_forward_glu("glu_odd", 1, 1, 1)
+    with pytest.raises(ops.W4a16Error):
+        dec.lin_forward_glu("glu_odd", 1, 1, 17)  # the same contract beyond the decode regime (refused before any launch)
     dec.upload_lin_synth("glu_ok", 64, 256, 128, 1, 2)
     with pytest.raises(ops.W4a16Error):
-        dec.lin_forward_glu("glu_ok", 1, 1, 17)
+        dec.lin_forward_glu("glu_ok", 1, 1, 0)
+    with pytest.raises(ops.W4a16Error):
+        dec.lin_forward_glu("glu_ok", 0, 1, 17)  # null operand
 
 
 # ------------------------------------------------------------------ the chain
@@ -239,6 +293,37 @@ def test_chain_small_many_layers(dec, orc, t):
     assert m["rel_l2"] < 2e-2  # rounding flips of f16 intermediates accumulate over 96 linears
     ms, _ = dec.bench_chain("small", layers, px, t, py, reps=3, warmup=1, use_graph=True)
     assert np.array_equal(cc.d2h(py, (t, hidden), np.uint16), staged)  # graph replays give the same bits
+    cc.free(px)
+    cc.free(py)
+
+
+@pytest.mark.parametrize("t", [40, 200])
+def test_chain_prefill_regime(dec, orc, t):
+    """The chain at prefill row counts (reference: chain_t_sel / forward_prefill, w4a16_dec/prefill.rs:81-207,
+    graphs.rs:368): 40 rows run the weight-streaming kernels, 200 the MFMA tiles; gate|up carries the SiLU*up epilogue
+    in both.  Stage-wise parity against the oracle, the one-call chain equal to the staged run bit for bit, and the
+    end-to-end result close to the oracle's independent run."""
+    say("chain prefill regime", t)
+    hidden, n_qkv, n_ff, group, layers = 256, 384, 512, 128, 6
+    shapes = {"attn_qkv": (n_qkv, hidden), "attn_output": (hidden, hidden), "ffn_gate_up": (2 * n_ff, hidden),
+              "ffn_down": (hidden, n_ff)}
+    seeds = dec.upload_chain_synth("pfc", layers, hidden, n_qkv, n_ff, group)
+    x = gen.normal_f16(57 + t, (t, hidden))
+    cc = dec.cc
+    # the gated streaming kernel never splits over k; the staged run's plain gate|up launch must sum in the same order
+    dec.set_decode_ksplit(-1)
+    try:
+        staged = _chain_stagewise(dec, orc, "pfc", seeds, shapes, group, layers, t, x, 8)
+        px, py = cc.to_device(x), cc.alloc(t * hidden * 2)
+        dec.chain_forward("pfc", 0, layers, px, t, py)
+        got = cc.d2h(py, (t, hidden), np.uint16)
+    finally:
+        dec.set_decode_ksplit(0)
+    assert np.array_equal(got, staged)
+    want = _chain_oracle(orc, "pfc", seeds, shapes, group, layers, x, 8)
+    m = parity.compare(_f16(got), _f16(want))
+    say("  end to end rel_l2", m["rel_l2"], "identical", float(np.mean(got == want)))
+    assert m["rel_l2"] < 1e-2
     cc.free(px)
     cc.free(py)
 
