@@ -287,7 +287,7 @@ def plan_sweep(out_path):
         time_forward(dec, names, xd, yd, max(PLAN_SWEEP_T), 30, 0, ops.PATH_PREFILL)
         for t in PLAN_SWEEP_T:
             rows = []
-            for tile in (64, 128):
+            for tile in (64, 96, 128):
                 for ks in (1, 2, 3, 4, 6, 8):
                     if ks > 1 and ks > (k // 128) // 4:
                         continue

@@ -179,7 +179,7 @@ int w4a16_lin_forward(w4a16_ctx* ctx, const char* name, uint64_t x_dev, uint64_t
  * kernel of w4a16_lin_forward_glu.  Out pointers may be NULL. */
 int w4a16_plan_decode(size_t n, size_t k, size_t group, size_t t, int cu_count, int glu, int* rows_per_wave,
                       int* waves_per_block, int* k_slices, size_t* lds_bytes);
-/* The launch plan of the prefill path (W4A16_PATH_PREFILL) for t rows: out = {block tile rows (64 or 128), k slices,
+/* The launch plan of the prefill path (W4A16_PATH_PREFILL) for t rows: out = {block tile rows (64, 96 or 128), k slices,
  * super-tile rows, super-tile columns, super-tile count}; `tile_rows` and `k_slices` pin a choice as
  * w4a16_set_prefill_tile / w4a16_set_prefill_ksplit do (0 = automatic); *price_us (may be NULL) receives the model's
  * estimate for the chosen plan.  Role of the reference's per-problem choice of thread-block shape
@@ -306,7 +306,7 @@ int w4a16_set_decode_ksplit(w4a16_ctx* ctx, int ksplit);
  * idle — narrow outputs at moderate t; the reference's prefill path makes the same choice inside its vendored GEMM),
  * -1 = never, n >= 1 = exactly n k slices (clamped so a slice has at least 4 k tiles). */
 int w4a16_set_prefill_ksplit(w4a16_ctx* ctx, int ksplit);
-/* Rows of the prefill kernel's block tile: 0 = automatic (64 up to 192 rows, else 128), 64 or 128.  The reference's
+/* Rows of the prefill kernel's block tile: 0 = automatic (priced with the k slices, w4a16_plan_prefill), 64, 96 or 128.  The reference's
  * vendored GEMM picks its thread-block shape per problem the same way (marlin_gemm_try, kernels/marlin.rs:94-213). */
 int w4a16_set_prefill_tile(w4a16_ctx* ctx, int rows);
 

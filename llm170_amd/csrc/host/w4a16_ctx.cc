@@ -70,6 +70,9 @@ static const char* const kPrefillSyms[] = {"w4a16_prefill_g128_f16", "w4a16_pref
                                            "w4a16_prefill_g128_f16_glu", "w4a16_prefill_g128_bf16_glu", "w4a16_prefill_g32_f16_glu",
                                            "w4a16_prefill_g32_bf16_glu", "w4a16_prefill_g128_f16_m64_glu", "w4a16_prefill_g128_bf16_m64_glu",
                                            "w4a16_prefill_g32_f16_m64_glu", "w4a16_prefill_g32_bf16_m64_glu",
+                                           "w4a16_prefill_g128_f16_m96", "w4a16_prefill_g128_bf16_m96", "w4a16_prefill_g32_f16_m96",
+                                           "w4a16_prefill_g32_bf16_m96", "w4a16_prefill_g128_f16_m96_glu", "w4a16_prefill_g128_bf16_m96_glu",
+                                           "w4a16_prefill_g32_f16_m96_glu", "w4a16_prefill_g32_bf16_m96_glu",
                                            "w4a16_moe_g128_f16_pf_glu", "w4a16_moe_g128_f16_pf_lin", "w4a16_moe_g128_bf16_pf_glu",
                                            "w4a16_moe_g128_bf16_pf_lin", "w4a16_moe_g32_f16_pf_glu", "w4a16_moe_g32_f16_pf_lin",
                                            "w4a16_moe_g32_bf16_pf_glu", "w4a16_moe_g32_bf16_pf_lin", nullptr};

@@ -312,8 +312,8 @@ static int launch_decode_glu(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_
 
 // Launch plan of the prefill GEMM (kernels/prefill.hip): a pure function of (t, n, k), the CU count and the pinned
 // settings, so that a CPU test can pin what it chooses at the layer shapes (w4a16_plan_prefill).
-// Block tile 128 x 256 (two workgroups per CU) or 64 x 256 (three per CU, 64 accumulator registers), the k range whole
-// or cut into 2, 3, 4, 6 or 8 slices (split-K: f32 partials in a context-owned workspace, added in slice order by a
+// Block tile 128 x 256 (two workgroups per CU), 96 x 256 or 64 x 256 (three per CU, 96 / 64 accumulator registers), the
+// k range whole or cut into 2, 3, 4, 6 or 8 slices (split-K: f32 partials in a context-owned workspace, added in slice order by a
 // second launch — deterministic), and the super-tile shape: every combination is priced and the cheapest runs.
 struct PrefillSuper {
     size_t sup_m, sup_n, supers, load;
@@ -356,16 +356,20 @@ static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t cus, int ti
     // measurements and were then fitted to a sweep of tile x slices over 108 (n, k, t) shapes (nine linears, t = 128
     // to 4096), minimising the time lost against the best choice of the sweep: 0.8 % lost on average, 9 % at worst,
     // where the earlier rule (generations x slice length x a tile factor, slices by doubling) lost 3 % and 22 %; fitted
-    // on four of the linears only it lost 0.9 % / 11 % on the other five.
+    // on four of the linears only it lost 0.9 % / 11 % on the other five.  The 96-row tile joined later with constants of
+    // its own fitted to a sweep of that tile over the same 108 shapes (the others kept): the plans gain 0.5 % on average,
+    // up to 14 % where its grid fills the generations better (11008 x 4096 at t = 1536, 17408 x 5120 at t = 1024,
+    // 5120 x 34816 at t = 1024: 4 %), and lose at most 3 % against the two-tile plans.
     auto us_per_k_tile = [](size_t rows, double per_cu) {
         static const double at[7] = {0.0, 0.5, 1.0, 1.5, 2.0, 2.5, 3.0};
-        static const double part64[7] = {1.0, 1.006, 1.595, 1.738, 1.95, 2.552, 2.903}, part128[5] = {1.5, 1.6, 2.416, 2.9, 3.37};
-        const double c = rows == 64 ? 3.0 : 2.0, full = rows == 64 ? 2.745 : 3.497;
-        const double* part = rows == 64 ? part64 : part128;
+        static const double part64[7] = {1.0, 1.006, 1.595, 1.738, 1.95, 2.552, 2.903}, part128[5] = {1.5, 1.6, 2.416, 2.9, 3.37},
+                            part96[7] = {1.25, 1.258, 1.994, 2.494, 2.729, 3.787, 4.077};
+        const double c = rows == 128 ? 2.0 : 3.0, full = rows == 64 ? 2.745 : rows == 96 ? 4.126 : 3.497;
+        const double* part = rows == 64 ? part64 : rows == 96 ? part96 : part128;
         const double gens = std::floor(per_cu / c), rem = per_cu - gens * c;
         double us = gens * full;
         if (rem > 1e-9) {
-            const int last = rows == 64 ? 6 : 4;
+            const int last = rows == 128 ? 4 : 6;
             int i = 1;
             while (i < last && rem > at[i]) i++;
             us += part[i - 1] + (part[i] - part[i - 1]) * (rem - at[i - 1]) / (at[i] - at[i - 1]);
@@ -373,7 +377,7 @@ static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t cus, int ti
         return us;
     };
     PrefillPlan best{128, 1, PrefillSuper{1, 1, 0, 0}, 1e30};
-    for (size_t rows : {(size_t)128, (size_t)64}) {
+    for (size_t rows : {(size_t)128, (size_t)96, (size_t)64}) {
         if (tile_m_forced && (size_t)tile_m_forced != rows) continue;
         const size_t tiles_m = (t + rows - 1) / rows;
         const PrefillSuper sup = super_for(tiles_m);
@@ -384,7 +388,7 @@ static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t cus, int ti
             if (ksplit_forced < 0 && nks != 1) continue;
             if (!forced && nks > 1 && (n % (glu ? 8 : 4) != 0 || nks > kt_n / 4)) continue;
             const double per_cu = (double)(sup.load * nks) * 8.0 / (double)cus;  // of the busiest XCD
-            const double gens = std::ceil(per_cu / (rows == 64 ? 3.0 : 2.0));
+            const double gens = std::ceil(per_cu / (rows == 128 ? 2.0 : 3.0));
             double us = (double)((kt_n + nks - 1) / nks) * us_per_k_tile(rows, per_cu) + 5.7 * gens;
             if (nks > 1) us += 6.0 + (double)nks * (double)t * (double)n * 8.0 / 9.76e6;
             if (us < best.us) best = PrefillPlan{rows, nks, sup, us};
@@ -396,7 +400,7 @@ static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t cus, int ti
 extern "C" int w4a16_plan_prefill(size_t t, size_t n, size_t k, int cu_count, int tile_rows, int k_slices, size_t out[5],
                                   double* price_us) {
     if (t == 0 || n == 0 || k == 0 || k % 128 != 0 || cu_count <= 0 || !out ||
-        (tile_rows != 0 && tile_rows != 64 && tile_rows != 128) || k_slices < -1 || k_slices > 16)
+        (tile_rows != 0 && tile_rows != 64 && tile_rows != 96 && tile_rows != 128) || k_slices < -1 || k_slices > 16)
         return w4_fail(W4A16_ERR_ARG, "plan_prefill: t=%zu n=%zu k=%zu cus=%d tile=%d slices=%d", t, n, k, cu_count, tile_rows, k_slices);
     const PrefillPlan P = plan_prefill(t, n, k, (size_t)cu_count, tile_rows, k_slices);
     out[0] = P.bm;
@@ -433,7 +437,7 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     const size_t bm = plan.bm, nks = plan.nks, sup_m = plan.sup.sup_m, sup_n = plan.sup.sup_n, supers = plan.sup.supers;
     const size_t grid = ((supers + 7) / 8) * (sup_m * sup_n) * 8;
     char sym[64];
-    snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s%s%s", L.group, L.scale_bf16 ? "bf16" : "f16", bm == 64 ? "_m64" : "", glu ? "_glu" : "");
+    snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s%s%s", L.group, L.scale_bf16 ? "bf16" : "f16", bm == 64 ? "_m64" : bm == 96 ? "_m96" : "", glu ? "_glu" : "");
     const unsigned shmem = (unsigned)(2 * bm * kW4PfKs * 2);  // two stages of bm rows x PF_KS halves
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = (out_f16 || glu) ? 1 : 0;
@@ -891,7 +895,7 @@ extern "C" int w4a16_set_decode_shape(w4a16_ctx* ctx, int rows_per_wave, int wav
 
 extern "C" int w4a16_set_prefill_tile(w4a16_ctx* ctx, int rows) {
     if (!ctx) return w4_fail(W4A16_ERR_ARG, "set_prefill_tile: null context");
-    if (rows != 0 && rows != 64 && rows != 128) return w4_fail(W4A16_ERR_ARG, "set_prefill_tile: 0 = automatic, 64 or 128 rows");
+    if (rows != 0 && rows != 64 && rows != 96 && rows != 128) return w4_fail(W4A16_ERR_ARG, "set_prefill_tile: 0 = automatic, 64, 96 or 128 rows");
     ctx->prefill_tile_m = rows;
     return 0;
 }

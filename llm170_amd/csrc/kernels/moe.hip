@@ -682,62 +682,69 @@ MOE_FAMILY(w4a16_moe_g128_f16, 128, false, 4)
 MOE_FAMILY(w4a16_moe_g128_bf16, 128, true, 4)
 
 // ---------------------------------------------------------------------------------------------------- routing
-// Softmax over all experts, k largest probabilities with ties to the lower index, weights renormalised by the
-// selected sum (w4a16_dec/mod.rs:168-185; device counterpart assets/moe.cu:686-759).  One wave per token, n <= 1024.
+// Routing rule of the reference (w4a16_dec/mod.rs:168-185, device counterpart assets/moe.cu:686-759): softmax over all
+// experts, the k largest probabilities with ties to the lower index, weights renormalised by the selected sum.
+// One wave per token, n <= 1024 (16 experts per lane).  Selection runs on ONE unique, totally ordered 64-bit key per
+// expert — the probability's bit pattern (monotone for non-negative floats) above the complement of the expert index —
+// so "larger probability, then lower index" is a plain unsigned maximum: a round takes the lane's largest key, a
+// butterfly of unsigned maxima over the wave, and retires the winner by comparing keys (0 = absent or taken; no real
+// key is 0 because index complements are non-zero).
+__device__ __forceinline__ unsigned long long topk_wave_max(unsigned long long v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned lo = __shfl_xor((unsigned)v, off), hi = __shfl_xor((unsigned)(v >> 32), off);
+        const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
 extern "C" __global__ __launch_bounds__(256) void w4a16_moe_topk_t(const float* __restrict__ lg, int* __restrict__ idx,
                                                                    float* __restrict__ wt, int t, int n, int k) {
+    constexpr int PER_LANE = 16;
     const int lane = threadIdx.x & 63;
-    const int ti = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (ti >= t) return;
-    const float* l = lg + (size_t)ti * n;
-    float pv[16];
-    float mx = -INFINITY;
+    const int token = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (token >= t) return;
+    const float* logits = lg + (size_t)token * n;
+    float e[PER_LANE];
+    float top = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < 16; j++) {
+    for (int j = 0; j < PER_LANE; j++) {
         const int i = lane + 64 * j;
-        pv[j] = i < n ? l[i] : -INFINITY;
-        mx = fmaxf(mx, pv[j]);
+        e[j] = i < n ? logits[i] : -INFINITY;
+        top = fmaxf(top, e[j]);
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    float sum = 0.f;
+    for (int off = 32; off > 0; off >>= 1) top = fmaxf(top, __shfl_xor(top, off));
+    float total = 0.f;
 #pragma unroll
-    for (int j = 0; j < 16; j++) {
-        pv[j] = (lane + 64 * j) < n ? expf(pv[j] - mx) : -1.0f;  // -1 marks absent or already taken
-        if (pv[j] > 0.f) sum += pv[j];
+    for (int j = 0; j < PER_LANE; j++) {
+        e[j] = lane + 64 * j < n ? expf(e[j] - top) : 0.f;
+        total += e[j];  // lane-local sum in index order, then the butterfly: the order the host statement follows too
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+    for (int off = 32; off > 0; off >>= 1) total += __shfl_xor(total, off);
+    unsigned long long key[PER_LANE];
 #pragma unroll
-    for (int j = 0; j < 16; j++)
-        if (pv[j] >= 0.f) pv[j] = pv[j] / sum;
-    float wsum = 0.f, mine = 0.f;  // lane r keeps the r-th selected probability
+    for (int j = 0; j < PER_LANE; j++) {
+        const unsigned i = (unsigned)(lane + 64 * j);
+        const float p = e[j] / total;
+        key[j] = i < (unsigned)n ? ((unsigned long long)__builtin_bit_cast(unsigned, p) << 32) | (unsigned long long)(~i) : 0ull;
+    }
+    float chosen_sum = 0.f, kept = 0.f;  // lane r keeps the r-th chosen probability (k <= 64)
     for (int r = 0; r < k; r++) {
-        float bv = -1.0f;
-        int bi = 0x7fffffff;
+        unsigned long long best = 0ull;
 #pragma unroll
-        for (int j = 0; j < 16; j++)
-            if (pv[j] > bv) {  // strict: the lower index wins inside a lane
-                bv = pv[j];
-                bi = lane + 64 * j;
-            }
+        for (int j = 0; j < PER_LANE; j++) best = key[j] > best ? key[j] : best;
+        best = topk_wave_max(best);
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ov = __shfl_xor(bv, off);
-            const int oi = __shfl_xor(bi, off);
-            if (ov > bv || (ov == bv && oi < bi)) {
-                bv = ov;
-                bi = oi;
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < 16; j++)
-            if (lane + 64 * j == bi) pv[j] = -1.0f;
-        if (lane == 0) idx[(size_t)ti * k + r] = bi;
-        if (lane == (r & 63)) mine = bv;
-        wsum += bv;
+        for (int j = 0; j < PER_LANE; j++) key[j] = key[j] == best ? 0ull : key[j];
+        const float p = __builtin_bit_cast(float, (unsigned)(best >> 32));
+        if (lane == 0) idx[(size_t)token * k + r] = (int)(~(unsigned)best);
+        kept = lane == r ? p : kept;
+        chosen_sum += p;
     }
-    if (lane < k) wt[(size_t)ti * k + lane] = mine / wsum;
+    if (lane < k) wt[(size_t)token * k + lane] = kept / chosen_sum;
 }
 
 // Stable counting sort of slots by expert with every expert's run padded to a multiple of `block`

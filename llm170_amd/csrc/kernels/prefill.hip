@@ -434,6 +434,10 @@ PREFILL_KERNEL(w4a16_prefill_g128_f16_m64, 128, false, 2, 3)
 PREFILL_KERNEL(w4a16_prefill_g128_bf16_m64, 128, true, 2, 3)
 PREFILL_KERNEL(w4a16_prefill_g32_f16_m64, 32, false, 2, 3)
 PREFILL_KERNEL(w4a16_prefill_g32_bf16_m64, 32, true, 2, 3)
+PREFILL_KERNEL(w4a16_prefill_g128_f16_m96, 128, false, 3, 3)
+PREFILL_KERNEL(w4a16_prefill_g128_bf16_m96, 128, true, 3, 3)
+PREFILL_KERNEL(w4a16_prefill_g32_f16_m96, 32, false, 3, 3)
+PREFILL_KERNEL(w4a16_prefill_g32_bf16_m96, 32, true, 3, 3)
 PREFILL_GLU_KERNEL(w4a16_prefill_g128_f16_glu, 128, false, 4, 2)
 PREFILL_GLU_KERNEL(w4a16_prefill_g128_bf16_glu, 128, true, 4, 2)
 PREFILL_GLU_KERNEL(w4a16_prefill_g32_f16_glu, 32, false, 4, 2)
@@ -442,6 +446,10 @@ PREFILL_GLU_KERNEL(w4a16_prefill_g128_f16_m64_glu, 128, false, 2, 3)
 PREFILL_GLU_KERNEL(w4a16_prefill_g128_bf16_m64_glu, 128, true, 2, 3)
 PREFILL_GLU_KERNEL(w4a16_prefill_g32_f16_m64_glu, 32, false, 2, 3)
 PREFILL_GLU_KERNEL(w4a16_prefill_g32_bf16_m64_glu, 32, true, 2, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_f16_m96_glu, 128, false, 3, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_bf16_m96_glu, 128, true, 3, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g32_f16_m96_glu, 32, false, 3, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g32_bf16_m96_glu, 32, true, 3, 3)
 PREFILL_MOE_KERNEL(w4a16_moe_g128_f16_pf_glu, 128, false, 1)
 PREFILL_MOE_KERNEL(w4a16_moe_g128_f16_pf_lin, 128, false, 2)
 PREFILL_MOE_KERNEL(w4a16_moe_g128_bf16_pf_glu, 128, true, 1)

@@ -15,21 +15,22 @@ QUANT = {"quant_method": "compressed-tensors", "format": "pack-quantized",
 
 
 def write_safetensors(path, tensors, metadata=True):
-    """tensors: {name: (dtype string, shape list, bytes)}"""
-    entries, blob, off = {}, bytearray(), 0
-    for name in sorted(tensors):
-        dtype, shape, data = tensors[name]
-        entries[name] = {"dtype": dtype, "shape": list(shape), "data_offsets": [off, off + len(data)]}
-        blob += data
-        off += len(data)
-    hdr = dict(entries)
-    if metadata:
-        hdr = {"__metadata__": {"format": "pt"}, **entries}
-    hb = json.dumps(hdr).encode()
-    with open(path, "wb") as f:
-        f.write(struct.pack("<Q", len(hb)))
-        f.write(hb)
-        f.write(bytes(blob))
+    """tensors: {name: (dtype string, shape list, bytes)}.  The archive layout (u64 header length, JSON header whose
+    entries give each tensor's byte range in the data section, then the data section) is the container's definition;
+    tensors are laid out in name order, each range derived from the running sizes."""
+    order = sorted(tensors)
+    ends = np.cumsum([len(tensors[name][2]) for name in order]).tolist()
+    starts = [0] + ends[:-1]
+    header = {"__metadata__": {"format": "pt"}} if metadata else {}
+    for name, lo, hi in zip(order, starts, ends):
+        dtype, shape, _ = tensors[name]
+        header[name] = {"dtype": dtype, "shape": [int(d) for d in shape], "data_offsets": [int(lo), int(hi)]}
+    text = json.dumps(header, separators=(",", ":")).encode("utf-8")
+    with open(path, "wb") as out:
+        out.write(len(text).to_bytes(8, "little"))
+        out.write(text)
+        for name in order:
+            out.write(tensors[name][2])
 
 
 def linear_tensors(base, n, k, group, bf16=False, seed=1):

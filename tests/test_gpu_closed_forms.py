@@ -77,7 +77,7 @@ def test_power_of_two_operands_give_the_exact_product(dec, n, k, t, what):
     if what == "prefill":
         runs = []
         try:
-            for tile in (64, 128):
+            for tile in (64, 96, 128):
                 for ks in (-1, 0, 2):  # unsplit, automatic, two k slices
                     dec.set_prefill_tile(tile)
                     dec.set_prefill_ksplit(ks)

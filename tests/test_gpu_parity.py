@@ -311,8 +311,8 @@ def test_stream_path_matches_oracle(dec, orc, n, k, group, bf16, t):
 
 @pytest.mark.parametrize("n,k,group,t", [(272, 384, 128, 70), (1000, 512, 128, 300), (512, 256, 32, 100), (2048, 2048, 128, 129)])
 def test_prefill_block_tiles_agree(dec, orc, n, k, group, t):
-    """64-row and 128-row block tiles: every output element sees the same sequence of MFMAs and rescales, so the two
-    give the same bits (unsplit), and both meet the contract against the oracle."""
+    """64-, 96- and 128-row block tiles: every output element sees the same sequence of MFMAs and rescales, so the
+    three give the same bits (unsplit), and all meet the contract against the oracle."""
     say("prefill tiles", n, k, group, t)
     q, s, x = gen.make_linear(n, k, group, t, seed=27)
     dec.upload_lin_g("pft", q, s, n, k, group, False)
@@ -323,21 +323,22 @@ def test_prefill_block_tiles_agree(dec, orc, n, k, group, t):
     out = {}
     try:
         dec.set_prefill_ksplit(-1)
-        for rows in (64, 128):
+        for rows in (64, 96, 128):
             dec.set_prefill_tile(rows)
             out[rows] = _device_forward(dec, "pft", x, t, ops.PATH_PREFILL)
             parity.assert_close(out[rows], want, "prefill tile %d" % rows)
             assert np.array_equal(_device_forward(dec, "pft", x, t, ops.PATH_PREFILL, out_f16=True),
                                   gen.f32_to_f16_bits(out[rows]))
         dec.set_prefill_ksplit(2)
-        dec.set_prefill_tile(64)
-        parity.assert_close(_device_forward(dec, "pft", x, t, ops.PATH_PREFILL), want, "prefill tile 64 split")
+        for rows in (64, 96):
+            dec.set_prefill_tile(rows)
+            parity.assert_close(_device_forward(dec, "pft", x, t, ops.PATH_PREFILL), want, "prefill tile %d split" % rows)
     finally:
         dec.set_prefill_tile(0)
         dec.set_prefill_ksplit(0)
-    assert np.array_equal(_bits(out[64]), _bits(out[128]))
+    assert np.array_equal(_bits(out[64]), _bits(out[128])) and np.array_equal(_bits(out[96]), _bits(out[128]))
     with pytest.raises(ops.W4a16Error):
-        dec.set_prefill_tile(96)
+        dec.set_prefill_tile(100)
 
 
 @pytest.mark.parametrize("n,k,t", [(34816, 5120, 512), (5120, 17408, 512), (34816, 5120, 4096), (34816, 5120, 1024),

@@ -47,10 +47,11 @@ def test_prefill_plan_super_tiles_cover_the_grid_and_pins_are_honoured():
         assert p["supers"] == sm * sn and 1 <= p["super_m"] <= 8 and p["super_n"] in (1, 2, 4, 8)
         assert p["k_slices"] == 1 or p["k_slices"] <= (k // 128) // 4
     assert ops.plan_prefill(4096, 34816, 5120, tile_rows=64)["tile_rows"] == 64
+    assert ops.plan_prefill(4096, 34816, 5120, tile_rows=96)["tile_rows"] == 96
     assert ops.plan_prefill(4096, 34816, 5120, k_slices=-1)["k_slices"] == 1
     assert ops.plan_prefill(512, 5120, 17408, k_slices=4)["k_slices"] == 4
     with pytest.raises(ops.W4a16Error):
-        ops.plan_prefill(512, 5120, 17408, tile_rows=96)
+        ops.plan_prefill(512, 5120, 17408, tile_rows=100)
 
 
 def test_decode_plan_at_the_layer_shapes():
