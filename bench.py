@@ -253,7 +253,26 @@ def bench_chain(dec, gen, ops, args):
                          "GBps": round(b / (ms * 1e-3) / 1e9, 1)})
     for p_ in (px, py, xw, yw):
         cc.free(p_)
+    # the same layers in the prefill regime (reference: chain_t_sel / forward_prefill, w4a16_dec/prefill.rs:81-207):
+    # 8 layers at M = 1024, the chain with its normalisation launches (gate|up carries SiLU*up in its epilogue) and
+    # the chain with the normalisations deferred across the MFMA-tiled linears
+    tp, lp = 1024, 8
+    pxp, pyp = cc.to_device(gen.normal_f16(405, (tp, hidden))), cc.alloc(tp * hidden * 2)
+    prefill_chain = {"layers": lp, "M": tp}
+    for fused in (False, True):
+        smp = [dec.bench_chain("c4", lp, pxp, tp, pyp, 3, warmup=1, use_graph=False, fused=fused)[0] / 3 for _ in range(ROUNDS)]
+        vv = gen.f16_bits_to_f32(cc.d2h(pyp, (tp, hidden), np.uint16)).astype(np.float64)
+        ok = bool(np.all(np.isfinite(vv)) and np.allclose(np.mean(vv * vv, axis=1), 1.0, atol=2e-3))
+        prefill_chain["normalisations_deferred" if fused else "normalisation_launches_kept"] = {
+            "ms_per_layer": round(sorted(smp)[ROUNDS // 2] / lp, 4), "ms_per_pass": spread(smp, 1.0, 4),
+            "output_finite_unit_mean_square": ok}
+    flops_layer = 2.0 * tp * sum(nn * kk for (nn, kk) in shapes.values())
+    best_layer = min(v["ms_per_layer"] for v in prefill_chain.values() if isinstance(v, dict) and v["output_finite_unit_mean_square"])
+    prefill_chain["TFLOPs_end_to_end"] = round(flops_layer / (best_layer * 1e-3) / 1e12, 1)
+    cc.free(pxp)
+    cc.free(pyp)
     return {"layers": layers, "M": t, "launches_per_layer": fig["launches_per_layer"], "ms_per_pass": best,
+            "prefill_regime": prefill_chain,
             "us_per_token": round(best * 1e3 / t, 2), "GBps_end_to_end": round(total / (best * 1e-3) / 1e9, 1),
             "hbm_frac_end_to_end": round(total / (best * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
             "normalisation_launches_kept": kept, "normalisations_deferred": deferred, "per_gemm": per_gemm}

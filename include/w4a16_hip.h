@@ -184,8 +184,8 @@ int w4a16_plan_decode(size_t n, size_t k, size_t group, size_t t, int cu_count, 
  * w4a16_set_prefill_tile / w4a16_set_prefill_ksplit do (0 = automatic); *price_us (may be NULL) receives the model's
  * estimate for the chosen plan.  Role of the reference's per-problem choice of thread-block shape
  * (kernels/marlin.rs:94-213).  Needs neither a context nor a GPU. */
-int w4a16_plan_prefill(size_t t, size_t n, size_t k, int cu_count, int tile_rows, int k_slices, size_t out[5],
-                       double* price_us);
+int w4a16_plan_prefill(size_t t, size_t n, size_t k, size_t group, int cu_count, int tile_rows, int k_slices,
+                       size_t out[5], double* price_us);
 
 /* w4a16_lin_forward for callers that cannot allocate.  NO COUNTERPART IN THE REFERENCE: it exists for code under HIP graph
  * capture, tight serving loops and harnesses that forbid hipMalloc.  w4a16_lin_forward's decode launch, when it splits k
@@ -244,6 +244,11 @@ int w4a16_lin_forward_glu_act(w4a16_ctx* ctx, const char* name, uint64_t x_dev, 
  * 6e-5 lose relative precision to f16 subnormals.  Nothing is detected at run time.  Residual streams of trained
  * models sit well inside; the synthetic 64-layer chain of random projections does not: the _scaled forms below lift the
  * precondition. */
+/* Row count: any t.  Up to 16 rows the decode kernel serves the call and a statistics array is [entries][16] floats
+ * (row m of entry e at e*16 + m); beyond 16 rows the MFMA-tiled kernel does (the linear must then hold only scales that
+ * kernel can divide by, W4A16_ERR_UNSUPPORTED otherwise) and a statistics array is [entries][ld] floats with ld = t
+ * rounded up to a multiple of 4.  *n_stats_out entries are written (at most n/16 resp. n/64: size stats_out_dev for
+ * that); producer and consumer of one array run at the same t. */
 int w4a16_lin_forward_deferred_norm(w4a16_ctx* ctx, const char* name, uint64_t x_dev, size_t ldx, size_t t,
                                     uint64_t stats_in_dev, size_t n_stats_in, size_t in_cols, uint64_t y_dev,
                                     int out_f16, uint64_t stats_out_dev, size_t stat_rows, size_t* n_stats_out,
@@ -435,7 +440,8 @@ int w4a16_act_mul_f16(w4a16_ctx* ctx, uint64_t gu_f32_dev, size_t n_ff, size_t t
 int w4a16_chain_forward(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers, uint64_t x_dev, size_t t,
                         uint64_t y_dev);
 /* The same chain with the normalisations inside it deferred across the linears (w4a16_lin_forward_deferred_norm), four
- * launches per layer instead of seven, t <= 16.  With r(v) = 1/sqrt(mean(v^2) + 1e-6) per row, s0 = 1 and x0 = x:
+ * launches per layer instead of seven (any t; beyond 16 rows on the MFMA-tiled kernels, plus a finish launch where a
+ * linear is split over k).  With r(v) = 1/sqrt(mean(v^2) + 1e-6) per row, s0 = 1 and x0 = x:
  *     v1 = s[l] * qkv(x[l])[:, :hidden]      a = f16(v1)
  *     v2 = r(v1) * attn_output(a)            b = f16(v2)
  *     gu = r(v2) * ffn_gate_up(b)            c = silu_mul_f16(gu)

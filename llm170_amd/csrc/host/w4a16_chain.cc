@@ -153,8 +153,7 @@ static int handover_exp(double bound) {
 extern "C" int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, size_t layer0, size_t n_layers,
                                          uint64_t x_dev, size_t t, uint64_t y_dev) {
     if (!ctx || !prefix || !x_dev || !y_dev) return w4_fail(W4A16_ERR_ARG, "chain_forward_fused: null argument");
-    if (n_layers == 0 || t == 0 || t > 16)
-        return w4_fail(W4A16_ERR_SHAPE, "chain_forward_fused: n_layers=%zu t=%zu (decode regime: 1..16 rows)", n_layers, t);
+    if (n_layers == 0 || t == 0) return w4_fail(W4A16_ERR_SHAPE, "chain_forward_fused: n_layers=%zu t=%zu", n_layers, t);
     W4ChainScratch& S = ctx->chain;
     uint64_t cur = x_dev;
     size_t n_prev = 0;  // partial sums the previous layer's down projection left in S.stats[2]
@@ -178,7 +177,11 @@ extern "C" int w4a16_chain_forward_fused(w4a16_ctx* ctx, const char* prefix, siz
         W4_TRY(w4_ensure(ctx, &S.h16b, &S.h16b_cap, t * n_ff * 2));
         W4_TRY(w4_ensure(ctx, &S.ping[0], &S.ping_cap[0], t * hidden * 2));
         for (int i = 0; i < 3; i++)
-            W4_TRY(w4_ensure(ctx, &S.stats[i], &S.stats_cap[i], ((std::max(n_qkv, hidden) + 15) / 16) * 64));
+            // decode regime: one entry of 16 floats per 16 output rows at most; beyond it one entry of t (rounded up to
+            // 4) floats per 64 output columns at most
+            W4_TRY(w4_ensure(ctx, &S.stats[i], &S.stats_cap[i],
+                             t <= 16 ? ((std::max(n_qkv, hidden) + 15) / 16) * 64
+                                     : ((std::max(n_qkv, hidden) + 63) / 64) * ((t + 3) / 4 * 4) * 4));
         const bool last = l + 1 == layer0 + n_layers;
         size_t n_a = 0, n_b = 0, n_d = 0;
         float rn[4];

@@ -66,7 +66,7 @@ static const char* const kDecodeSyms[] = {
     nullptr};
 static const char* const kPrefillSyms[] = {"w4a16_prefill_g128_f16", "w4a16_prefill_g128_bf16", "w4a16_prefill_g32_f16",
                                            "w4a16_prefill_g32_bf16", "w4a16_prefill_g128_f16_m64", "w4a16_prefill_g128_bf16_m64", "w4a16_prefill_g32_f16_m64",
-                                           "w4a16_prefill_g32_bf16_m64", "w4a16_prefill_splitk_sum",
+                                           "w4a16_prefill_g32_bf16_m64", "w4a16_prefill_splitk_sum", "w4a16_prefill_splitk_finish",
                                            "w4a16_prefill_g128_f16_glu", "w4a16_prefill_g128_bf16_glu", "w4a16_prefill_g32_f16_glu",
                                            "w4a16_prefill_g32_bf16_glu", "w4a16_prefill_g128_f16_m64_glu", "w4a16_prefill_g128_bf16_m64_glu",
                                            "w4a16_prefill_g32_f16_m64_glu", "w4a16_prefill_g32_bf16_m64_glu",

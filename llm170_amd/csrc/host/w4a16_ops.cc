@@ -324,7 +324,8 @@ struct PrefillPlan {
     double us;  // the price it won with
 };
 
-static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t cus, int tile_m_forced, int ksplit_forced, bool glu = false) {
+static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t group, size_t cus, int tile_m_forced, int ksplit_forced,
+                                bool glu = false) {
     // a gated launch tiles the n/2 output columns by 128 (each block tile holds the matching 128 up columns as well)
     const size_t tiles_n = glu ? (n / 2 + kW4PfBn / 2 - 1) / (kW4PfBn / 2) : (n + kW4PfBn - 1) / kW4PfBn, kt_n = k / 128;
     // Super-tile shape for a grid of tiles_m x tiles_n block tiles: sup_m <= 8 along m, sup_n in {8, 4, 2, 1} along n.
@@ -379,6 +380,7 @@ static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t cus, int ti
     PrefillPlan best{128, 1, PrefillSuper{1, 1, 0, 0}, 1e30};
     for (size_t rows : {(size_t)128, (size_t)96, (size_t)64}) {
         if (tile_m_forced && (size_t)tile_m_forced != rows) continue;
+        if (rows == 96 && group != 128 && !tile_m_forced) continue;  // the group-32 builds of that tile spill: only when pinned
         const size_t tiles_m = (t + rows - 1) / rows;
         const PrefillSuper sup = super_for(tiles_m);
         const size_t forced = ksplit_forced > 0 ? std::max<size_t>(1, std::min<size_t>((size_t)ksplit_forced, kt_n / 4)) : 0;
@@ -397,12 +399,12 @@ static PrefillPlan plan_prefill(size_t t, size_t n, size_t k, size_t cus, int ti
     return best;
 }
 
-extern "C" int w4a16_plan_prefill(size_t t, size_t n, size_t k, int cu_count, int tile_rows, int k_slices, size_t out[5],
-                                  double* price_us) {
-    if (t == 0 || n == 0 || k == 0 || k % 128 != 0 || cu_count <= 0 || !out ||
+extern "C" int w4a16_plan_prefill(size_t t, size_t n, size_t k, size_t group, int cu_count, int tile_rows, int k_slices,
+                                  size_t out[5], double* price_us) {
+    if (t == 0 || n == 0 || k == 0 || k % 128 != 0 || (group != 128 && group != 32) || cu_count <= 0 || !out ||
         (tile_rows != 0 && tile_rows != 64 && tile_rows != 96 && tile_rows != 128) || k_slices < -1 || k_slices > 16)
         return w4_fail(W4A16_ERR_ARG, "plan_prefill: t=%zu n=%zu k=%zu cus=%d tile=%d slices=%d", t, n, k, cu_count, tile_rows, k_slices);
-    const PrefillPlan P = plan_prefill(t, n, k, (size_t)cu_count, tile_rows, k_slices);
+    const PrefillPlan P = plan_prefill(t, n, k, group, (size_t)cu_count, tile_rows, k_slices);
     out[0] = P.bm;
     out[1] = P.nks;
     out[2] = P.sup.sup_m;
@@ -412,25 +414,66 @@ extern "C" int w4a16_plan_prefill(size_t t, size_t n, size_t k, int cu_count, in
     return 0;
 }
 
+// Host mirror of PfEpi (kernels/prefill.hip): same members in the same order.
+struct PfEpiHost {
+    uint64_t stats_in = 0, stats_out = 0, resid = 0, nw = 0;
+    int n_stats_in = 0, ld_stats = 0, stat_cols = 0, ldx = 0;
+    float inv_cols_in = 0.f, in_scale = 1.f, out_scale = 1.f;
+};
+static_assert(sizeof(PfEpiHost) == 64, "PfEpi is four pointers, four ints and three floats, padded to 64 bytes");
+
+// Floats between the rows' entries of a statistics array: 16 in the decode regime (kernels/decode.hip), the row count
+// rounded up to 4 beyond it.
+static size_t stats_ld(size_t t) { return t <= 16 ? 16 : (t + 3) / 4 * 4; }
+
 // Prefill GEMM (kernels/prefill.hip).  glu_act >= 0: the linear is a fused gate|up projection and y receives
-// f16 [t][n/2] = act(gate) * up (W4A16_ACT_*), the element-wise kernel folded into the epilogue.
-static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16, int glu_act = -1) {
+// f16 [t][n/2] = act(gate) * up (W4A16_ACT_*), the element-wise kernel folded into the epilogue.  norm != null: the
+// parts of a normalisation deferred across this linear (row factor from the producer's statistics, residual, norm
+// weight, statistics of the output, power-of-two hand-over factors), as in the decode kernel.
+static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16, int glu_act = -1,
+                          DecodeNorm* norm = nullptr) {
     const bool glu = glu_act >= 0;
     if (glu && L.n % 32 != 0) return w4_fail(W4A16_ERR_SHAPE, "prefill glu: n=%zu must be a multiple of 32 (gate and up halves of whole row blocks)", L.n);
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has no tiled copy (needs k %% 128 == 0)");
     if (!L.scales_regular)
         return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: linear has a zero or non-finite scale (use the decode path)");
-    if (t * L.k * 2 >= 0x80000000ull || L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
+    PfEpiHost epi;
+    size_t ldx = L.k;
+    bool has_epi = false;
+    if (norm) {
+        W4_TRY(check_decode_norm(L, t, *norm));
+        if (glu && (norm->stats_out || norm->resid || norm->nw))
+            return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill glu: the gated output takes no statistics, residual or norm weight");
+        ldx = norm->ldx ? norm->ldx : L.k;
+        epi.stats_in = norm->stats_in;
+        epi.n_stats_in = (int)norm->n_stats_in;
+        epi.inv_cols_in = norm->in_cols ? 1.0f / (float)norm->in_cols : 0.0f;
+        epi.ld_stats = (int)stats_ld(t);
+        epi.stats_out = norm->stats_out;
+        epi.stat_cols = norm->stats_out ? (int)std::min<size_t>(norm->stat_rows, L.n) : 0;
+        epi.resid = norm->resid;
+        epi.nw = norm->nw;
+        epi.ldx = (int)ldx;
+        epi.in_scale = std::ldexp(1.0f, norm->in_exp);
+        epi.out_scale = std::ldexp(1.0f, -norm->out_exp);
+        has_epi = epi.stats_in || epi.stats_out || epi.resid || epi.nw || norm->in_exp != 0 || norm->out_exp != 0;
+        norm->n_stats_out = 0;
+    }
+    if (((t - 1) * ldx + L.k) * 2 >= 0x80000000ull || L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
         return w4_fail(W4A16_ERR_SHAPE, "prefill: x or the tiled weights reach 2 GiB, beyond the buffer-descriptor range");
+    // A split launch finishes in a second kernel.  With epilogue options that kernel works on whole 1024-column
+    // chunks of a row; where the shape does not allow it (or for the gated form) the k range stays whole.
+    int ksplit = ctx->prefill_ksplit;
+    if (has_epi && (glu || L.n % 1024 != 0)) ksplit = -1;
     // the plan depends on (t, n, k) and the pinned settings only and is kept per shape
     PrefillPlan plan;
     {
-        const auto key = std::make_tuple(t, L.n, L.k, ctx->prefill_tile_m + (glu ? 1000 : 0), ctx->prefill_ksplit);
+        const auto key = std::make_tuple(t, L.n, L.k, ctx->prefill_tile_m + (glu ? 1000 : 0), ksplit);
         const auto hit = ctx->prefill_plans.find(key);
         if (hit != ctx->prefill_plans.end()) {
             plan = PrefillPlan{hit->second[0], hit->second[1], PrefillSuper{hit->second[2], hit->second[3], hit->second[4], 0}, 0.0};
         } else {
-            plan = plan_prefill(t, L.n, L.k, (size_t)std::max(ctx->cu_count, 1), ctx->prefill_tile_m, ctx->prefill_ksplit, glu);
+            plan = plan_prefill(t, L.n, L.k, L.group, (size_t)std::max(ctx->cu_count, 1), ctx->prefill_tile_m, ksplit, glu);
             ctx->prefill_plans[key] = {plan.bm, plan.nks, plan.sup.sup_m, plan.sup.sup_n, plan.sup.supers};
         }
     }
@@ -438,12 +481,14 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     const size_t grid = ((supers + 7) / 8) * (sup_m * sup_n) * 8;
     char sym[64];
     snprintf(sym, sizeof sym, "w4a16_prefill_g%zu_%s%s%s", L.group, L.scale_bf16 ? "bf16" : "f16", bm == 64 ? "_m64" : bm == 96 ? "_m96" : "", glu ? "_glu" : "");
-    const unsigned shmem = (unsigned)(2 * bm * kW4PfKs * 2);  // two stages of bm rows x PF_KS halves
+    // two stages of bm rows x PF_KS halves, then bm words (row factors of the dense kernels)
+    const unsigned shmem = (unsigned)(2 * bm * kW4PfKs * 2 + bm * 4);
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = (out_f16 || glu) ? 1 : 0;
     int spm = (int)sup_m, spn = (int)sup_n, act = glu ? glu_act : 0, glu_i = glu ? 1 : 0;
     if (nks == 1) {
-        void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &spm, &spn, &act};  // act: gated kernels only
+        if (norm && epi.stats_out) norm->n_stats_out = ((size_t)epi.stat_cols + 63) / 64;  // one entry per wave's 64 columns
+        void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &spm, &spn, &act, &epi};
         return w4_launch(ctx, sym, (unsigned)grid, 1, kW4PfThreads, shmem, params);
     }
     if (L.n % (glu ? 8 : 4) != 0) return w4_fail(W4A16_ERR_UNSUPPORTED, "prefill: split-K needs n %% %d == 0", glu ? 8 : 4);
@@ -451,9 +496,17 @@ static int launch_prefill(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y
     W4_TRY(w4_ensure(ctx, &ctx->prefill_ws, &ctx->prefill_ws_cap, count * 4 * nks));
     uint64_t ws = ctx->prefill_ws;
     int zero = 0;
-    void* params[] = {&qt, &st, &x, &ws, &row_blocks, &ki, &ni, &ti, &zero, &spm, &spn, &act};
+    PfEpiHost slice_epi;  // the slices only need the row stride of x; the finish kernel applies the options
+    slice_epi.ldx = (int)ldx;
+    void* params[] = {&qt, &st, &x, &ws, &row_blocks, &ki, &ni, &ti, &zero, &spm, &spn, &act, &slice_epi};
     W4_TRY(w4_launch(ctx, sym, (unsigned)grid, (unsigned)nks, kW4PfThreads, shmem, params));
     int nksi = (int)nks;
+    if (has_epi) {
+        if (t * (L.n / 1024) > 0x7fffffffu) return w4_fail(W4A16_ERR_SHAPE, "prefill: t=%zu n=%zu exceed the finish launch", t, L.n);
+        if (norm && epi.stats_out) norm->n_stats_out = ((size_t)epi.stat_cols + 1023) / 1024;  // one entry per 1024-column chunk
+        void* fp[] = {&ws, &y, &nksi, &ti, &ni, &of, &epi};
+        return w4_launch(ctx, "w4a16_prefill_splitk_finish", (unsigned)(t * (L.n / 1024)), 1, 256, 0, fp);
+    }
     size_t cnt = count;
     void* rp[] = {&ws, &y, &nksi, &cnt, &of, &glu_i, &ni, &act};
     return w4_launch(ctx, "w4a16_prefill_splitk_sum", std::min<unsigned>(ceil_div(count / (glu ? 8 : 4), 256), 4096), 1, 256, 0, rp);
@@ -795,7 +848,15 @@ extern "C" int w4a16_lin_forward_deferred_norm_scaled(w4a16_ctx* ctx, const char
     nm.nw = nw_dev;
     nm.in_exp = in_exp;
     nm.out_exp = out_exp;
-    W4_TRY(launch_decode(ctx, *L, x_dev, y_dev, t, out_f16, &nm));
+    if (t <= 16) {
+        W4_TRY(launch_decode(ctx, *L, x_dev, y_dev, t, out_f16, &nm));
+    } else {
+        // beyond the decode regime the MFMA-tiled kernel carries the same options in its epilogue (statistics arrays
+        // are then [entries][t rounded up to 4] floats); it needs scales it can divide by
+        if (!L->scales_regular)
+            return w4_fail(W4A16_ERR_UNSUPPORTED, "lin_forward_deferred_norm %s: t=%zu runs the MFMA-tiled kernel, which cannot take this linear's zero, non-finite or out-of-range scale", name, t);
+        W4_TRY(launch_prefill(ctx, *L, x_dev, y_dev, t, out_f16, -1, &nm));
+    }
     if (n_stats_out) *n_stats_out = nm.n_stats_out;
     return 0;
 }
@@ -823,7 +884,12 @@ extern "C" int w4a16_lin_forward_glu_deferred_norm_scaled(w4a16_ctx* ctx, const 
     nm.act = act;
     nm.in_exp = in_exp;
     nm.out_exp = out_exp;
-    return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t, &nm);
+    if (t <= 16) return launch_decode_glu(ctx, *L, x_dev, y_f16_dev, t, &nm);
+    if (act != W4A16_ACT_SILU && act != W4A16_ACT_GELU_TANH)
+        return w4_fail(W4A16_ERR_ARG, "lin_forward_glu_deferred_norm %s: activation %d (0 = silu, 1 = gelu, tanh form)", name, act);
+    if (!L->scales_regular)
+        return w4_fail(W4A16_ERR_UNSUPPORTED, "lin_forward_glu_deferred_norm %s: t=%zu runs the MFMA-tiled kernel, which cannot take this linear's zero, non-finite or out-of-range scale", name, t);
+    return launch_prefill(ctx, *L, x_dev, y_f16_dev, t, 1, act, &nm);
 }
 
 extern "C" int w4a16_lin_forward_host(w4a16_ctx* ctx, const char* name, const uint16_t* x_f16, void* y, size_t t,

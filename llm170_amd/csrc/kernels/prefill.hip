@@ -68,12 +68,30 @@ struct PfGroup {
     int ns, x_rows, x_div, n_exp, act_kind;
 };
 
+// Epilogue options of the dense kernels (MODE 0 and 3), the prefill-regime form of what the decode kernel does for a
+// normalisation deferred across linears (the element-wise parts of the reference's norm_resid, assets/norm.cu:4-48,
+// moved into the linears either side of it).  Every part is optional (a null pointer / 0 / 1.0 switches it off):
+//   consumer side: stats_in [n_stats_in][ld_stats] are partial sums of squares of the INPUT rows left by the launch
+//     that produced x; the output row m is multiplied by 1/sqrt(sum_e stats_in[e][m] * inv_cols_in + 1e-6) * in_scale
+//     (in_scale = 2^e undoes the power-of-two factor x was handed over with); ldx = halves between x rows (0 = k);
+//   producer side: resid f32 [t][n] takes the output (v = resid + y, written back); stats_out[(tile_n*4 + wave)][m]
+//     receives this wave's partial sum of v^2 over its columns below stat_cols (one entry per wave and block tile
+//     column, no atomics); nw f32 [n] multiplies what y receives; out_scale = 2^-e is applied last.
+struct PfEpi {
+    const float* stats_in;
+    float* stats_out;
+    float* resid;
+    const float* nw;
+    int n_stats_in, ld_stats, stat_cols, ldx;
+    float inv_cols_in, in_scale, out_scale;
+};
+
 template <int G, bool SBF, int MI, int MODE = 0>
 __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                              const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
                                              int k, int n, int t, int out_f16, int sup_m, int sup_n,
-                                             const PfGroup<MODE> gp = PfGroup<MODE>()) {
-    extern __shared__ _Float16 lds[];  // 2 stages x [PF_BM][PF_LDA]; grouped: then the segment's PF_BM slot ids
+                                             const PfGroup<MODE> gp = PfGroup<MODE>(), const PfEpi epi = PfEpi()) {
+    extern __shared__ _Float16 lds[];  // 2 stages x [PF_BM][PF_LDA]; then PF_BM ints: slot ids (grouped) / row factors (dense)
     constexpr int GPT = W4_TILE_K / G;
     constexpr int PF_BM = 32 * MI, PF_STAGE_BYTES = PF_BM * PF_LDA * 2;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -112,7 +130,8 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
         n0 = blockIdx.x * (MODE == 1 ? PF_BN / 2 : PF_BN);
     }
 
-    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, (unsigned)(DENSE ? t : gp.x_rows) * (unsigned)k * 2u);
+    const unsigned ldx = DENSE && epi.ldx ? (unsigned)epi.ldx : (unsigned)k;  // halves between x rows
+    const __amdgpu_buffer_rsrc_t xr = w4_make_rsrc(x, DENSE ? ((unsigned)(t - 1) * ldx + (unsigned)k) * 2u : (unsigned)gp.x_rows * (unsigned)k * 2u);
     const __amdgpu_buffer_rsrc_t qr = w4_make_rsrc(qt, (unsigned)row_blocks * (unsigned)kt_n * 1024u);
     const __amdgpu_buffer_rsrc_t sr = w4_make_rsrc(st, (unsigned)row_blocks * (unsigned)kg_n * 32u);
 
@@ -128,7 +147,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     for (int i = 0; i < MI; i++) {
         const int c = tid + i * PF_THREADS, row = c >> 3, kc = (c & 7) ^ (row & 7);
         if (DENSE) {
-            xa_off[i] = (m0 + row < t) ? ((unsigned)(m0 + row) * (unsigned)k + (unsigned)kc * 8u) * 2u : W4_OOB;
+            xa_off[i] = (m0 + row < t) ? ((unsigned)(m0 + row) * ldx + (unsigned)kc * 8u) * 2u : W4_OOB;
         } else {
             const int id = gp.sorted_ids[m0 + row];  // padding rows carry the sentinel ns: zeros, never stored
             xa_off[i] = id < gp.ns ? ((unsigned)(id / gp.x_div) * (unsigned)k + (unsigned)kc * 8u) * 2u : W4_OOB;
@@ -136,6 +155,27 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     }
     int* const seg_ids = reinterpret_cast<int*>(lds_base + 2 * PF_STAGE_BYTES);
     if (!DENSE && tid < PF_BM) seg_ids[tid] = gp.sorted_ids[m0 + tid];  // visible after the first barrier
+    // Dense, input statistics given: the 1/rms factor of this block's PF_BM input rows, once, into the same LDS words
+    // (thread r < PF_BM owns row m0 + r: entries added in index order with eight loads in flight — the same bits on
+    // every run; consecutive threads read consecutive floats of an entry).  Read back in the epilogue.
+    float* const row_fac = reinterpret_cast<float*>(lds_base + 2 * PF_STAGE_BYTES);
+    if (DENSE && epi.stats_in != nullptr && tid < PF_BM) {
+        const int row = m0 + tid;
+        float sum = 0.f;
+        if (row < t) {
+            const float* sp = epi.stats_in + row;
+            int e = 0;
+            for (; e + 8 <= epi.n_stats_in; e += 8) {
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = sp[(size_t)(e + j) * epi.ld_stats];
+#pragma unroll
+                for (int j = 0; j < 8; j++) sum += v[j];
+            }
+            for (; e < epi.n_stats_in; e++) sum += sp[(size_t)e * epi.ld_stats];
+        }
+        row_fac[tid] = (float)(1.0 / sqrt((double)sum * (double)epi.inv_cols_in + 1e-6)) * epi.in_scale;
+    }
     auto load_a = [&](int s, int buf) {
 #pragma unroll
         for (int i = 0; i < MI; i++)
@@ -302,6 +342,8 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
         }
         return;
     }
+    // x arrived as its true value times 1/in_scale and (with input statistics) un-normalised: one factor per row
+    const bool use_fac = DENSE && (epi.stats_in != nullptr || (epi.in_scale != 1.0f && epi.in_scale != 0.0f));
     if (MODE == 3 && gridDim.y == 1) {
         const int n_ff = n >> 1, col = n0 + wn * 32 + nl;
         if (col >= n_ff) return;
@@ -313,31 +355,82 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
                 if (row < t) {
                     float gt = acc[mi][0][e] * unit[0], up = acc[mi][1][e] * unit[1];
                     asm volatile("" : "+v"(gt), "+v"(up));  // the sums are rounded to f32 as the separate launch stores them
+                    if (use_fac) {
+                        const float f = epi.stats_in != nullptr ? row_fac[row - m0] : epi.in_scale;
+                        gt *= f;
+                        up *= f;
+                    }
                     float v = w4_act_mul(gt, up, gp.act_kind);
                     asm volatile("" : "+v"(v));  // and the product before the f16 conversion, as in the separate kernel
+                    if (epi.out_scale != 1.0f && epi.out_scale != 0.0f) {
+                        v *= epi.out_scale;
+                        asm volatile("" : "+v"(v));
+                    }
                     reinterpret_cast<_Float16*>(y)[(size_t)row * n_ff + col] = (_Float16)v;
                 }
             }
         }
         return;
     }
-    if (gridDim.y > 1) y = reinterpret_cast<float*>(y) + (size_t)blockIdx.y * (size_t)t * (size_t)n;  // partial (f32)
+    if (gridDim.y > 1) {  // partial (f32) of a split launch: w4a16_prefill_splitk_sum finishes (activation, epilogue options)
+        y = reinterpret_cast<float*>(y) + (size_t)blockIdx.y * (size_t)t * (size_t)n;
 #pragma unroll
-    for (int ni = 0; ni < 2; ni++) {
-        const int col = MODE == 3 ? ni * (n >> 1) + n0 + wn * 32 + nl : n0 + wn * 64 + ni * 32 + nl;
-        if (MODE == 3 ? n0 + wn * 32 + nl >= (n >> 1) : col >= n) continue;
+        for (int ni = 0; ni < 2; ni++) {
+            const int col = MODE == 3 ? ni * (n >> 1) + n0 + wn * 32 + nl : n0 + wn * 64 + ni * 32 + nl;
+            if (MODE == 3 ? n0 + wn * 32 + nl >= (n >> 1) : col >= n) continue;
 #pragma unroll
-        for (int mi = 0; mi < MI; mi++) {
+            for (int mi = 0; mi < MI; mi++) {
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int row = m0 + mi * 32 + 8 * (e >> 2) + 4 * khalf + (e & 3);
-                if (row < t) {
-                    const float v = acc[mi][ni][e] * unit[ni];
+                for (int e = 0; e < 16; e++) {
+                    const int row = m0 + mi * 32 + 8 * (e >> 2) + 4 * khalf + (e & 3);
+                    if (row < t) reinterpret_cast<float*>(y)[(size_t)row * n + col] = acc[mi][ni][e] * unit[ni];
+                }
+            }
+        }
+        return;
+    }
+    // MODE 0, whole k range: y = acc * unit, then the optional parts in the order of the decode kernel's epilogue — row
+    // factor, residual stream, statistics of what continues, norm weight, power-of-two hand-over factor
+    const bool plain = !use_fac && epi.resid == nullptr && epi.stats_out == nullptr && epi.nw == nullptr && (epi.out_scale == 1.0f || epi.out_scale == 0.0f);
+#pragma unroll
+    for (int mi = 0; mi < MI; mi++) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const int row = m0 + mi * 32 + 8 * (e >> 2) + 4 * khalf + (e & 3);
+            float p = 0.f;  // this lane's share of the row's sum of squares
+            if (row < t) {
+                const float f = !use_fac ? 1.0f : epi.stats_in != nullptr ? row_fac[row - m0] : epi.in_scale;
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) {
+                    const int col = n0 + wn * 64 + ni * 32 + nl;
+                    if (col >= n) continue;
+                    float v = acc[mi][ni][e] * unit[ni];
+                    if (!plain) {
+                        asm volatile("" : "+v"(v));
+                        if (use_fac) v *= f;
+                        if (epi.resid != nullptr) {
+                            float* const rp = epi.resid + (size_t)row * n + col;
+                            v += *rp;
+                            *rp = v;
+                        }
+                        if (col < epi.stat_cols) p = __builtin_fmaf(v, v, p);
+                        if (epi.nw != nullptr) v *= epi.nw[col];
+                        if (epi.out_scale != 1.0f && epi.out_scale != 0.0f) {
+                            v *= epi.out_scale;
+                            asm volatile("" : "+v"(v));  // rounded to f32 on its own, not fused into the f16 conversion
+                        }
+                    }
                     if (out_f16)
                         reinterpret_cast<_Float16*>(y)[(size_t)row * n + col] = (_Float16)v;
                     else
                         reinterpret_cast<float*>(y)[(size_t)row * n + col] = v;
                 }
+            }
+            if (epi.stats_out != nullptr) {  // uniform: the 32 lanes of a row (same khalf) add up in a fixed order
+#pragma unroll
+                for (int off = 16; off > 0; off >>= 1) p += __shfl_xor(p, off);
+                if (nl == 0 && row < t && n0 + wn * 64 < epi.stat_cols)
+                    epi.stats_out[(size_t)((n0 + wn * 64) >> 6) * epi.ld_stats + row] = p;
             }
         }
     }
@@ -346,19 +439,20 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
 #define PREFILL_KERNEL(NAME, G, SBF, MI, WPE)                                                                      \
     extern "C" __global__ __launch_bounds__(PF_THREADS) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(      \
         const u4_t* qt, const uint16_t* st, const uint16_t* x, void* y, int row_blocks, int k, int n, int t,          \
-        int out_f16, int sup_m, int sup_n) {                                                                           \
-        prefill_body<G, SBF, MI>(qt, st, x, y, row_blocks, k, n, t, out_f16, sup_m, sup_n);                            \
+        int out_f16, int sup_m, int sup_n, int act_kind, PfEpi epi) {                                                  \
+        (void)act_kind;                                                                                                \
+        prefill_body<G, SBF, MI>(qt, st, x, y, row_blocks, k, n, t, out_f16, sup_m, sup_n, PfGroup<0>(), epi);         \
     }
 
-// Dense gated kernels: the arguments of PREFILL_KERNEL plus the activation (W4A16_ACT_*); y is f16 [t][n/2], or the f32
+// Dense gated kernels: same arguments (the plain kernels ignore act_kind, W4A16_ACT_*); y is f16 [t][n/2], or the f32
 // partials [slices][t][n] of a split launch.
 #define PREFILL_GLU_KERNEL(NAME, G, SBF, MI, WPE)                                                                  \
     extern "C" __global__ __launch_bounds__(PF_THREADS) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(      \
         const u4_t* qt, const uint16_t* st, const uint16_t* x, void* y, int row_blocks, int k, int n, int t,          \
-        int out_f16, int sup_m, int sup_n, int act_kind) {                                                             \
+        int out_f16, int sup_m, int sup_n, int act_kind, PfEpi epi) {                                                  \
         PfGroup<3> gp;                                                                                                 \
         gp.act_kind = act_kind;                                                                                        \
-        prefill_body<G, SBF, MI, 3>(qt, st, x, y, row_blocks, k, n, t, out_f16, sup_m, sup_n, gp);                     \
+        prefill_body<G, SBF, MI, 3>(qt, st, x, y, row_blocks, k, n, t, out_f16, sup_m, sup_n, gp, epi);                \
     }
 
 // Grouped kernels for the expert FFN: same arguments as the streaming grouped kernels of moe.hip (blk must be 64, the
@@ -423,6 +517,62 @@ extern "C" __global__ __launch_bounds__(256) void w4a16_prefill_splitk_sum(const
         } else {
             reinterpret_cast<f4_t*>(y)[i] = a;
         }
+    }
+}
+
+// Finish of a split launch that carries epilogue options (MODE 0 only; n % 1024 == 0): one workgroup per (row,
+// 1024-column chunk) adds the slices in order and applies the options of PfEpi in the order of the unsplit epilogue.
+// Statistics: one entry per chunk, stats_out[chunk][row] (the four waves' sums folded in wave order).
+extern "C" __global__ __launch_bounds__(256) void w4a16_prefill_splitk_finish(const float* __restrict__ part, void* __restrict__ y,
+                                                                              int nks, int t, int n, int out_f16, PfEpi epi) {
+    __shared__ float red[4];
+    __shared__ float fac_s;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int chunks = n >> 10, row = blockIdx.x / chunks, chunk = blockIdx.x - row * chunks;
+    if (row >= t) return;
+    const bool use_fac = epi.stats_in != nullptr || (epi.in_scale != 1.0f && epi.in_scale != 0.0f);
+    if (epi.stats_in != nullptr && wave == 0) {
+        float sum = 0.f;
+        for (int e = lane; e < epi.n_stats_in; e += 64) sum += epi.stats_in[(size_t)e * epi.ld_stats + row];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+        if (lane == 0) fac_s = (float)(1.0 / sqrt((double)sum * (double)epi.inv_cols_in + 1e-6)) * epi.in_scale;
+    }
+    if (epi.stats_in != nullptr) __syncthreads();
+    const float f = !use_fac ? 1.0f : epi.stats_in != nullptr ? fac_s : epi.in_scale;
+    const int col = (chunk << 10) + tid * 4;
+    const size_t count = (size_t)t * (size_t)n, at = (size_t)row * n + col;
+    f4_t a = *reinterpret_cast<const f4_t*>(part + at);
+    for (int ks = 1; ks < nks; ks++) a += *reinterpret_cast<const f4_t*>(part + (size_t)ks * count + at);
+    float p = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float v = a[j];
+        if (use_fac) v *= f;
+        if (epi.resid != nullptr) {
+            v += epi.resid[at + j];
+            epi.resid[at + j] = v;
+        }
+        if (col + j < epi.stat_cols) p = __builtin_fmaf(v, v, p);
+        if (epi.nw != nullptr) v *= epi.nw[col + j];
+        if (epi.out_scale != 1.0f && epi.out_scale != 0.0f) {
+            v *= epi.out_scale;
+            asm volatile("" : "+v"(v));
+        }
+        a[j] = v;
+    }
+    if (out_f16) {
+        h4_t o = {(_Float16)a[0], (_Float16)a[1], (_Float16)a[2], (_Float16)a[3]};
+        *reinterpret_cast<h4_t*>(reinterpret_cast<_Float16*>(y) + at) = o;
+    } else {
+        *reinterpret_cast<f4_t*>(reinterpret_cast<float*>(y) + at) = a;
+    }
+    if (epi.stats_out != nullptr) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) p += __shfl_xor(p, off);
+        if (lane == 0) red[wave] = p;
+        __syncthreads();
+        if (tid == 0 && (chunk << 10) < epi.stat_cols) epi.stats_out[(size_t)chunk * epi.ld_stats + row] = ((red[0] + red[1]) + red[2]) + red[3];
     }
 }
 

@@ -59,7 +59,7 @@ _SIGS = {
     "w4a16_noalloc_workspace_bytes": (C.c_size_t, []),
     "w4a16_plan_decode": (C.c_int, [C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.POINTER(C.c_int),
                                     C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_size_t)]),
-    "w4a16_plan_prefill": (C.c_int, [C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_int,
+    "w4a16_plan_prefill": (C.c_int, [C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_int,
                                      C.POINTER(C.c_size_t), C.POINTER(C.c_double)]),
     "w4a16_lin_forward_glu": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_size_t]),
     "w4a16_lin_forward_glu_act": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64, C.c_size_t, C.c_int]),

@@ -27,12 +27,12 @@ def plan_decode(n, k, group, t, cu_count=256, glu=False):
     return {"rows_per_wave": rows.value, "waves_per_block": waves.value, "k_slices": nks.value, "lds_bytes": lds.value}
 
 
-def plan_prefill(t, n, k, cu_count=256, tile_rows=0, k_slices=0):
+def plan_prefill(t, n, k, cu_count=256, tile_rows=0, k_slices=0, group=128):
     """Launch plan of the prefill path (no context, no GPU): dict of tile_rows, k_slices, super_m, super_n, supers,
     price_us."""
     out = (C.c_size_t * 5)()
     us = C.c_double()
-    ffi.check(ffi.load().w4a16_plan_prefill(t, n, k, cu_count, tile_rows, k_slices, out, C.byref(us)))
+    ffi.check(ffi.load().w4a16_plan_prefill(t, n, k, group, cu_count, tile_rows, k_slices, out, C.byref(us)))
     return {"tile_rows": out[0], "k_slices": out[1], "super_m": out[2], "super_n": out[3], "supers": out[4],
             "price_us": us.value}
 

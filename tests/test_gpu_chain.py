@@ -439,10 +439,137 @@ def test_deferred_norm_many_partial_sums_and_glu(dec, orc):
             dec.lin_forward_deferred_norm("dg", px, t, py, ldx=k - 8)
         with pytest.raises(ops.W4a16Error):  # statistics without their count
             dec.lin_forward_deferred_norm("dg", px, t, py, stats_in=pp, n_stats_in=0, in_cols=in_cols)
-        with pytest.raises(ops.W4a16Error):  # decode regime only
-            dec.lin_forward_deferred_norm("dg", px, 17, py)
     finally:
         for p_ in (px, pp, py, pc):
+            cc.free(p_)
+
+
+@pytest.mark.parametrize("t,n,k,group,ksplit", [(40, 400, 1024, 128, -1), (300, 400, 1024, 128, -1), (130, 2048, 4096, 128, 0),
+                                                (130, 2048, 4096, 128, 4), (100, 320, 512, 32, -1), (600, 5120, 5120, 128, 0)])
+def test_deferred_norm_linear_beyond_the_decode_regime(dec, orc, t, n, k, group, ksplit):
+    """The same options on the MFMA-tiled kernel (t > 16): row factor from partial sums laid out [entries][ld], x a column
+    slice of a wider matrix, residual stream, statistics of the output (whole k range: one entry per 64 columns; split
+    over k: one per 1024-column chunk, applied by the finish kernel), norm weight, power-of-two hand-over factors."""
+    say("deferred norm prefill", t, n, k, group, ksplit)
+    ldx, in_cols, n_in = k + 512, 777, 37
+    stat_rows = n - 100
+    q, s, _ = gen.make_linear(n, k, group, 1, seed=121 + t)
+    dec.upload_lin_g("dnp", q, s, n, k, group, False)
+    xw = gen.normal_f16(15 + t, (t, ldx))
+    x = np.ascontiguousarray(xw[:, :k])
+    rng = np.random.default_rng(t)
+    ld = (t + 3) // 4 * 4
+    prev = np.zeros((n_in, ld), np.float32)
+    prev[:, :t] = (rng.standard_normal((n_in, t)) ** 2 * 100).astype(np.float32)
+    s_in = (1.0 / np.sqrt(prev.astype(np.float64).sum(0)[:t] / in_cols + 1e-6)).astype(np.float32)
+    if n * t <= 1 << 18:
+        lane = orc.gemm_lane(x, t, q, s, n, k, group, False, 16)
+    else:
+        cc_ = dec.cc
+        pxx, pyy = cc_.to_device(x), cc_.alloc(t * n * 4)
+        dec.lin_forward("dnp", pxx, pyy, t, path=ops.PATH_LANE)
+        lane = cc_.d2h(pyy, (t, n), np.float32)
+        cc_.free(pxx)
+        cc_.free(pyy)
+    resid0 = (rng.standard_normal((t, n)) * 0.5).astype(np.float32)
+    nw = (1.0 + 0.3 * rng.standard_normal(n)).astype(np.float32)
+    cc = dec.cc
+    cap = ((n + 63) // 64) * ld * 4
+    px, pp, py, ps = cc.to_device(xw), cc.to_device(prev), cc.alloc(t * n * 4), cc.alloc(cap)
+    pr, pw = cc.to_device(resid0), cc.to_device(nw)
+    dec.set_prefill_ksplit(ksplit)
+    try:
+        # factor + statistics
+        cc.memset0(ps, cap)
+        n_out = dec.lin_forward_deferred_norm("dnp", px, t, py, ldx=ldx, stats_in=pp, n_stats_in=n_in, in_cols=in_cols,
+                                              stats_out=ps, stat_rows=stat_rows)
+        say("   ", cc.last_launch_symbol(), "entries", n_out)
+        y = cc.d2h(py, (t, n), np.float32)
+        want = (s_in[:, None] * lane).astype(np.float32)
+        parity.assert_close(y, want, "deferred norm prefill t%d" % t)
+        st = cc.d2h(ps, (n_out, ld), np.float32)
+        got_ss = st.astype(np.float64).sum(0)[:t]
+        want_ss = (y[:, :stat_rows].astype(np.float64) ** 2).sum(1)
+        assert np.all(np.abs(got_ss / want_ss - 1.0) < 1e-5)
+        # f16 out = the f32 value rounded once; the statistics repeat bit for bit
+        n2 = dec.lin_forward_deferred_norm("dnp", px, t, py, out_f16=True, ldx=ldx, stats_in=pp, n_stats_in=n_in,
+                                           in_cols=in_cols, stats_out=ps, stat_rows=stat_rows)
+        assert n2 == n_out and np.array_equal(cc.d2h(py, (t, n), np.uint16), gen.f32_to_f16_bits(y))
+        assert np.array_equal(cc.d2h(ps, (n_out, ld), np.float32)[:, :t], st[:, :t])
+        # residual stream + norm weight + hand-over factors: v = resid + s_in * 2^3 * (W x); y = f16(v * nw * 2^-2)
+        dec.lin_forward_deferred_norm("dnp", px, t, py, out_f16=True, ldx=ldx, stats_in=pp, n_stats_in=n_in, in_cols=in_cols,
+                                      stats_out=ps, stat_rows=stat_rows, resid=pr, nw=pw, in_exp=3, out_exp=2)
+        v = cc.d2h(pr, (t, n), np.float32)
+        v_want = resid0 + (s_in[:, None] * np.float32(8.0)) * lane
+        parity.assert_close(v, v_want.astype(np.float32), "residual stream prefill t%d" % t)
+        y16 = cc.d2h(py, (t, n), np.uint16)
+        assert np.array_equal(y16, gen.f32_to_f16_bits((v * nw[None, :]).astype(np.float32) * np.float32(0.25)))
+        got_ss = cc.d2h(ps, (n_out, ld), np.float32).astype(np.float64).sum(0)[:t]
+        assert np.all(np.abs(got_ss / (v[:, :stat_rows].astype(np.float64) ** 2).sum(1) - 1.0) < 1e-5)
+        # without any option it is the plain prefill launch
+        dec.lin_forward_deferred_norm("dnp", px, t, py, ldx=ldx)
+        plain = dec.gemv_host("dnp", x, t=t, path=ops.PATH_PREFILL)
+        assert np.array_equal(cc.d2h(py, (t, n), np.float32).view(np.uint32), plain.view(np.uint32))
+    finally:
+        dec.set_prefill_ksplit(0)
+        for p_ in (px, pp, py, ps, pr, pw):
+            cc.free(p_)
+
+
+@pytest.mark.parametrize("t", [40, 300])
+def test_deferred_norm_glu_beyond_the_decode_regime(dec, orc, t):
+    """The gated projection at t > 16: the factor (with its power of two) reaches gate and up before act(g) * u, the
+    result leaves times 2^-out_exp."""
+    n, k, n_in, in_cols = 1024, 512, 70, 4096
+    q, s, x = gen.make_linear(n, k, 128, t, seed=177)
+    dec.upload_lin_g("dgp", q, s, n, k, 128, False)
+    ld = (t + 3) // 4 * 4
+    prev = np.zeros((n_in, ld), np.float32)
+    prev[:, :t] = (np.random.default_rng(9).standard_normal((n_in, t)) ** 2).astype(np.float32)
+    s_in = (1.0 / np.sqrt(prev.astype(np.float64).sum(0)[:t] / in_cols + 1e-6)).astype(np.float32)
+    gu = ((s_in[:, None] * np.float32(4.0)) * orc.gemm_lane(x, t, q, s, n, k, 128, False, 8)).astype(np.float32)
+    cc = dec.cc
+    px, pp, pc = cc.to_device(x), cc.to_device(prev), cc.alloc(t * (n // 2) * 2)
+    try:
+        dec.lin_forward_glu_deferred_norm("dgp", px, t, pc, stats_in=pp, n_stats_in=n_in, in_cols=in_cols, in_exp=2, out_exp=1)
+        assert dec.cc.last_launch_symbol().endswith("_glu")
+        c = _f16(cc.d2h(pc, (t, n // 2), np.uint16)).astype(np.float64) * 2.0
+        cw = _f16(orc.silu_mul_f16_rows(gu)).astype(np.float64)
+        rms = float(np.sqrt(np.mean(cw * cw)))
+        assert np.all(np.abs(c - cw) <= 2 * parity.f16_ulp(np.maximum(np.abs(cw), rms / parity.CLAMP_DIV)))
+    finally:
+        for p_ in (px, pp, pc):
+            cc.free(p_)
+
+
+@pytest.mark.parametrize("t", [40, 200])
+def test_fused_chain_prefill_regime(dec, orc, t):
+    """w4a16_chain_forward_fused beyond 16 rows (four launches per layer on the MFMA-tiled kernels, split over k where
+    the planner says so): against the oracle's fused statement, against the un-fused chain, deterministic."""
+    say("fused chain prefill regime", t)
+    hidden, n_qkv, n_ff, group, layers = 1024, 1536, 2048, 128, 4
+    shapes = {"attn_qkv": (n_qkv, hidden), "attn_output": (hidden, hidden), "ffn_gate_up": (2 * n_ff, hidden),
+              "ffn_down": (hidden, n_ff)}
+    seeds = dec.upload_chain_synth("fpf", layers, hidden, n_qkv, n_ff, group)
+    x = gen.normal_f16(61 + t, (t, hidden))
+    cc = dec.cc
+    px, py, pz = cc.to_device(x), cc.alloc(t * hidden * 2), cc.alloc(t * hidden * 2)
+    try:
+        dec.chain_forward_fused("fpf", 0, layers, px, t, py)
+        got = cc.d2h(py, (t, hidden), np.uint16)
+        assert np.all(np.isfinite(_f16(got)))
+        want = _fused_oracle(orc, "fpf", seeds, shapes, group, layers, x, 8)
+        m = parity.compare(_f16(got), _f16(want))
+        say("  fused vs oracle rel_l2", m["rel_l2"])
+        assert m["rel_l2"] < 1e-2
+        dec.chain_forward("fpf", 0, layers, px, t, pz)
+        m2 = parity.compare(_f16(got), _f16(cc.d2h(pz, (t, hidden), np.uint16)))
+        say("  fused vs unfused rel_l2", m2["rel_l2"])
+        assert m2["rel_l2"] < 1e-2
+        dec.chain_forward_fused("fpf", 0, layers, px, t, py)
+        assert np.array_equal(cc.d2h(py, (t, hidden), np.uint16), got)
+    finally:
+        for p_ in (px, py, pz):
             cc.free(p_)
 
 
@@ -570,8 +697,6 @@ def test_fused_chain_small_many_layers(dec, orc, t):
             assert np.array_equal(cc.d2h(py, (t, hidden), np.uint16), got)  # deterministic
         dec.bench_chain("fsmall", layers, px, t, py, reps=3, warmup=1, use_graph=True, fused=True)
         assert np.array_equal(cc.d2h(py, (t, hidden), np.uint16), got)  # graph replays give the same bits
-        with pytest.raises(ops.W4a16Error):
-            dec.chain_forward_fused("fsmall", 0, layers, px, 17, py)
     finally:
         for p_ in (px, py, pz):
             cc.free(p_)
