@@ -436,9 +436,10 @@ struct MoeMmStage {
 // One block = (segment of blk = 16*TT slots, group of W units); wave w owns unit group*W + w over the whole k range.
 // KS: the launch may be split over k across workgroups (dense linears run as one expert; the expert FFN never splits, and
 // its kernels are built without the epilogue that costs them registers).
-template <int G, bool SBF, bool GLU, int TT, int DEPTH, bool KS>
+// TT: the 16-slot blocks of the segment this workgroup multiplies (those that hold a slot); TTMAX: the blocks of a full
+// segment, which size a wave's share of the split-k workspace.
+template <int G, bool SBF, bool GLU, int TT, int TTMAX, int DEPTH, bool KS>
 __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
-    static_assert(DEPTH % 2 == 0, "the x double buffer alternates with the ring position");
     extern __shared__ _Float16 xs[];  // [2][16*TT][MOE_LDX]
     constexpr int GPT = W4_TILE_K / G;
     constexpr int ROWS = 16 * TT;
@@ -485,20 +486,21 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
         xg_off[p] = slot < ns ? ((unsigned)(slot / x_div) * (unsigned)k + (unsigned)(tid & 15) * 8u) * 2u : W4_OOB;
         xl_off[p] = row < ROWS ? row * MOE_LDX + (tid & 15) * 8 : -1;
     }
-    // x tiles travel global -> registers -> LDS two k tiles ahead of their use (two register sets): the gathered rows
-    // come from L2 with a latency longer than one k tile of compute
-    u4_t xreg[2][TT];
-    auto load_x = [&](int set, int kt) {
+    // x tiles travel global -> registers -> LDS two k tiles ahead of their use: the gathered rows come from L2 with a
+    // latency longer than one k tile of compute.  One register set: an iteration stores the tile loaded in the previous
+    // one and then loads the next into the same registers.
+    u4_t xreg[TT];
+    auto load_x = [&](u4_t (&r)[TT], int kt) {
 #pragma unroll
         for (int p = 0; p < TT; p++)
-            xreg[set][p] = __builtin_amdgcn_raw_buffer_load_b128(
+            r[p] = __builtin_amdgcn_raw_buffer_load_b128(
                 xr, (kt < kt_hi && xg_off[p] != W4_OOB) ? xg_off[p] + (unsigned)kt * (W4_TILE_K * 2u) : W4_OOB, 0, 0);
     };
-    auto store_x = [&](int set, int buf) {
+    auto store_x = [&](const u4_t (&r)[TT], int buf) {
         _Float16* base = xs + buf * (ROWS * MOE_LDX);
 #pragma unroll
         for (int p = 0; p < TT; p++)
-            if (xl_off[p] >= 0) *reinterpret_cast<u4_t*>(base + xl_off[p]) = xreg[set][p];
+            if (xl_off[p] >= 0) *reinterpret_cast<u4_t*>(base + xl_off[p]) = r[p];
     };
 
     const unsigned qoff[2] = {(unsigned)rbA * (unsigned)kt_n * 1024u + (unsigned)lane * 16u,
@@ -544,9 +546,23 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
                 const h8_t a = w4_deq8(qw);
                 if (G == 32) {
                     const f4_t sc = moe_scale4<G, SBF, w>(s_.s[rb]);
+                    if constexpr (TT <= 3) {
+                        // all MFMAs of the group issue before the first scaled sum: the sums of the first result run
+                        // while the matrix pipe finishes the last (T = 512: 115.4 -> 113.8 us; with four results
+                        // in flight the kernel loses more to registers than it gains)
+                        f4_t p[TT];
 #pragma unroll
-                    for (int tt = 0; tt < TT; tt++)
-                        acc[rb][tt] = w4_fma4(sc, __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], zero, 0, 0, 0), acc[rb][tt]);
+                        for (int tt = 0; tt < TT; tt++) p[tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], zero, 0, 0, 0);
+                        if constexpr (TT == 1) asm volatile("" : "+v"(p[0]));
+                        if constexpr (TT == 2) asm volatile("" : "+v"(p[0]), "+v"(p[1]));
+                        if constexpr (TT == 3) asm volatile("" : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]));
+#pragma unroll
+                        for (int tt = 0; tt < TT; tt++) acc[rb][tt] = w4_fma4(sc, p[tt], acc[rb][tt]);
+                    } else {
+#pragma unroll
+                        for (int tt = 0; tt < TT; tt++)
+                            acc[rb][tt] = w4_fma4(sc, __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], zero, 0, 0, 0), acc[rb][tt]);
+                    }
 #pragma unroll
                     for (int tt = 0; tt < TT; tt++) asm volatile("" : "+v"(acc[rb][tt]));
                 } else {
@@ -570,22 +586,29 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
         }
     };
 
-    // prologue: the slice's first x tile into LDS buffer 0, the second in registers, DEPTH weight stages in flight
-    load_x(0, kt_lo);
-    load_x(1, kt_lo + 1);
+    // prologue: the slice's first x tile into LDS buffer 0, the second in registers (both loads issued before the first
+    // is stored: the first tile's registers are free again before the accumulators are live), DEPTH weight stages in
+    // flight
+    {
+        u4_t first[TT];
+        load_x(first, kt_lo);
+        load_x(xreg, kt_lo + 1);
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) load_w(stage[d], kt_lo + d);
-    store_x(0, 0);
+        for (int d = 0; d < DEPTH; d++) load_w(stage[d], kt_lo + d);
+        store_x(first, 0);
+    }
     __syncthreads();
+    int xb = 0;  // LDS buffer of the tile being multiplied
     for (int kt0 = kt_lo; kt0 < kt_hi; kt0 += DEPTH) {
 #pragma unroll
-        for (int d = 0; d < DEPTH; d++) {  // DEPTH is even: register set and LDS buffer of the slice's i-th tile are i & 1 = d & 1
+        for (int d = 0; d < DEPTH; d++) {
             const int kt = kt0 + d;
-            if (kt < kt_hi) compute(stage[d], d & 1);
+            if (kt < kt_hi) compute(stage[d], xb);
             load_w(stage[d], kt + DEPTH);
-            store_x((d + 1) & 1, (d + 1) & 1);  // tile kt+1, loaded an iteration ago, into the buffer tile kt-1 was read from
-            load_x(d & 1, kt + 2);              // out of range past the last tile: zeros, no traffic
+            store_x(xreg, xb ^ 1);  // tile kt+1, loaded an iteration ago, into the buffer tile kt-1 was read from
+            load_x(xreg, kt + 2);   // out of range past the last tile: zeros, no traffic
             __syncthreads();
+            xb ^= 1;
         }
     }
 
@@ -597,7 +620,7 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
         // cache-bypassing loads behind an agent-scope acquire fence in the wave that drew the last ticket; the slice
         // offset travels in the vector offset (scalar offset 0) so that the compiler inserts the wait state a write to
         // the data registers of a 16-byte store needs, and the tiles stay live until the stores have completed.
-        constexpr unsigned PER_WAVE = 2u * TT * 1024u;
+        constexpr unsigned PER_WAVE = 2u * TTMAX * 1024u;
         const unsigned per_slice = gridDim.x * (unsigned)W * PER_WAVE;
         const __amdgpu_buffer_rsrc_t wr = w4_make_rsrc(ws, per_slice * (unsigned)nks);
         const unsigned mine = (blockIdx.x * (unsigned)W + (unsigned)wave) * PER_WAVE + (unsigned)lane * 16u;
@@ -646,18 +669,39 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     }
 }
 
+// A segment's slots are a prefix of it (the alignment pads an expert's run at its end), so the first slot of each
+// 16-slot block tells whether the block holds any: the workgroup runs the body built for the blocks that do, and the
+// MFMAs, scaled sums and x rows of all-padding blocks are never issued (128 experts, top-8, T = 512: runs of 32 +- 6
+// slots in 48-slot segments, every other expert fills two blocks of three).
+template <int G, bool SBF, bool GLU, int TT, int DEPTH, bool KS>
+__device__ __forceinline__ void moe_mm_entry(MOE_PARAMS) {
+    if constexpr (TT == 1) {
+        moe_mm_body<G, SBF, GLU, 1, 1, DEPTH, KS>(MOE_ARGS);
+    } else {
+        const int units = GLU ? row_blocks >> 1 : (row_blocks + 1) >> 1;
+        const int seg = blockIdx.x / ((units + wpb - 1) / wpb);
+        int live = 1;
+#pragma unroll
+        for (int p = 1; p < TT; p++) live += sorted_ids[seg * blk + 16 * p] < ns ? 1 : 0;
+        if (live == 1) moe_mm_body<G, SBF, GLU, 1, TT, DEPTH, KS>(MOE_ARGS);
+        else if (TT == 2 || live == 2) moe_mm_body<G, SBF, GLU, 2, TT, DEPTH, KS>(MOE_ARGS);
+        else if (TT == 3 || live == 3) moe_mm_body<G, SBF, GLU, TT >= 3 ? 3 : 2, TT, DEPTH, KS>(MOE_ARGS);
+        else moe_mm_body<G, SBF, GLU, TT, TT, DEPTH, KS>(MOE_ARGS);
+    }
+}
+
 #define MOE_DEC_KERNEL(NAME, G, SBF, GLU, XL, DEPTH)                                  \
     extern "C" __global__ __launch_bounds__(512) void NAME(MOE_PARAMS) {              \
         moe_dec_body<G, SBF, GLU, XL, DEPTH>(MOE_ARGS);                               \
     }
 #define MOE_MM_KERNEL(NAME, G, SBF, GLU, TT, DEPTH, KS)                               \
     extern "C" __global__ __launch_bounds__(512) void NAME(MOE_PARAMS) {              \
-        moe_mm_body<G, SBF, GLU, TT, DEPTH, KS>(MOE_ARGS);                            \
+        moe_mm_entry<G, SBF, GLU, TT, DEPTH, KS>(MOE_ARGS);                           \
     }
 // Ring depths, from sweeps on the 128-expert shape: the one-slot segments of the direct mode run best with two k tiles
 // in flight per wave (T = 4..12: 9-11 % faster than four: fewer registers, more waves resident at once); so do the
 // segments of up to 16 slots (5 % faster than three).  The LDS-staged kernels keep two (group 32) or four (group 128);
-// their ring depth must be even (the x double buffer alternates with the ring position).
+// the LDS buffer of a k tile alternates on its own, whatever the ring depth.
 #define MOE_FAMILY(PFX, G, SBF, DMM)                             \
     MOE_DEC_KERNEL(PFX##_dec_glu_x1, G, SBF, true, 1, 2)     \
     MOE_DEC_KERNEL(PFX##_dec_glu_x4, G, SBF, true, 4, 2)     \
@@ -676,8 +720,11 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
     MOE_MM_KERNEL(PFX##_mm_lin_t3_ks, G, SBF, false, 3, DMM, true) \
     MOE_MM_KERNEL(PFX##_mm_lin_t4_ks, G, SBF, false, 4, DMM, true)
 
-MOE_FAMILY(w4a16_moe_g32_f16, 32, false, 2)
-MOE_FAMILY(w4a16_moe_g32_bf16, 32, true, 2)
+#ifndef MOE_G32_DEPTH
+#define MOE_G32_DEPTH 2
+#endif
+MOE_FAMILY(w4a16_moe_g32_f16, 32, false, MOE_G32_DEPTH)
+MOE_FAMILY(w4a16_moe_g32_bf16, 32, true, MOE_G32_DEPTH)
 MOE_FAMILY(w4a16_moe_g128_f16, 128, false, 4)
 MOE_FAMILY(w4a16_moe_g128_bf16, 128, true, 4)
 

