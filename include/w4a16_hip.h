@@ -153,6 +153,15 @@ int w4a16_lin_drop_raw(w4a16_ctx* ctx, const char* name);
  * fused gate|up arenas (upload.rs:1116-1235).  Parts need the same k, group and scale type and their as-given operands;
  * drop_parts != 0 unregisters them afterwards.  A fused gate|up linear is what w4a16_lin_forward_glu takes. */
 int w4a16_lin_fuse(w4a16_ctx* ctx, const char* name, const char* const* parts, size_t n_parts, int drop_parts);
+/* gemv_multi_dev / gemv_multi_t_dev (w4a16_dec/kernels/gemv.rs:189-332) over the segment table {weights, scales, out,
+ * n, k} that build_multi_tables writes per layer (w4a16_dec/buffers.rs:229-366): ONE decode launch for the linears
+ * fused under `name`, every part into its own output.  outs_dev: n_outs device addresses (a host array), n_outs = the
+ * number of parts given to w4a16_lin_fuse (2..4); output i receives f16 or f32 [t][n_i], the rows of part i, with the
+ * bits w4a16_lin_forward writes to y[:, first_i : first_i + n_i] of the fused linear.  Parts must be multiples of 16
+ * rows (W4A16_ERR_SHAPE otherwise); decode steps only: t > 16 is W4A16_ERR_UNSUPPORTED (w4a16_lin_forward then writes
+ * the parts side by side in one tensor, which the consumers in this library read through a row stride). */
+int w4a16_lin_forward_multi(w4a16_ctx* ctx, const char* name, uint64_t x_dev, const uint64_t* outs_dev, size_t n_outs,
+                            size_t t, int out_f16);
 /* lin_spec (w4a16_dec/mod.rs:1193-1206): shape of a registered linear. */
 int w4a16_lin_info(w4a16_ctx* ctx, const char* name, size_t* n, size_t* k, size_t* group, int* scale_bf16,
                    int* has_tiled, int* has_raw);

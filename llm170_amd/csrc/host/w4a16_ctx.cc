@@ -63,6 +63,10 @@ static const char* const kDecodeSyms[] = {
     "w4a16_decode_g128_bf16_glu_x1", "w4a16_decode_g128_bf16_glu_x2", "w4a16_decode_g128_bf16_glu_x4",
     "w4a16_decode_g32_f16_glu_x1", "w4a16_decode_g32_f16_glu_x2", "w4a16_decode_g32_f16_glu_x4",
     "w4a16_decode_g32_bf16_glu_x1", "w4a16_decode_g32_bf16_glu_x2", "w4a16_decode_g32_bf16_glu_x4",
+    "w4a16_decode_g128_f16_multi_x1", "w4a16_decode_g128_f16_multi_x2", "w4a16_decode_g128_f16_multi_x4",
+    "w4a16_decode_g128_bf16_multi_x1", "w4a16_decode_g128_bf16_multi_x2", "w4a16_decode_g128_bf16_multi_x4",
+    "w4a16_decode_g32_f16_multi_x1", "w4a16_decode_g32_f16_multi_x2", "w4a16_decode_g32_f16_multi_x4",
+    "w4a16_decode_g32_bf16_multi_x1", "w4a16_decode_g32_bf16_multi_x2", "w4a16_decode_g32_bf16_multi_x4",
     nullptr};
 static const char* const kPrefillSyms[] = {"w4a16_prefill_g128_f16", "w4a16_prefill_g128_bf16", "w4a16_prefill_g32_f16",
                                            "w4a16_prefill_g32_bf16", "w4a16_prefill_g128_f16_m64", "w4a16_prefill_g128_bf16_m64", "w4a16_prefill_g32_f16_m64",

@@ -25,6 +25,7 @@ struct W4Lin {
     size_t row_blocks = 0;
     bool scales_regular = true;  // every scale finite and non-zero (the MFMA prefill kernel divides by them)
     float row_norm_max = -1.0f;  // largest row norm of the dequantised weights, computed on first request (< 0: not yet)
+    std::vector<size_t> part_n;  // a fused linear: the rows of each part, in order (empty for a linear uploaded as one)
 };
 
 // The experts of one MoE layer: two arenas in the tiled layout, experts at a fixed stride

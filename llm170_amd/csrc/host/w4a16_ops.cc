@@ -220,8 +220,18 @@ static int check_decode_norm(const W4Lin& L, size_t t, const DecodeNorm& nm) {
     return 0;
 }
 
+// Host mirror of DecodeMulti (kernels/decode.hip): outputs and first rows of parts 1..3 of a fused linear; a first row
+// of INT_MAX means "no such part" (the value every single-output launch passes).
+struct DecodeMultiHost {
+    uint64_t out[3] = {0, 0, 0};
+    int first[3] = {0x7fffffff, 0x7fffffff, 0x7fffffff};
+    int reserved = 0;
+};
+static_assert(sizeof(DecodeMultiHost) == 40, "DecodeMulti is three pointers and four ints");
+
 static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y, size_t t, int out_f16,
-                         DecodeNorm* norm = nullptr, const DecodeWorkspace* fixed_ws = nullptr) {
+                         DecodeNorm* norm = nullptr, const DecodeWorkspace* fixed_ws = nullptr,
+                         const DecodeMultiHost* multi = nullptr) {
     if (t == 0 || t > 16) return w4_fail(W4A16_ERR_SHAPE, "decode: t=%zu outside 1..16", t);
     if (!L.q_tiled) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode: linear has no tiled copy (needs k %% 128 == 0)");
     if (L.row_blocks * (L.k / 128) * 1024 >= 0x80000000ull)
@@ -235,7 +245,7 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     in.group = L.group;
     in.t = t;
     in.cu_count = ctx->cu_count;
-    in.rows_per_wave = ctx->decode_rows_per_wave;
+    in.rows_per_wave = multi ? 32 : ctx->decode_rows_per_wave;  // the kernels with one output per part are built for two row blocks per wave
     in.waves_per_block = ctx->decode_waves_per_block;
     in.ksplit = ctx->decode_ksplit;
     in.extra_lds = decode_stats_lds(nm);
@@ -247,7 +257,10 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     // x loads per k tile: one serves up to 4 token rows, two up to 8, four up to 16 (kernels/decode.hip)
     const int xl = t <= 4 ? 1 : t <= 8 ? 2 : 4;
     char sym[64];
-    snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_rb%d_x%d", L.group, L.scale_bf16 ? "bf16" : "f16", rb, xl);
+    if (multi)
+        snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_multi_x%d", L.group, L.scale_bf16 ? "bf16" : "f16", xl);
+    else
+        snprintf(sym, sizeof sym, "w4a16_decode_g%zu_%s_rb%d_x%d", L.group, L.scale_bf16 ? "bf16" : "f16", rb, xl);
     uint64_t qt = L.q_tiled, st = L.s_tiled;
     int row_blocks = (int)L.row_blocks, ki = (int)L.k, ni = (int)L.n, ti = (int)t, of = out_f16 ? 1 : 0;
     DecodeWorkspace W;
@@ -259,8 +272,14 @@ static int launch_decode(w4a16_ctx* ctx, const W4Lin& L, uint64_t x, uint64_t y,
     int act_kind = 0;  // no activation in the plain linear
     float in_scale = std::ldexp(1.0f, nm.in_exp), out_scale = std::ldexp(1.0f, -nm.out_exp);
     nm.n_stats_out = s_out ? std::min(blocks, (size_t)ceil_div((size_t)stat_rows, (size_t)rb * 16)) : 0;
+    DecodeMultiHost mo;
+    if (multi) {
+        if (s_out || resid || nw) return w4_fail(W4A16_ERR_UNSUPPORTED, "decode: a launch with one output per part takes no statistics, residual or norm weight");
+        mo = *multi;
+    }
+    // the last entry is read by the kernels with one output per part only (the argument count is the kernel's own)
     void* params[] = {&qt, &st, &x, &y, &row_blocks, &ki, &ni, &ti, &of, &ws, &tk, &waves, &nks, &kt_per_slice, &kt_per_wave,
-                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind, &in_scale, &out_scale};
+                      &ldx, &s_in, &n_in, &inv_cols, &s_out, &stat_rows, &resid, &nw, &act_kind, &in_scale, &out_scale, &mo};
     return w4_launch(ctx, sym, (unsigned)blocks, (unsigned)nks, (unsigned)(waves * 64), P.shmem, params);
 }
 
@@ -622,6 +641,7 @@ extern "C" int w4a16_lin_fuse(w4a16_ctx* ctx, const char* name, const char* cons
                            name, parts[i], L.k, L.group, L.scale_bf16, F.k, F.group, F.scale_bf16);
         }
         F.n += L.n;
+        F.part_n.push_back(L.n);
         F.scales_regular = F.scales_regular && L.scales_regular;
     }
     if (F.n > 0x7fffffffu) return w4_fail(W4A16_ERR_SHAPE, "lin_fuse %s: n=%zu too large", name, F.n);
@@ -650,6 +670,39 @@ extern "C" int w4a16_lin_fuse(w4a16_ctx* ctx, const char* name, const char* cons
             }
         }
     return 0;
+}
+
+// One decode launch over a fused linear with one output per part (the reference's multi-linear GEMV: a table of
+// {weights, scales, out, n, k} segments, w4a16_dec/buffers.rs:229-366, launched by kernels/gemv.rs:189-332).
+extern "C" int w4a16_lin_forward_multi(w4a16_ctx* ctx, const char* name, uint64_t x_dev, const uint64_t* outs_dev,
+                                       size_t n_outs, size_t t, int out_f16) {
+    if (!ctx || !name || !outs_dev) return w4_fail(W4A16_ERR_ARG, "lin_forward_multi: null argument");
+    W4Lin* L = nullptr;
+    W4_TRY(w4_find_lin(ctx, name, &L));
+    if (L->part_n.size() < 2)
+        return w4_fail(W4A16_ERR_ARG, "lin_forward_multi %s: not a fused linear (w4a16_lin_fuse makes one)", name);
+    if (n_outs != L->part_n.size())
+        return w4_fail(W4A16_ERR_ARG, "lin_forward_multi %s: %zu outputs for %zu parts", name, n_outs, L->part_n.size());
+    if (n_outs > 4)
+        return w4_fail(W4A16_ERR_UNSUPPORTED, "lin_forward_multi %s: %zu parts (one launch writes up to four outputs)", name, n_outs);
+    if (!x_dev) return w4_fail(W4A16_ERR_ARG, "lin_forward_multi %s: null x", name);
+    if (t == 0) return w4_fail(W4A16_ERR_SHAPE, "lin_forward_multi %s: t=0", name);
+    if (t > 16)
+        return w4_fail(W4A16_ERR_UNSUPPORTED, "lin_forward_multi %s: t=%zu: one output per part exists for decode steps (t <= 16); beyond, w4a16_lin_forward writes the parts side by side in one [t][n] tensor", name, t);
+    DecodeMultiHost mo;
+    size_t first = 0;
+    for (size_t i = 0; i < n_outs; i++) {
+        if (!outs_dev[i]) return w4_fail(W4A16_ERR_ARG, "lin_forward_multi %s: output %zu is null", name, i);
+        if (L->part_n[i] % 16 != 0)
+            return w4_fail(W4A16_ERR_SHAPE, "lin_forward_multi %s: part %zu has %zu rows; parts must be multiples of 16 rows (a 16-row block writes one output)", name, i, L->part_n[i]);
+        if (i > 0) {
+            mo.out[i - 1] = outs_dev[i];
+            mo.first[i - 1] = (int)first;
+        }
+        first += L->part_n[i];
+    }
+    W4_TRY(w4_hip(hipSetDevice(ctx->device), "hipSetDevice"));
+    return launch_decode(ctx, *L, x_dev, outs_dev[0], t, out_f16, nullptr, nullptr, &mo);
 }
 
 // Second half of a registration: build the tiled copy from the as-given operands already on the device and enter

@@ -55,14 +55,26 @@ __device__ __forceinline__ u4_t w4_row_shl(u4_t v) {
 // GLU (RB = 2 only): the linear is a fused gate|up projection (rows 0..n/2 gate, n/2..n up); the wave owns gate row
 // block u and up row block u + n/32 and writes f16(silu(gate) * up) [t][n/2] instead of the two sums — the
 // elementwise kernel between the projections (assets/ew.cu:9-32) folded into the producer, same f32 arithmetic.
-template <int G, bool SBF, int RB, int DEPTH, int XL, bool GLU = false>
+// Outputs of a launch over fused linears (plain kernels only).  Part 0 writes y; part j >= 1 starts at output row
+// first[j - 1] (a multiple of 16) and writes out[j - 1], each part as its own [t][rows of the part] tensor.  A launch
+// with one output passes first[] = INT_MAX: every row then selects y and the row length n.
+struct DecodeMulti {
+    unsigned long long out[3];
+    int first[3];
+    int reserved;
+};
+
+#define DECODE_ONE_OUTPUT (DecodeMulti{{0ull, 0ull, 0ull}, {0x7fffffff, 0x7fffffff, 0x7fffffff}, 0})
+
+template <int G, bool SBF, int RB, int DEPTH, int XL, bool GLU = false, bool MULTI = false>
 __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const uint16_t* __restrict__ st,
                                             const uint16_t* __restrict__ x, void* __restrict__ y, int row_blocks,
                                             int k, int n, int t, int out_f16, f4_t* ws, int* tickets, int W, int nks,
                                             int kt_per_slice, int kt_per_wave, int ldx,
                                             const float* __restrict__ stats_in, int n_stats_in, float inv_cols_in,
                                             float* __restrict__ stats_out, int stat_rows, float* __restrict__ resid,
-                                            const float* __restrict__ nw, int act_kind, float in_scale, float out_scale) {
+                                            const float* __restrict__ nw, int act_kind, float in_scale, float out_scale,
+                                            DecodeMulti mo) {
     extern __shared__ f4_t red[];  // [W][RB][64] partial tiles of the in-block split-K, then the waves' staged scales
     constexpr int GPT = W4_TILE_K / G;  // scale groups per k tile
     constexpr int C = 4 / XL;           // 32-k chunks (MFMAs) served by one x load
@@ -383,24 +395,39 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
     for (int rb = 0; rb < RB; rb++) {
         if (nb0 + rb >= row_blocks) break;
         const int row = (nb0 + rb) * 16 + 4 * g;
+        // the part this row block belongs to (uniform: parts start at multiples of 16): its output, first row and end
+        const int rb_row = (nb0 + rb) * 16;
+        unsigned long long base = reinterpret_cast<unsigned long long>(y);
+        int first = 0, end = n;
+        if constexpr (MULTI) {
+            end = min(mo.first[0], n);
+#pragma unroll
+            for (int j = 0; j < 3; j++)
+                if (rb_row >= mo.first[j]) {
+                    base = mo.out[j];
+                    first = mo.first[j];
+                    end = j < 2 ? min(mo.first[j + 1], n) : n;
+                }
+        }
+        const size_t at = (size_t)m * (size_t)(end - first) + (size_t)(row - first);
         if (out_f16) {
-            _Float16* yo = reinterpret_cast<_Float16*>(y) + (size_t)m * n + row;
-            if (row + 3 < n) {
+            _Float16* yo = reinterpret_cast<_Float16*>(base) + at;
+            if (row + 3 < end) {
                 h4_t v = {(_Float16)acc[rb][0], (_Float16)acc[rb][1], (_Float16)acc[rb][2], (_Float16)acc[rb][3]};
                 *reinterpret_cast<h4_t*>(yo) = v;
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    if (row + i < n) yo[i] = (_Float16)acc[rb][i];
+                    if (row + i < end) yo[i] = (_Float16)acc[rb][i];
             }
         } else {
-            float* yo = reinterpret_cast<float*>(y) + (size_t)m * n + row;
-            if (row + 3 < n) {
+            float* yo = reinterpret_cast<float*>(base) + at;
+            if (row + 3 < end) {
                 *reinterpret_cast<f4_t*>(yo) = acc[rb];
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    if (row + i < n) yo[i] = acc[rb][i];
+                    if (row + i < end) yo[i] = acc[rb][i];
             }
         }
     }
@@ -433,7 +460,27 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                                                         float in_scale, float out_scale) {           \
         decode_body<G, SBF, RB, DECODE_DEPTH(BUDGET, G, RB, XL), XL>(                                                \
             qt, st, x, y, row_blocks, k, n, t, out_f16, ws, tickets, waves, nks, kt_per_slice, kt_per_wave, ldx,     \
-            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw, act_kind, in_scale, out_scale);                           \
+            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw, act_kind, in_scale, out_scale,       \
+            DECODE_ONE_OUTPUT);                                                                                      \
+    }
+// The same kernel with one output per part of a fused linear (two row blocks per wave): a symbol of its own, because
+// the 40 more bytes of kernel arguments cost every launch 0.2 us, whether it has parts or not (measured on the 27B
+// shapes at t = 1 and 4).
+#define DECODE_MULTI_KERNEL_X(NAME, G, SBF, XL, BUDGET, ATTR)                                                         \
+    extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
+                                                                        const uint16_t* x, void* y, int row_blocks,  \
+                                                                        int k, int n, int t, int out_f16, f4_t* ws,  \
+                                                                        int* tickets, int waves, int nks,            \
+                                                                        int kt_per_slice, int kt_per_wave, int ldx,  \
+                                                                        const float* stats_in, int n_stats_in,       \
+                                                                        float inv_cols_in, float* stats_out,         \
+                                                                        int stat_rows, float* resid,                 \
+                                                                        const float* nw, int act_kind,               \
+                                                                        float in_scale, float out_scale,             \
+                                                                        DecodeMulti mo) {                            \
+        decode_body<G, SBF, 2, DECODE_DEPTH(BUDGET, G, 2, XL), XL, false, true>(                                     \
+            qt, st, x, y, row_blocks, k, n, t, out_f16, ws, tickets, waves, nks, kt_per_slice, kt_per_wave, ldx,     \
+            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw, act_kind, in_scale, out_scale, mo);  \
     }
 #define DECODE_GLU_KERNEL_X(NAME, G, SBF, XL, BUDGET, ATTR)                                                           \
     extern "C" __global__ __launch_bounds__(512) ATTR void NAME##_x##XL(const u4_t* qt, const uint16_t* st,          \
@@ -448,7 +495,8 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
                                                                         float in_scale, float out_scale) {           \
         decode_body<G, SBF, 2, DECODE_DEPTH(BUDGET, G, 2, XL), XL, true>(                                            \
             qt, st, x, y, row_blocks, k, n, t, out_f16, ws, tickets, waves, nks, kt_per_slice, kt_per_wave, ldx,     \
-            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw, act_kind, in_scale, out_scale);                           \
+            stats_in, n_stats_in, inv_cols_in, stats_out, stat_rows, resid, nw, act_kind, in_scale, out_scale,       \
+            DECODE_ONE_OUTPUT);                                                                                      \
     }
 #define DECODE_HI __attribute__((amdgpu_waves_per_eu(6, 6)))
 #define DECODE_MID __attribute__((amdgpu_waves_per_eu(5, 5)))
@@ -477,6 +525,17 @@ DECODE_KERNEL_LO3(w4a16_decode_g128_bf16_rb4, 128, true, 4)
 DECODE_KERNEL_LO3(w4a16_decode_g32_bf16_rb1, 32, true, 1)
 DECODE_KERNEL_LO3(w4a16_decode_g32_bf16_rb2, 32, true, 2)
 DECODE_KERNEL_LO3(w4a16_decode_g32_bf16_rb4, 32, true, 4)
+// one output per part of a fused linear
+#define DECODE_MULTI_G128(NAME, SBF)                                                                       \
+    DECODE_MULTI_KERNEL_X(NAME, 128, SBF, 1, 24, DECODE_HI) DECODE_MULTI_KERNEL_X(NAME, 128, SBF, 2, 24, DECODE_MID) \
+    DECODE_MULTI_KERNEL_X(NAME, 128, SBF, 4, 64, DECODE_LO)
+#define DECODE_MULTI_G32(NAME, SBF)                                                                      \
+    DECODE_MULTI_KERNEL_X(NAME, 32, SBF, 1, 24, DECODE_LO) DECODE_MULTI_KERNEL_X(NAME, 32, SBF, 2, 24, DECODE_LO) \
+    DECODE_MULTI_KERNEL_X(NAME, 32, SBF, 4, 24, DECODE_LO)
+DECODE_MULTI_G128(w4a16_decode_g128_f16_multi, false)
+DECODE_MULTI_G128(w4a16_decode_g128_bf16_multi, true)
+DECODE_MULTI_G32(w4a16_decode_g32_f16_multi, false)
+DECODE_MULTI_G32(w4a16_decode_g32_bf16_multi, true)
 // fused gate|up with the SiLU*up epilogue (two row blocks per wave by construction)
 #define DECODE_GLU_G128(NAME, SBF)                                                                     \
     DECODE_GLU_KERNEL_X(NAME, 128, SBF, 1, 24, DECODE_HI) DECODE_GLU_KERNEL_X(NAME, 128, SBF, 2, 24, DECODE_MID) \

@@ -80,6 +80,8 @@ _SIGS = {
     "w4a16_dequant_dump": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int, C.c_uint64]),
     "w4a16_lin_untile": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_uint64]),
     "w4a16_lin_fuse": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_char_p), C.c_size_t, C.c_int]),
+    "w4a16_lin_forward_multi": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64, C.POINTER(C.c_uint64), C.c_size_t, C.c_size_t,
+                                          C.c_int]),
     "w4a16_set_decode_shape": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "w4a16_set_decode_ksplit": (C.c_int, [C.c_void_p, C.c_int]),
     "w4a16_set_prefill_tile": (C.c_int, [C.c_void_p, C.c_int]),

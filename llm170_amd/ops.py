@@ -231,6 +231,12 @@ class W4a16Dec:
         arr = (C.c_char_p * len(parts))(*[p.encode() for p in parts])
         ffi.check(self.cc.lib.w4a16_lin_fuse(self.cc.h, name.encode(), arr, len(parts), int(bool(drop_parts))))
 
+    def lin_forward_multi(self, name, x_dev, outs_dev, t, out_f16=False):
+        """gemv_multi_t_dev (w4a16_dec/kernels/gemv.rs:270-300): one decode launch over a fused linear, one output per
+        part."""
+        arr = (C.c_uint64 * len(outs_dev))(*outs_dev)
+        ffi.check(self.cc.lib.w4a16_lin_forward_multi(self.cc.h, name.encode(), x_dev, arr, len(outs_dev), t, int(bool(out_f16))))
+
     def lin_spec(self, name):
         n, k, g = C.c_size_t(), C.c_size_t(), C.c_size_t()
         bf, tiled, raw = C.c_int(), C.c_int(), C.c_int()
