@@ -94,6 +94,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     extern __shared__ _Float16 lds[];  // 2 stages x [PF_BM][PF_LDA]; then PF_BM ints: slot ids (grouped) / row factors (dense)
     constexpr int GPT = W4_TILE_K / G;
     constexpr int PF_BM = 32 * MI, PF_STAGE_BYTES = PF_BM * PF_LDA * 2;
+    constexpr bool PF_WAVE_PRIO = MI <= 3 && G == 128;  // see the k loop
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave;  // 4 waves along n
@@ -246,6 +247,12 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
                 //   MFMA of the group, with the scale of the next k tile (already loaded), so the VALU work of tile j
                 //   runs in the shadow of the MFMAs of tiles j+1.. instead of stalling the next stage's first MFMAs;
                 //   group 32: at the first k16 of each 32-k group, before the tile's first MFMA.
+                // Wave priority (the 64- and 96-row tiles, three waves per SIMD): raised while a stage's MFMAs issue,
+                // dropped for the accumulator rescale at the end of a k tile, so that a wave in that VALU-only stretch
+                // yields the issue port to the waves that feed the matrix pipe (M = 512: 186 -> 180 us, M = 1024:
+                // 328 -> 317 us on 5120 x 34816; 17408 x 5120 at M = 4096: 630 -> 620 us).  With two waves per SIMD
+                // (the 128-row tile) the same costs 1 % at M = 4096 and is left out.
+                if (PF_WAVE_PRIO && kbl == 0) __builtin_amdgcn_s_setprio(1);
                 const bool boundary32 = G == 32 && h == 0;
                 float ratio[2] = {1.f, 1.f};
                 if (boundary32) {
@@ -285,6 +292,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
                     }
                 }
                 if (last128) {
+                    if (PF_WAVE_PRIO) __builtin_amdgcn_s_setprio(0);
 #pragma unroll
                     for (int ni = 0; ni < 2; ni++)
 #pragma unroll
