@@ -240,7 +240,9 @@ __device__ __forceinline__ void moe_dec_body(MOE_PARAMS) {
     for (int r = -1; r < rounds; r++) {
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
+            __builtin_amdgcn_s_setprio(1);  // compute ahead of the waves that are queueing loads (1-2 % at T <= 4)
             if (r >= 0) compute(stage[d]);
+            __builtin_amdgcn_s_setprio(0);
             __builtin_amdgcn_sched_barrier(0);
             load(stage[d], kt0 + (r + 1) * DEPTH + d);
             __builtin_amdgcn_sched_barrier(0);
@@ -359,7 +361,9 @@ __device__ __forceinline__ void moe_down_sum_body(const char* __restrict__ qa, c
     for (int r = -1; r < rounds; r++) {
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
+            __builtin_amdgcn_s_setprio(1);  // compute ahead of the waves that are queueing loads (1-2 % at T <= 4)
             if (r >= 0) compute(stage[d]);
+            __builtin_amdgcn_s_setprio(0);
             __builtin_amdgcn_sched_barrier(0);
             load(stage[d], (r + 1) * DEPTH + d);
             __builtin_amdgcn_sched_barrier(0);
@@ -603,7 +607,10 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
             const int kt = kt0 + d;
+            // a wave that holds a landed tile issues ahead of the waves that are queueing loads (about 1 % at every T)
+            __builtin_amdgcn_s_setprio(1);
             if (kt < kt_hi) compute(stage[d], xb);
+            __builtin_amdgcn_s_setprio(0);
             load_w(stage[d], kt + DEPTH);
             store_x(xreg, xb ^ 1);  // tile kt+1, loaded an iteration ago, into the buffer tile kt-1 was read from
             load_x(xreg, kt + 2);   // out of range past the last tile: zeros, no traffic
