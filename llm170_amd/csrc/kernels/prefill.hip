@@ -94,7 +94,6 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     extern __shared__ _Float16 lds[];  // 2 stages x [PF_BM][PF_LDA]; then PF_BM ints: slot ids (grouped) / row factors (dense)
     constexpr int GPT = W4_TILE_K / G;
     constexpr int PF_BM = 32 * MI, PF_STAGE_BYTES = PF_BM * PF_LDA * 2;
-    constexpr bool PF_WAVE_PRIO = MI <= 3 && G == 128;  // see the k loop
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave;  // 4 waves along n
@@ -226,6 +225,8 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     const int kt_lo = DENSE ? (kt_n * (int)blockIdx.y) / (int)gridDim.y : 0,
               kt_hi = DENSE ? (kt_n * ((int)blockIdx.y + 1)) / (int)gridDim.y : kt_n;
     const int stages = 2 * kt_hi;
+    // wave priority over a stage's MFMAs (see the k loop): the 64- and 96-row tiles, and launches split over k
+    const bool PF_WAVE_PRIO = G == 128 && (MI <= 3 || (DENSE && gridDim.y > 1));
 
     load_a(2 * kt_lo, 0);
     load_b(bq, sc, kt_lo);
@@ -251,7 +252,8 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
                 // dropped for the accumulator rescale at the end of a k tile, so that a wave in that VALU-only stretch
                 // yields the issue port to the waves that feed the matrix pipe (M = 512: 186 -> 180 us, M = 1024:
                 // 328 -> 317 us on 5120 x 34816; 17408 x 5120 at M = 4096: 630 -> 620 us).  With two waves per SIMD
-                // (the 128-row tile) the same costs 1 % at M = 4096 and is left out.
+                // (the 128-row tile) the same costs 1 % at M = 4096 on that shape and gains 1-2 % in launches split over
+                // k (17408 x 5120 at M = 1024, three slices: 173 -> 169 us), so that tile takes it in split launches.
                 if (PF_WAVE_PRIO && kbl == 0) __builtin_amdgcn_s_setprio(1);
                 const bool boundary32 = G == 32 && h == 0;
                 float ratio[2] = {1.f, 1.f};
