@@ -796,6 +796,32 @@ def test_scaled_handover_is_exact(dec, e, t):
             cc.free(p_)
 
 
+@pytest.mark.parametrize("rows", [2, 65])
+def test_scaled_handover_error_bound_with_a_large_exponent(dec, rows):
+    """A hand-over factor far larger than the values need (out_exp = 9 on outputs of magnitude ~1): elements below
+    2^(out_exp - 14) leave as f16 subnormals.  Against the f32 output of the same launch shape the handed-over value times
+    2^out_exp is within half an f16 step of a normal value or 2^(out_exp - 25) of a subnormal one, the bound the header
+    states — in the decode kernel (2 rows) and in the MFMA-tiled one (65 rows)."""
+    say("scaled hand-over bound", rows)
+    cc = dec.cc
+    n1, k1, e = 1024, 512, 9
+    q1, s1, x = gen.make_linear(n1, k1, 128, rows, seed=81)
+    dec.upload_lin_g("shb", q1, s1, n1, k1, 128, False)
+    px, pf, ph = cc.to_device(x), cc.alloc(rows * n1 * 4), cc.alloc(rows * n1 * 2)
+    try:
+        dec.lin_forward_deferred_norm("shb", px, rows, pf, out_f16=False, in_exp=0, out_exp=0)
+        dec.lin_forward_deferred_norm("shb", px, rows, ph, out_f16=True, in_exp=0, out_exp=e)
+        v = cc.d2h(pf, (rows, n1), np.float32).astype(np.float64)
+        got = np.ldexp(gen.f16_bits_to_f32(cc.d2h(ph, (rows, n1), np.uint16)).astype(np.float64), e)
+        small = np.abs(v) < 2.0 ** (e - 14)
+        assert small.mean() > 0.01 and (~small).mean() > 0.5  # both kinds occur
+        bound = np.where(small, 2.0 ** (e - 25), np.abs(v) * 2.0 ** -11)
+        assert np.all(np.abs(got - v) <= bound * 1.0000001), float((np.abs(got - v) / bound).max())
+    finally:
+        for p_ in (px, pf, ph):
+            cc.free(p_)
+
+
 def test_fused_chain_keeps_large_outputs_in_range(dec, orc):
     """Weights thirty times larger than the other chains': the down projection's output passes 65504, so an un-scaled
     f16 hand-over would carry Inf across the layer boundary.  The chain with the normalisations deferred stays finite
