@@ -540,33 +540,18 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
             for (int tt = 0; tt < TT; tt++) b[tt] = *reinterpret_cast<const h8_t*>(xb + tt * 16 * MOE_LDX + w * 32);
 #pragma unroll
             for (int rb = 0; rb < 2; rb++) {
-                // G = 32: every 32-k group's products are scaled on their own, and left alone the compiler issues all 8 * TT
-                // MFMAs of a k tile into separate result registers before the first scaled sum (220 VGPRs at TT = 3,
-                // two waves per SIMD).  The empty asm statements pin the order group by group: this group's unpack
-                // starts after the previous group's sums, so one group's results are live at a time (<= 128 VGPRs, four
-                // waves per SIMD, which hide the MFMA -> VALU latency this ordering exposes).
+                // G = 32 (segments of 64 slots only; smaller ones run compute32 below): every 32-k group's products are
+                // scaled on their own, and left alone the compiler issues all 8 * TT MFMAs of a k tile into separate
+                // result registers before the first scaled sum.  The empty asm statements pin the order group by group:
+                // this group's unpack starts after the previous group's sums, so one group's results are live at a time.
                 unsigned qw = s_.q[rb][w];
                 if (G == 32) asm volatile("" : "+v"(qw));
                 const h8_t a = w4_deq8(qw);
                 if (G == 32) {
                     const f4_t sc = moe_scale4<G, SBF, w>(s_.s[rb]);
-                    if constexpr (TT <= 3) {
-                        // all MFMAs of the group issue before the first scaled sum: the sums of the first result run
-                        // while the matrix pipe finishes the last (T = 512: 115.4 -> 113.8 us; with four results
-                        // in flight the kernel loses more to registers than it gains)
-                        f4_t p[TT];
 #pragma unroll
-                        for (int tt = 0; tt < TT; tt++) p[tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], zero, 0, 0, 0);
-                        if constexpr (TT == 1) asm volatile("" : "+v"(p[0]));
-                        if constexpr (TT == 2) asm volatile("" : "+v"(p[0]), "+v"(p[1]));
-                        if constexpr (TT == 3) asm volatile("" : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]));
-#pragma unroll
-                        for (int tt = 0; tt < TT; tt++) acc[rb][tt] = w4_fma4(sc, p[tt], acc[rb][tt]);
-                    } else {
-#pragma unroll
-                        for (int tt = 0; tt < TT; tt++)
-                            acc[rb][tt] = w4_fma4(sc, __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], zero, 0, 0, 0), acc[rb][tt]);
-                    }
+                    for (int tt = 0; tt < TT; tt++)
+                        acc[rb][tt] = w4_fma4(sc, __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], zero, 0, 0, 0), acc[rb][tt]);
 #pragma unroll
                     for (int tt = 0; tt < TT; tt++) asm volatile("" : "+v"(acc[rb][tt]));
                 } else {
@@ -590,6 +575,58 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
         }
     };
 
+    // Group size 32, up to three 16-slot blocks, software-pipelined by hand: a k tile is eight groups (32 k x one row
+    // block), each TT MFMAs into fresh results, the scale conversion and 4 * TT scaled sums.  Issue order per group: its
+    // MFMAs; then the NEXT group's unpack (and, when the 32-k chunk changes, the next B operands from LDS) while the
+    // matrix pipe works; then this group's scaled sums; then the next group's MFMAs, whose operands are ready.  A wave
+    // does not wait for its own MFMAs (the order "unpack, MFMAs, sums" group by group left 5-8 idle cycles after every
+    // MFMA for the other waves to fill).  Scheduling barriers hold the phases in this order; one group's results are
+    // live at a time.  128 experts, top-8: T = 64 77.6 -> 76.1 us, T = 512 117.9 -> 115.6 us; with four blocks the
+    // extra registers cost a wave per SIMD (T = 1024 +2 %), so 64-slot segments keep the plain order.
+    auto compute32 = [&](const MoeMmStage<2>& s_, int buf) {
+        const _Float16* xb = xs + buf * (ROWS * MOE_LDX) + c * MOE_LDX + q * 8;
+        const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+        h8_t b[TT];
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++) b[tt] = *reinterpret_cast<const h8_t*>(xb + tt * 16 * MOE_LDX);
+        h8_t a = w4_deq8(s_.q[0][0]);
+        auto group = [&](auto gc) {
+            constexpr int g = decltype(gc)::value, w = g >> 1, rb = g & 1;
+            f4_t p[TT];
+#pragma unroll
+            for (int tt = 0; tt < TT; tt++) p[tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[tt], zero, 0, 0, 0);
+            if constexpr (TT == 1) asm volatile("" : "+v"(p[0]));
+            if constexpr (TT == 2) asm volatile("" : "+v"(p[0]), "+v"(p[1]));
+            if constexpr (TT == 3) asm volatile("" : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]));
+            if constexpr (TT == 4) asm volatile("" : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]), "+v"(p[3]));
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (g < 7) {
+                constexpr int w2 = (g + 1) >> 1, rb2 = (g + 1) & 1;
+                if constexpr (w2 != w) {
+#pragma unroll
+                    for (int tt = 0; tt < TT; tt++) b[tt] = *reinterpret_cast<const h8_t*>(xb + tt * 16 * MOE_LDX + w2 * 32);
+                }
+                a = w4_deq8(s_.q[rb2][w2]);
+                asm volatile("" : "+v"(a));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const f4_t sc = moe_scale4<G, SBF, w>(s_.s[rb]);
+#pragma unroll
+            for (int tt = 0; tt < TT; tt++) acc[rb][tt] = w4_fma4(sc, p[tt], acc[rb][tt]);
+#pragma unroll
+            for (int tt = 0; tt < TT; tt++) asm volatile("" : "+v"(acc[rb][tt]));
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        group(std::integral_constant<int, 0>{});
+        group(std::integral_constant<int, 1>{});
+        group(std::integral_constant<int, 2>{});
+        group(std::integral_constant<int, 3>{});
+        group(std::integral_constant<int, 4>{});
+        group(std::integral_constant<int, 5>{});
+        group(std::integral_constant<int, 6>{});
+        group(std::integral_constant<int, 7>{});
+    };
+
     // prologue: the slice's first x tile into LDS buffer 0, the second in registers (both loads issued before the first
     // is stored: the first tile's registers are free again before the accumulators are live), DEPTH weight stages in
     // flight
@@ -609,7 +646,10 @@ __device__ __forceinline__ void moe_mm_body(MOE_PARAMS) {
             const int kt = kt0 + d;
             // a wave that holds a landed tile issues ahead of the waves that are queueing loads (about 1 % at every T)
             __builtin_amdgcn_s_setprio(1);
-            if (kt < kt_hi) compute(stage[d], xb);
+            if (kt < kt_hi) {
+                if constexpr (G == 32 && TT <= 3) compute32(stage[d], xb);
+                else compute(stage[d], xb);
+            }
             __builtin_amdgcn_s_setprio(0);
             load_w(stage[d], kt + DEPTH);
             store_x(xreg, xb ^ 1);  // tile kt+1, loaded an iteration ago, into the buffer tile kt-1 was read from
