@@ -157,7 +157,9 @@ int w4a16_lin_fuse(w4a16_ctx* ctx, const char* name, const char* const* parts, s
  * n, k} that build_multi_tables writes per layer (w4a16_dec/buffers.rs:229-366): ONE decode launch for the linears
  * fused under `name`, every part into its own output.  outs_dev: n_outs device addresses (a host array), n_outs = the
  * number of parts given to w4a16_lin_fuse (2..4); output i receives f16 or f32 [t][n_i], the rows of part i, with the
- * bits w4a16_lin_forward writes to y[:, first_i : first_i + n_i] of the fused linear.  Parts must be multiples of 16
+ * bits w4a16_lin_forward writes to y[:, first_i : first_i + n_i] of the fused linear when that launch runs two row blocks
+ * per wave as this one always does (w4a16_set_decode_shape(ctx, 32, 0); another launch shape may split k differently
+ * and differ in the last bits).  Parts must be multiples of 16
  * rows (W4A16_ERR_SHAPE otherwise); decode steps only: t > 16 is W4A16_ERR_UNSUPPORTED (w4a16_lin_forward then writes
  * the parts side by side in one tensor, which the consumers in this library read through a row stride). */
 int w4a16_lin_forward_multi(w4a16_ctx* ctx, const char* name, uint64_t x_dev, const uint64_t* outs_dev, size_t n_outs,
