@@ -241,14 +241,15 @@ __device__ __forceinline__ void decode_body(const u4_t* __restrict__ qt, const u
         const char* sc = sc0 + r * (DEPTH * GPT * 32);  // the staged scales are older than every ring load: no wait of their own
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
-            // One row block per wave (seven resident waves per SIMD): a wave that holds a landed tile issues ahead of
-            // the waves that are only queueing their next loads, so the tile's registers are free for the next load
-            // sooner (t = 1 on 5120 x 34816: 17.20 -> 17.05 us, four same-box rounds; with two row blocks per wave the
-            // same costs 0.6 % at t = 4 and is left out).
-            if (RB == 1) __builtin_amdgcn_s_setprio(1);
+            // A wave that holds a landed tile issues ahead of the waves that are only queueing their next loads, so the
+            // tile's registers are free for the next load sooner: one row block per wave (seven resident waves per
+            // SIMD), t = 1 on 5120 x 34816: 17.20 -> 17.05 us over four same-box rounds; four row blocks per wave,
+            // 17408 x 5120 at t = 8 / 16: 13.65 -> 13.45 / 15.88 -> 15.76 us.  With two row blocks per wave the same
+            // costs 0.6 % on the wide shape at t = 4 and is left out.
+            if (RB != 2) __builtin_amdgcn_s_setprio(1);
             if (r >= 0) compute(stage[d], sc, d);
             __builtin_amdgcn_sched_barrier(0);
-            if (RB == 1) __builtin_amdgcn_s_setprio(0);
+            if (RB != 2) __builtin_amdgcn_s_setprio(0);
             load(stage[d], kt0 + (r + 1) * DEPTH + d);
             __builtin_amdgcn_sched_barrier(0);
         }
