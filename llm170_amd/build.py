@@ -27,6 +27,8 @@ DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-targe
 # a library routine (expf) must expand identically in every code object so that fused epilogues give the bits of the
 # separate kernels.  Kernels that want a fused multiply-add write __builtin_fmaf.
 FUSED_OK = set()
+# per-file backend options: the dense group-128 prefill kernels schedule for instruction-level parallelism
+EXTRA_FLAGS = {"prefill_g128": ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]}
 
 
 HASH_PATH = os.path.join(PKG, "assets", "SOURCE_HASH")
@@ -70,7 +72,7 @@ def build_asset(name):
     flags = list(DEVICE_FLAGS)
     if name in FUSED_OK:
         flags[flags.index("-ffp-contract=off")] = "-ffp-contract=fast"
-    cmd = ["hipcc"] + flags + ["-I", KERNEL_DIR, "-o", out, src]
+    cmd = ["hipcc"] + flags + EXTRA_FLAGS.get(name, []) + ["-I", KERNEL_DIR, "-o", out, src]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (name, r.stdout))

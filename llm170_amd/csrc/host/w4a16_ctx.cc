@@ -68,14 +68,16 @@ static const char* const kDecodeSyms[] = {
     "w4a16_decode_g32_f16_multi_x1", "w4a16_decode_g32_f16_multi_x2", "w4a16_decode_g32_f16_multi_x4",
     "w4a16_decode_g32_bf16_multi_x1", "w4a16_decode_g32_bf16_multi_x2", "w4a16_decode_g32_bf16_multi_x4",
     nullptr};
-static const char* const kPrefillSyms[] = {"w4a16_prefill_g128_f16", "w4a16_prefill_g128_bf16", "w4a16_prefill_g32_f16",
-                                           "w4a16_prefill_g32_bf16", "w4a16_prefill_g128_f16_m64", "w4a16_prefill_g128_bf16_m64", "w4a16_prefill_g32_f16_m64",
+static const char* const kPrefillG128Syms[] = {
+    "w4a16_prefill_g128_f16", "w4a16_prefill_g128_bf16", "w4a16_prefill_g128_f16_m64", "w4a16_prefill_g128_bf16_m64",
+    "w4a16_prefill_g128_f16_m96", "w4a16_prefill_g128_bf16_m96", "w4a16_prefill_g128_f16_glu", "w4a16_prefill_g128_bf16_glu",
+    "w4a16_prefill_g128_f16_m64_glu", "w4a16_prefill_g128_bf16_m64_glu", "w4a16_prefill_g128_f16_m96_glu",
+    "w4a16_prefill_g128_bf16_m96_glu", nullptr};
+static const char* const kPrefillSyms[] = {"w4a16_prefill_g32_f16", "w4a16_prefill_g32_bf16", "w4a16_prefill_g32_f16_m64",
                                            "w4a16_prefill_g32_bf16_m64", "w4a16_prefill_splitk_sum", "w4a16_prefill_splitk_finish",
-                                           "w4a16_prefill_g128_f16_glu", "w4a16_prefill_g128_bf16_glu", "w4a16_prefill_g32_f16_glu",
-                                           "w4a16_prefill_g32_bf16_glu", "w4a16_prefill_g128_f16_m64_glu", "w4a16_prefill_g128_bf16_m64_glu",
+                                           "w4a16_prefill_g32_f16_glu", "w4a16_prefill_g32_bf16_glu",
                                            "w4a16_prefill_g32_f16_m64_glu", "w4a16_prefill_g32_bf16_m64_glu",
-                                           "w4a16_prefill_g128_f16_m96", "w4a16_prefill_g128_bf16_m96", "w4a16_prefill_g32_f16_m96",
-                                           "w4a16_prefill_g32_bf16_m96", "w4a16_prefill_g128_f16_m96_glu", "w4a16_prefill_g128_bf16_m96_glu",
+                                           "w4a16_prefill_g32_f16_m96", "w4a16_prefill_g32_bf16_m96",
                                            "w4a16_prefill_g32_f16_m96_glu", "w4a16_prefill_g32_bf16_m96_glu",
                                            "w4a16_moe_g128_f16_pf_glu", "w4a16_moe_g128_f16_pf_lin", "w4a16_moe_g128_bf16_pf_glu",
                                            "w4a16_moe_g128_bf16_pf_lin", "w4a16_moe_g32_f16_pf_glu", "w4a16_moe_g32_f16_pf_lin",
@@ -113,6 +115,7 @@ static const W4Asset kAssets[] = {
     {"layout", kLayoutSyms},
     {"decode", kDecodeSyms},
     {"prefill", kPrefillSyms},
+    {"prefill_g128", kPrefillG128Syms},
     {"moe", kMoeSyms},
     {"glue", kGlueSyms},
     {"util", kUtilSyms},

@@ -490,6 +490,24 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
                                       row_blocks, k, n, 0, y_f16, 1, 1, gp);                                             \
     }
 
+// This file builds two code objects.  Compiled on its own it holds everything but the dense group-128 kernels;
+// prefill_g128.hip includes it with PF_DENSE_G128 defined and holds those twelve, built with the backend's max-ILP
+// instruction scheduler (5120 x 34816 at M = 4096: 1.204 -> 1.193 ms, the other layer shapes -0.2...-0.6 %; the
+// group-32 builds spill registers under that scheduler and keep the default).
+#ifdef PF_DENSE_G128
+PREFILL_KERNEL(w4a16_prefill_g128_f16, 128, false, 4, 2)
+PREFILL_KERNEL(w4a16_prefill_g128_bf16, 128, true, 4, 2)
+PREFILL_KERNEL(w4a16_prefill_g128_f16_m64, 128, false, 2, 3)
+PREFILL_KERNEL(w4a16_prefill_g128_bf16_m64, 128, true, 2, 3)
+PREFILL_KERNEL(w4a16_prefill_g128_f16_m96, 128, false, 3, 3)
+PREFILL_KERNEL(w4a16_prefill_g128_bf16_m96, 128, true, 3, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_f16_glu, 128, false, 4, 2)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_bf16_glu, 128, true, 4, 2)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_f16_m64_glu, 128, false, 2, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_bf16_m64_glu, 128, true, 2, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_f16_m96_glu, 128, false, 3, 3)
+PREFILL_GLU_KERNEL(w4a16_prefill_g128_bf16_m96_glu, 128, true, 3, 3)
+#else
 // y[i] = sum over the nks partials of a split-K launch, added in split order in f32; f32 or f16 out.
 // glu != 0: the partials are those of a fused gate|up linear, [slices][t][n]; y is f16 [t][n/2] = act(g) * u on the
 // summed gate and up columns (act_kind as in w4_act_mul), the same arithmetic as the unsplit gated epilogue.
@@ -586,28 +604,16 @@ extern "C" __global__ __launch_bounds__(256) void w4a16_prefill_splitk_finish(co
     }
 }
 
-PREFILL_KERNEL(w4a16_prefill_g128_f16, 128, false, 4, 2)
-PREFILL_KERNEL(w4a16_prefill_g128_bf16, 128, true, 4, 2)
 PREFILL_KERNEL(w4a16_prefill_g32_f16, 32, false, 4, 2)
 PREFILL_KERNEL(w4a16_prefill_g32_bf16, 32, true, 4, 2)
-PREFILL_KERNEL(w4a16_prefill_g128_f16_m64, 128, false, 2, 3)
-PREFILL_KERNEL(w4a16_prefill_g128_bf16_m64, 128, true, 2, 3)
 PREFILL_KERNEL(w4a16_prefill_g32_f16_m64, 32, false, 2, 3)
 PREFILL_KERNEL(w4a16_prefill_g32_bf16_m64, 32, true, 2, 3)
-PREFILL_KERNEL(w4a16_prefill_g128_f16_m96, 128, false, 3, 3)
-PREFILL_KERNEL(w4a16_prefill_g128_bf16_m96, 128, true, 3, 3)
 PREFILL_KERNEL(w4a16_prefill_g32_f16_m96, 32, false, 3, 3)
 PREFILL_KERNEL(w4a16_prefill_g32_bf16_m96, 32, true, 3, 3)
-PREFILL_GLU_KERNEL(w4a16_prefill_g128_f16_glu, 128, false, 4, 2)
-PREFILL_GLU_KERNEL(w4a16_prefill_g128_bf16_glu, 128, true, 4, 2)
 PREFILL_GLU_KERNEL(w4a16_prefill_g32_f16_glu, 32, false, 4, 2)
 PREFILL_GLU_KERNEL(w4a16_prefill_g32_bf16_glu, 32, true, 4, 2)
-PREFILL_GLU_KERNEL(w4a16_prefill_g128_f16_m64_glu, 128, false, 2, 3)
-PREFILL_GLU_KERNEL(w4a16_prefill_g128_bf16_m64_glu, 128, true, 2, 3)
 PREFILL_GLU_KERNEL(w4a16_prefill_g32_f16_m64_glu, 32, false, 2, 3)
 PREFILL_GLU_KERNEL(w4a16_prefill_g32_bf16_m64_glu, 32, true, 2, 3)
-PREFILL_GLU_KERNEL(w4a16_prefill_g128_f16_m96_glu, 128, false, 3, 3)
-PREFILL_GLU_KERNEL(w4a16_prefill_g128_bf16_m96_glu, 128, true, 3, 3)
 PREFILL_GLU_KERNEL(w4a16_prefill_g32_f16_m96_glu, 32, false, 3, 3)
 PREFILL_GLU_KERNEL(w4a16_prefill_g32_bf16_m96_glu, 32, true, 3, 3)
 PREFILL_MOE_KERNEL(w4a16_moe_g128_f16_pf_glu, 128, false, 1)
@@ -618,3 +624,4 @@ PREFILL_MOE_KERNEL(w4a16_moe_g32_f16_pf_glu, 32, false, 1)
 PREFILL_MOE_KERNEL(w4a16_moe_g32_f16_pf_lin, 32, false, 2)
 PREFILL_MOE_KERNEL(w4a16_moe_g32_bf16_pf_glu, 32, true, 1)
 PREFILL_MOE_KERNEL(w4a16_moe_g32_bf16_pf_lin, 32, true, 2)
+#endif

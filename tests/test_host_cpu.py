@@ -50,12 +50,28 @@ def expand_kernel_macros(text):
     return names
 
 
+def kernel_text(kdir, asset):
+    """The text one code object is compiled from.  A source may be a few lines that define a selector and include
+    another source (prefill_g128.hip builds the dense group-128 kernels of prefill.hip); `#ifdef SELECTOR ... #else ...
+    #endif` blocks of the included text are resolved the way the preprocessor would for that code object."""
+    text = open(os.path.join(kdir, asset + ".hip")).read()
+    defined = set(re.findall(r"^#define\s+(\w+)\s*$", text, flags=re.M))
+    inc = re.search(r'^#include "(\w+\.hip)"', text, flags=re.M)
+    if inc:
+        text = open(os.path.join(kdir, inc.group(1))).read()
+
+    def pick(m):
+        return m.group(2) if m.group(1) in defined else m.group(3)
+
+    return re.sub(r"^#ifdef (PF_\w+)\n(.*?)^#else\n(.*?)^#endif\n", pick, text, flags=re.M | re.S)
+
+
 def test_manifest_matches_kernel_sources():
     """Precedent: manifest symbols == extern "C" __global__ symbols of the .cu files (assets.rs:394-443)."""
     man = ffi.manifest()
     kdir = os.path.join(ROOT, "llm170_amd", "csrc", "kernels")
     for asset, syms in man.items():
-        text = open(os.path.join(kdir, asset + ".hip")).read()
+        text = kernel_text(kdir, asset)
         names = set(re.findall(r'extern "C" __global__[^;{]*?\bvoid\s+(w4a16_\w+)\s*\(', text))
         # kernels stamped out by macros: expand `#define M(...) body` textually until only `void <name>(` remain
         names |= expand_kernel_macros(text)
