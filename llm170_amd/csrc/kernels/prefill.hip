@@ -225,8 +225,7 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
     const int kt_lo = DENSE ? (kt_n * (int)blockIdx.y) / (int)gridDim.y : 0,
               kt_hi = DENSE ? (kt_n * ((int)blockIdx.y + 1)) / (int)gridDim.y : kt_n;
     const int stages = 2 * kt_hi;
-    // wave priority over a stage's MFMAs (see the k loop): the 64- and 96-row tiles, and launches split over k
-    const bool PF_WAVE_PRIO = G == 128 && (MI <= 3 || (DENSE && gridDim.y > 1));
+    constexpr bool PF_WAVE_PRIO = G == 128;  // wave priority over a stage's MFMAs (see the k loop)
 
     load_a(2 * kt_lo, 0);
     load_b(bq, sc, kt_lo);
@@ -248,12 +247,13 @@ __device__ __forceinline__ void prefill_body(const u4_t* __restrict__ qt, const 
                 //   MFMA of the group, with the scale of the next k tile (already loaded), so the VALU work of tile j
                 //   runs in the shadow of the MFMAs of tiles j+1.. instead of stalling the next stage's first MFMAs;
                 //   group 32: at the first k16 of each 32-k group, before the tile's first MFMA.
-                // Wave priority (the 64- and 96-row tiles, three waves per SIMD): raised while a stage's MFMAs issue,
-                // dropped for the accumulator rescale at the end of a k tile, so that a wave in that VALU-only stretch
-                // yields the issue port to the waves that feed the matrix pipe (M = 512: 186 -> 180 us, M = 1024:
-                // 328 -> 317 us on 5120 x 34816; 17408 x 5120 at M = 4096: 630 -> 620 us).  With two waves per SIMD
-                // (the 128-row tile) the same costs 1 % at M = 4096 on that shape and gains 1-2 % in launches split over
-                // k (17408 x 5120 at M = 1024, three slices: 173 -> 169 us), so that tile takes it in split launches.
+                // Wave priority: raised while a stage's MFMAs issue, dropped for the accumulator rescale at the end of a
+                // k tile, so that a wave in that VALU-only stretch yields the issue port to the waves that feed the
+                // matrix pipe.  64- and 96-row tiles (three waves per SIMD): M = 512 186 -> 180 us, M = 1024 328 -> 317 us
+                // on 5120 x 34816; 17408 x 5120 at M = 4096 630 -> 620 us.  128-row tile (two waves per SIMD), built with
+                // the max-ILP scheduler: 5120 x 34816 at M = 4096 -0.5...-1.5 % on five boxes (with the default
+                // scheduler the same lost 0.4-0.9 % on the faster boxes).  Group 32 rescales inside the stage and has no
+                // such stretch.
                 if (PF_WAVE_PRIO && kbl == 0) __builtin_amdgcn_s_setprio(1);
                 const bool boundary32 = G == 32 && h == 0;
                 float ratio[2] = {1.f, 1.f};
